@@ -1,0 +1,209 @@
+"""Cache manager: paged keys and values with a block table per request, and
+slots of fixed-size per-request state.
+
+Layers whose mixers need the same span of the past form a *group*: all keys
+(window None) or the last `window` positions. A group has its own page ids,
+allocator and block tables; every cache instance (one per plan entry that
+writes keys and values) in the group has its own pools, indexed by the
+group's page ids. A request holds one *slot*: its row in every group's block
+table and its row of the state tensor.
+
+Pages are given back when a request is released and, in a window group, as
+soon as the window has passed them: with n cached positions, the next query
+is at position >= n and sees keys >= n - window + 1, so every page whose last
+position is <= n - window is freed (its block-table entry becomes -1).
+
+The reference's cache is one slab per (layer, slot) addressed by
+seq * stride + pos * Hkv * D (src/runtime/kv_cache.h:25-42); its lengths live
+in the caller (src/api/ninfer_c_api.cpp:28-32). Introspection successors of
+src/api/ninfer_c_api.cpp:99-114: `kv_bytes_per_token`, `pages_total`,
+`pages_free`.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from ..parts.base import CacheNeed
+from .pages import OutOfPages, PageAllocator
+
+
+@dataclass
+class CacheGroup:
+    window: Optional[int]
+    allocator: PageAllocator
+    instances: List[int] = field(default_factory=list)   # plan entries with pools in this group
+    tables: Dict[int, List[int]] = field(default_factory=dict)  # slot -> page of each logical page
+    window_freed: int = 0
+
+
+class CacheManager:
+    """Host side of the cache: who holds which page. Device pools are made by
+    `allocate_pools` so that this class can be tested without a device."""
+
+    def __init__(self, needs: Sequence[Optional[CacheNeed]], page_size: int, num_pages: int,
+                 max_seqs: int, max_context: int, state_floats: int = 0):
+        self.page_size = page_size
+        self.max_seqs = max_seqs
+        self.max_context = max_context
+        self.max_pages_per_request = -(-max_context // page_size)
+        self.state_floats = state_floats
+        self.needs = list(needs)
+        self.groups: List[CacheGroup] = []
+        self.group_of_instance: Dict[int, int] = {}
+        by_window: Dict[Optional[int], int] = {}
+        for i, need in enumerate(self.needs):
+            if need is None:
+                continue
+            if need.window not in by_window:
+                by_window[need.window] = len(self.groups)
+                self.groups.append(CacheGroup(need.window, PageAllocator(num_pages)))
+            g = by_window[need.window]
+            self.groups[g].instances.append(i)
+            self.group_of_instance[i] = g
+        self._free_slots: List[int] = list(range(max_seqs - 1, -1, -1))
+        self._length: Dict[int, int] = {}
+        self.pools: Dict[int, Tuple[object, object]] = {}
+        self.state = None
+
+    # ---- device memory -----------------------------------------------------
+    def allocate_pools(self, device, dtype) -> None:
+        import torch
+        for i, need in enumerate(self.needs):
+            if need is None:
+                continue
+            n = self.groups[self.group_of_instance[i]].allocator.num_pages
+            shape = (n, need.kv_heads, self.page_size, need.head_dim)
+            self.pools[i] = (torch.zeros(shape, dtype=dtype, device=device),
+                             torch.zeros(shape, dtype=dtype, device=device))
+        self.state = torch.zeros((self.max_seqs, max(self.state_floats, 1)),
+                                 dtype=torch.float32, device=device)
+
+    # ---- slots ---------------------------------------------------------------
+    @property
+    def free_slots(self) -> int:
+        return len(self._free_slots)
+
+    def live_slots(self) -> List[int]:
+        return sorted(self._length)
+
+    def acquire(self) -> int:
+        """A free slot with empty block tables and zeroed state."""
+        if not self._free_slots:
+            raise RuntimeError(f"all {self.max_seqs} request slots are in use")
+        slot = self._free_slots.pop()
+        self._length[slot] = 0
+        for g in self.groups:
+            g.tables[slot] = []
+        if self.state is not None and self.state_floats:
+            self.state[slot].zero_()
+        return slot
+
+    def release(self, slot: int) -> None:
+        """Give back every page the request holds in every group, and its slot."""
+        if slot not in self._length:
+            raise RuntimeError(f"slot {slot} released but not held")
+        for g in self.groups:
+            g.allocator.free([p for p in g.tables.pop(slot) if p >= 0])
+        del self._length[slot]
+        self._free_slots.append(slot)
+
+    def length(self, slot: int) -> int:
+        return self._length[slot]
+
+    # ---- pages ---------------------------------------------------------------
+    def pages_needed(self, slot: int, new_len: int) -> List[int]:
+        want = -(-new_len // self.page_size)
+        return [max(0, want - len(g.tables[slot])) for g in self.groups]
+
+    def can_reserve(self, slot: int, new_len: int) -> bool:
+        return all(n <= g.allocator.free_pages
+                   for n, g in zip(self.pages_needed(slot, new_len), self.groups))
+
+    def reserve(self, slot: int, new_len: int) -> None:
+        """Pages for positions < new_len in every group, or OutOfPages with
+        nothing taken in any group."""
+        if new_len > self.max_context:
+            raise OutOfPages(f"request would hold {new_len} tokens; max_context is "
+                             f"{self.max_context}")
+        need = self.pages_needed(slot, new_len)
+        for n, g in zip(need, self.groups):
+            if n > g.allocator.free_pages:
+                raise OutOfPages(f"need {n} pages in the group with window {g.window}, "
+                                 f"{g.allocator.free_pages} are free")
+        for n, g in zip(need, self.groups):
+            g.tables[slot].extend(g.allocator.alloc(n))
+
+    def reserve_all(self, wants: Sequence[Tuple[int, int]]) -> None:
+        """`reserve` for several (slot, new_len) at once: all or nothing."""
+        total = [0] * len(self.groups)
+        for slot, new_len in wants:
+            if new_len > self.max_context:
+                raise OutOfPages(f"request would hold {new_len} tokens; max_context is "
+                                 f"{self.max_context}")
+            for i, n in enumerate(self.pages_needed(slot, new_len)):
+                total[i] += n
+        for n, g in zip(total, self.groups):
+            if n > g.allocator.free_pages:
+                raise OutOfPages(f"need {n} pages in the group with window {g.window}, "
+                                 f"{g.allocator.free_pages} are free")
+        for slot, new_len in wants:
+            self.reserve(slot, new_len)
+
+    def commit(self, slot: int, new_len: int) -> None:
+        """The request now has new_len cached positions; free what its windows
+        have passed."""
+        if new_len < self._length[slot]:
+            raise RuntimeError("a request's cached length cannot shrink")
+        self._length[slot] = new_len
+        for g in self.groups:
+            if g.window is None:
+                continue
+            table = g.tables[slot]
+            # pages whose last position (p+1)*ps - 1 <= new_len - window
+            dead = (new_len - g.window + 1) // self.page_size
+            gone = []
+            for p in range(min(max(dead, 0), len(table))):
+                if table[p] >= 0:
+                    gone.append(table[p])
+                    table[p] = -1
+            if gone:
+                g.allocator.free(gone)
+                g.window_freed += len(gone)
+
+    # ---- what a step needs ---------------------------------------------------
+    def block_table(self, group: int, slots: Sequence[int], width: Optional[int] = None
+                    ) -> np.ndarray:
+        """int32 [len(slots), width] block-table rows, -1 where no page is held."""
+        g = self.groups[group]
+        if width is None:
+            width = max([len(g.tables[s]) for s in slots] + [1])
+        out = np.full((len(slots), width), -1, dtype=np.int32)
+        for i, s in enumerate(slots):
+            t = g.tables[s]
+            out[i, :len(t)] = t
+        return out
+
+    # ---- introspection -------------------------------------------------------
+    def kv_bytes_per_token(self, bytes_per_element: int) -> int:
+        return sum(2 * n.kv_heads * n.head_dim * bytes_per_element
+                   for n in self.needs if n is not None)
+
+    def pages_total(self, group: int = 0) -> int:
+        return self.groups[group].allocator.num_pages
+
+    def pages_free(self, group: int = 0) -> int:
+        return self.groups[group].allocator.free_pages
+
+    def pages_reused(self) -> int:
+        return sum(g.allocator.reused for g in self.groups)
+
+    def check(self) -> None:
+        """No page lost, held twice, or held by nobody."""
+        for g in self.groups:
+            g.allocator.check()
+            held = [p for t in g.tables.values() for p in t if p >= 0]
+            assert len(held) == len(set(held)), "a page is in two block tables"
+            assert len(held) == g.allocator.in_use, "allocator and block tables disagree"

@@ -1,0 +1,127 @@
+"""Typed configuration of Qwen2-MoE (`Qwen2MoeForCausalLM`, model_type
+`qwen2_moe`), read from the architecture's own config.json keys.
+
+Keys and defaults the reference reads: src/models/config.cpp:12-43
+(`num_key_value_heads` defaults to the head count :21-23, `head_dim` to
+hidden/heads :25-27, `rope_theta` to 1e6 :29-30, `tie_word_embeddings` to
+false :31-32). The keys it does not read (shared expert size, `norm_topk_prob`,
+`decoder_sparse_step`, `mlp_only_layers`, the sliding-window keys) are read
+here because the architecture has them.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional
+
+from .base import ConfigError, KeyReader
+
+
+@dataclass(frozen=True)
+class Qwen2MoeConfig:
+    vocab_size: int
+    hidden_size: int
+    num_hidden_layers: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    intermediate_size: int
+    rms_norm_eps: float
+    rope_theta: float
+    tie_word_embeddings: bool
+    num_experts: int
+    num_experts_per_tok: int
+    moe_intermediate_size: int
+    shared_expert_intermediate_size: int
+    norm_topk_prob: bool
+    decoder_sparse_step: int
+    mlp_only_layers: List[int] = field(default_factory=list)
+    use_sliding_window: bool = False
+    sliding_window: Optional[int] = None
+    max_window_layers: int = 0
+    eos_token_id: Optional[int] = None
+    architecture: str = "Qwen2MoeForCausalLM"
+
+    # ---- derived, layer by layer -------------------------------------
+    def layer_is_sparse(self, layer: int) -> bool:
+        """Experts on layer l iff l is not in mlp_only_layers, there are
+        experts, and (l + 1) is a multiple of decoder_sparse_step."""
+        return (layer not in self.mlp_only_layers and self.num_experts > 0
+                and (layer + 1) % self.decoder_sparse_step == 0)
+
+    def layer_window(self, layer: int) -> Optional[int]:
+        """Window of layer l: `sliding_window` for l >= max_window_layers when
+        use_sliding_window, else none."""
+        if self.use_sliding_window and layer >= self.max_window_layers:
+            return self.sliding_window
+        return None
+
+    @staticmethod
+    def from_dict(raw: Dict[str, Any]) -> "Qwen2MoeConfig":
+        r = KeyReader(raw)
+        mt = r.opt_str("model_type", "qwen2_moe")
+        if mt != "qwen2_moe":
+            raise ConfigError(f"config.json: key 'model_type' must be 'qwen2_moe', got {mt!r}")
+        vocab = r.need_int("vocab_size", 1)
+        hidden = r.need_int("hidden_size", 1)
+        layers = r.need_int("num_hidden_layers", 1)
+        heads = r.need_int("num_attention_heads", 1)
+        kv_heads = r.opt_int("num_key_value_heads", heads, 1)
+        inter = r.need_int("intermediate_size", 1)
+        head_dim = r.opt_int("head_dim", None, 1)
+        if head_dim is None:
+            if hidden % heads:
+                raise ConfigError("config.json: 'hidden_size' is not a multiple of "
+                                  "'num_attention_heads' and 'head_dim' is not given")
+            head_dim = hidden // heads
+        if heads % kv_heads:
+            raise ConfigError(f"config.json: 'num_attention_heads' ({heads}) must be a "
+                              f"multiple of 'num_key_value_heads' ({kv_heads})")
+        if head_dim % 2:
+            raise ConfigError(f"config.json: 'head_dim' must be even, got {head_dim}")
+        eps = r.need_float("rms_norm_eps")
+        if not eps > 0:
+            raise ConfigError(f"config.json: key 'rms_norm_eps' must be > 0, got {eps}")
+        theta = r.opt_float("rope_theta", 1e6)
+        if not theta > 0:
+            raise ConfigError(f"config.json: key 'rope_theta' must be > 0, got {theta}")
+        if r.opt_raw("rope_scaling") is not None:
+            raise ConfigError("config.json: key 'rope_scaling' is not supported (must be null)")
+        act = r.opt_str("hidden_act", "silu")
+        if act != "silu":
+            raise ConfigError(f"config.json: key 'hidden_act' must be 'silu', got {act!r}")
+        experts = r.need_int("num_experts", 1)
+        top_k = r.need_int("num_experts_per_tok", 1)
+        if top_k > experts:
+            raise ConfigError(f"config.json: 'num_experts_per_tok' ({top_k}) exceeds "
+                              f"'num_experts' ({experts})")
+        moe_inter = r.need_int("moe_intermediate_size", 1)
+        shared_inter = r.need_int("shared_expert_intermediate_size", 1)
+        sparse_step = r.opt_int("decoder_sparse_step", 1, 1)
+        mlp_only = r.opt_int_list("mlp_only_layers", [])
+        for l in mlp_only:
+            if l >= layers:
+                raise ConfigError(f"config.json: 'mlp_only_layers' names layer {l} but the "
+                                  f"model has {layers}")
+        use_win = r.opt_bool("use_sliding_window", False)
+        window = r.opt_int("sliding_window", None, 1)
+        max_win_layers = r.opt_int("max_window_layers", 0, 0)
+        if use_win and window is None:
+            raise ConfigError("config.json: 'use_sliding_window' is true but "
+                              "'sliding_window' is missing")
+        eos = r.opt_raw("eos_token_id")
+        if isinstance(eos, list):
+            eos = eos[0] if eos else None
+        if eos is not None and (isinstance(eos, bool) or not isinstance(eos, int)):
+            raise ConfigError("config.json: key 'eos_token_id' must be an integer")
+        return Qwen2MoeConfig(
+            vocab_size=vocab, hidden_size=hidden, num_hidden_layers=layers,
+            num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=head_dim,
+            intermediate_size=inter, rms_norm_eps=eps, rope_theta=theta,
+            tie_word_embeddings=r.opt_bool("tie_word_embeddings", False),
+            num_experts=experts, num_experts_per_tok=top_k,
+            moe_intermediate_size=moe_inter,
+            shared_expert_intermediate_size=shared_inter,
+            norm_topk_prob=r.opt_bool("norm_topk_prob", False),
+            decoder_sparse_step=sparse_step, mlp_only_layers=mlp_only,
+            use_sliding_window=use_win, sliding_window=window,
+            max_window_layers=max_win_layers, eos_token_id=eos)

@@ -1,0 +1,25 @@
+// Entry point of paged attention: checks the arguments and picks a kernel.
+#include "attention.h"
+
+using namespace ninfer;
+
+// force_generic != 0 runs the plain one-wave-per-(row, head) kernel whatever
+// the shape (tests compare the fast kernels with it).
+extern "C" int ninfer_paged_attention(const AttnArgs* a, int force_generic, hipStream_t stream) {
+  NINFER_REQUIRE(a->T > 0 && a->S > 0, "paged_attention: T=%d S=%d must be positive", a->T, a->S);
+  NINFER_REQUIRE(a->Hq > 0 && a->Hkv > 0 && a->Hq % a->Hkv == 0,
+                 "paged_attention: %d query heads are not a multiple of %d kv heads", a->Hq,
+                 a->Hkv);
+  NINFER_REQUIRE(a->D > 0 && a->D % 2 == 0, "paged_attention: head size %d must be even", a->D);
+  NINFER_REQUIRE(a->page_size > 0 && a->bt_stride > 0, "paged_attention: bad page size %d or "
+                 "table width %d", a->page_size, a->bt_stride);
+  NINFER_REQUIRE(a->window >= 0, "paged_attention: window %d must be >= 0", a->window);
+  NINFER_REQUIRE(a->dtype == kF32 || a->dtype == kBF16, "paged_attention: unknown dtype %d",
+                 a->dtype);
+  NINFER_REQUIRE(a->q_stride >= a->Hq * a->D, "paged_attention: row stride %d < %d", a->q_stride,
+                 a->Hq * a->D);
+  (void)force_generic;
+  return attention_generic(a->q, a->q_stride, a->kpool, a->vpool, a->block_table, a->bt_stride,
+                           a->positions, a->row_seq, a->out, a->T, a->Hq, a->Hkv, a->D,
+                           a->page_size, a->window, a->scale, a->dtype, stream);
+}

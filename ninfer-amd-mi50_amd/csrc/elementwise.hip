@@ -1,0 +1,195 @@
+// Row-wise kernels: embedding gather, RMSNorm with the residual sum fused in,
+// bias + rotary + paged cache write, and the expert combine.
+//
+// The residual stream is 32-bit in both precisions; activations are `T`
+// (float or bf16). Sums of squares, rsqrt, rotation angles and weighted sums
+// are 32-bit.
+#include "common.h"
+
+namespace ninfer {
+
+// x[t,:] = table[token[t],:]   (reference src/ops/kernels.hip:150-159)
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ tokens, const T* __restrict__ table,
+                             float* __restrict__ out, int H) {
+  int64_t t = blockIdx.x;
+  const T* src = table + (int64_t)tokens[t] * H;
+  float* dst = out + t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_f32(src[i]);
+}
+
+// y = (x [+ delta]) * rsqrt(mean(.^2) + eps) * gain  (reference
+// src/ops/kernels.hip:17-41 and :100-129). With rows == nullptr the sum is
+// written back to x; with rows the kernel reads row rows[i] and leaves x alone.
+// The reduction order depends only on H and the block size, never on the
+// number of rows.
+template <typename T>
+__global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta,
+                               const float* __restrict__ gain, T* __restrict__ out,
+                               const int* __restrict__ rows, int H, float eps) {
+  __shared__ float red[16];
+  int64_t r_out = blockIdx.x;
+  int64_t r_in = rows ? rows[r_out] : r_out;
+  float* xr = x + r_in * H;
+  const T* dr = delta ? delta + r_in * H : nullptr;
+  T* orow = out + r_out * H;
+  float acc = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = xr[i];
+    if (dr) v += to_f32(dr[i]);
+    acc += v * v;
+  }
+  float total = block_sum(acc, red);
+  float inv = rsqrtf(total / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = xr[i];
+    if (dr) {
+      v += to_f32(dr[i]);
+      if (!rows) xr[i] = v;
+    }
+    orow[i] = from_f32<T>(v * inv * gain[i]);
+  }
+}
+
+// One block per (row, head) of the fused q|k|v row. Adds the bias, rotates q
+// heads in place and k heads on their way into the page; v heads are copied.
+// Pairs are (i, i + rot/2) within the first `rot` dims of a head (reference
+// src/ops/kernels.hip:86-91, full rotation there); dims >= rot pass through.
+// Page lookup: logical page pos / page_size of the row's request.
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restrict__ bias,
+                                     const int* __restrict__ positions,
+                                     const int* __restrict__ row_seq,
+                                     const float* __restrict__ inv_freq, int rot, int Hq, int Hkv,
+                                     int D, T* __restrict__ kpool, T* __restrict__ vpool,
+                                     const int* __restrict__ block_table, int bt_stride,
+                                     int page_size, int write_kv) {
+  int t = blockIdx.x;
+  int head = blockIdx.y;
+  int d = threadIdx.x;
+  int W = (Hq + 2 * Hkv) * D;
+  int col = head * D + d;
+  T* row = qkv + (int64_t)t * W;
+  bool is_q = head < Hq;
+  bool is_k = !is_q && head < Hq + Hkv;
+  if (!is_q && !write_kv) return;  // uniform per block
+  int pos = positions[t];
+  float v = 0.f, partner = 0.f;
+  int half = rot >> 1;
+  if (d < D) {
+    v = to_f32(row[col]) + (bias ? bias[col] : 0.f);
+    if ((is_q || is_k) && d < rot) {
+      int pd = d < half ? d + half : d - half;
+      partner = to_f32(row[head * D + pd]) + (bias ? bias[head * D + pd] : 0.f);
+    }
+  }
+  __syncthreads();  // all reads of the row are done before q is rewritten
+  if (d >= D) return;
+  float res = v;
+  if ((is_q || is_k) && d < rot) {
+    int i = d < half ? d : d - half;
+    float phi = (float)pos * inv_freq[i];
+    float c = cosf(phi), s = sinf(phi);
+    res = d < half ? v * c - partner * s : partner * s + v * c;
+  }
+  if (is_q) {
+    row[col] = from_f32<T>(res);
+    return;
+  }
+  int seq = row_seq[t];
+  int page = block_table[(int64_t)seq * bt_stride + pos / page_size];
+  int kvh = is_k ? head - Hq : head - Hq - Hkv;
+  int64_t off = (((int64_t)page * Hkv + kvh) * page_size + (pos % page_size)) * D + d;
+  (is_k ? kpool : vpool)[off] = from_f32<T>(res);
+}
+
+// residual[t,:] += sum_j w[t,j] * y[t*k + j,:] + sigmoid(gate[t]) * shared[t,:]
+// in that order, in 32-bit (the reference scales and scatter-adds rounded
+// rows: src/ops/kernels.hip:216-223, src/ops/moe.hip:22-31).
+template <typename T>
+__global__ void moe_combine_kernel(float* __restrict__ residual, const T* __restrict__ y,
+                                   const float* __restrict__ w, const T* __restrict__ shared,
+                                   const float* __restrict__ gate, int H, int k) {
+  int64_t t = blockIdx.x;
+  float g = 0.f;
+  if (shared) g = gate ? 1.f / (1.f + expf(-gate[t])) : 1.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float acc = 0.f;
+    for (int j = 0; j < k; ++j) acc += w[t * k + j] * to_f32(y[(t * k + j) * H + i]);
+    if (shared) acc += g * to_f32(shared[t * H + i]);
+    residual[t * H + i] += acc;
+  }
+}
+
+}  // namespace ninfer
+
+using namespace ninfer;
+
+extern "C" int ninfer_embed(const int* tokens, const void* table, float* out, int T, int H,
+                            int dtype, hipStream_t stream) {
+  NINFER_REQUIRE(T > 0 && H > 0, "embed: T=%d H=%d must be positive", T, H);
+  NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "embed: unknown dtype %d", dtype);
+  if (dtype == kF32)
+    embed_kernel<float><<<T, 256, 0, stream>>>(tokens, (const float*)table, out, H);
+  else
+    embed_kernel<bf16><<<T, 256, 0, stream>>>(tokens, (const bf16*)table, out, H);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int ninfer_rmsnorm(float* x, const void* delta, const float* gain, void* out,
+                              const int* rows, int n_rows, int H, float eps, int dtype,
+                              hipStream_t stream) {
+  NINFER_REQUIRE(n_rows > 0 && H > 0, "rmsnorm: rows=%d H=%d must be positive", n_rows, H);
+  NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "rmsnorm: unknown dtype %d", dtype);
+  int block = H >= 2048 ? 512 : 256;
+  if (dtype == kF32)
+    rmsnorm_kernel<float><<<n_rows, block, 0, stream>>>(x, (const float*)delta, gain, (float*)out,
+                                                       rows, H, eps);
+  else
+    rmsnorm_kernel<bf16><<<n_rows, block, 0, stream>>>(x, (const bf16*)delta, gain, (bf16*)out,
+                                                      rows, H, eps);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int ninfer_rope_kv_write(void* qkv, const float* bias, const int* positions,
+                                    const int* row_seq, const float* inv_freq, int rot_dim, int Hq,
+                                    int Hkv, int D, void* kpool, void* vpool,
+                                    const int* block_table, int bt_stride, int page_size,
+                                    int write_kv, int T, int dtype, hipStream_t stream) {
+  NINFER_REQUIRE(T > 0, "rope_kv_write: T=%d must be positive", T);
+  NINFER_REQUIRE(D > 0 && D <= 1024, "rope_kv_write: head size %d not in [1,1024]", D);
+  NINFER_REQUIRE(rot_dim >= 0 && rot_dim <= D && rot_dim % 2 == 0,
+                 "rope_kv_write: rotary size %d must be even and <= head size %d", rot_dim, D);
+  NINFER_REQUIRE(rot_dim == 0 || inv_freq, "rope_kv_write: rotary size %d without a table", rot_dim);
+  NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "rope_kv_write: unknown dtype %d", dtype);
+  NINFER_REQUIRE(page_size > 0 && bt_stride > 0, "rope_kv_write: bad page size or table width");
+  dim3 grid(T, Hq + 2 * Hkv);
+  int block = (D + 63) / 64 * 64;
+  if (dtype == kF32)
+    rope_kv_write_kernel<float><<<grid, block, 0, stream>>>(
+        (float*)qkv, bias, positions, row_seq, inv_freq, rot_dim, Hq, Hkv, D, (float*)kpool,
+        (float*)vpool, block_table, bt_stride, page_size, write_kv);
+  else
+    rope_kv_write_kernel<bf16><<<grid, block, 0, stream>>>(
+        (bf16*)qkv, bias, positions, row_seq, inv_freq, rot_dim, Hq, Hkv, D, (bf16*)kpool,
+        (bf16*)vpool, block_table, bt_stride, page_size, write_kv);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int ninfer_moe_combine(float* residual, const void* y, const float* w,
+                                  const void* shared, const float* gate, int T, int H, int k,
+                                  int dtype, hipStream_t stream) {
+  NINFER_REQUIRE(T > 0 && H > 0 && k > 0, "moe_combine: T=%d H=%d k=%d must be positive", T, H, k);
+  NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "moe_combine: unknown dtype %d", dtype);
+  if (dtype == kF32)
+    moe_combine_kernel<float><<<T, 256, 0, stream>>>(residual, (const float*)y, w,
+                                                    (const float*)shared, gate, H, k);
+  else
+    moe_combine_kernel<bf16><<<T, 256, 0, stream>>>(residual, (const bf16*)y, w,
+                                                   (const bf16*)shared, gate, H, k);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,242 @@
+// Sampling on the device, one block per row of logits.
+//
+// Order of operations as in the reference's CPU sampler
+// (src/runtime/engine.cpp:18-82): repetition penalty -> greedy if
+// temperature <= 0 -> / temperature -> top-k -> softmax -> top-p -> draw.
+// Differences, all deliberate: the penalty arrives as (token, count) pairs
+// (a token seen c times is penalised c times, as the reference's loop over
+// the history does); top-k and top-p are found by radix selection on the
+// ordered bit pattern of the scaled logits instead of a sort, so ties at a
+// threshold are all kept; probabilities are held as 32.32 fixed-point
+// integers so every sum is exact and the draw does not depend on the order of
+// additions; the draw walks the kept tokens in index order with a uniform
+// number `u` in [0,1) that the caller derives from (seed, request, draw
+// index), so it does not depend on what else is in the batch. top_k <= 0
+// keeps all tokens (the reference clamps to >= 1).
+#include "common.h"
+
+namespace ninfer {
+
+constexpr int kSampleThreads = 1024;
+
+__device__ __forceinline__ uint32_t ordered_key(float v) {
+  uint32_t b = __float_as_uint(v);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);  // ascending with the float order
+}
+
+// Largest key t such that the sum of weight(i) over kept i with key(i) >= t
+// reaches `target`. 4 passes of an 8-bit histogram. `hist` is 256 uint64 in LDS.
+template <typename KeyFn, typename WeightFn>
+__device__ uint32_t radix_select(int V, unsigned long long target, unsigned long long* hist,
+                                 uint32_t* shared_out, KeyFn key, WeightFn weight) {
+  uint32_t prefix = 0, mask = 0;
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    for (int b = threadIdx.x; b < 256; b += blockDim.x) hist[b] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+      uint32_t k = key(i);
+      if ((k & mask) == prefix) {
+        unsigned long long w = weight(i, k);
+        if (w) atomicAdd(&hist[(k >> shift) & 255], w);
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      unsigned long long run = 0;
+      int b = 255;
+      for (; b > 0; --b) {
+        if (run + hist[b] >= target) break;
+        run += hist[b];
+      }
+      shared_out[0] = (uint32_t)b;
+      // mass above the chosen bin no longer counts towards the target
+      ((unsigned long long*)(shared_out + 2))[0] = run;
+    }
+    __syncthreads();
+    uint32_t b = shared_out[0];
+    target -= ((unsigned long long*)(shared_out + 2))[0];
+    prefix |= b << shift;
+    mask |= 255u << shift;
+    __syncthreads();
+  }
+  return prefix;
+}
+
+__global__ __launch_bounds__(kSampleThreads) void sample_kernel(
+    const float* __restrict__ logits, int ld, int V, float* __restrict__ work,
+    const float* __restrict__ temperature, const int* __restrict__ top_k,
+    const float* __restrict__ top_p, const float* __restrict__ rep_penalty,
+    const int* __restrict__ pen_tokens, const int* __restrict__ pen_counts,
+    const int* __restrict__ pen_offsets, const float* __restrict__ uniform,
+    int* __restrict__ out) {
+  __shared__ unsigned long long hist[256];
+  __shared__ unsigned long long sums[kSampleThreads];
+  __shared__ float fred[kSampleThreads / 64];
+  __shared__ int ired[kSampleThreads / 64];
+  __shared__ __align__(8) uint32_t sel[4];
+
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const float* row = logits + (int64_t)r * ld;
+  float* w = work + (int64_t)r * V;
+  const float temp = temperature[r];
+
+  // repetition penalty on a copy of the row
+  for (int i = tid; i < V; i += blockDim.x) w[i] = row[i];
+  __syncthreads();
+  float rp = rep_penalty ? rep_penalty[r] : 1.f;
+  if (rp != 1.f && pen_offsets) {
+    for (int e = pen_offsets[r] + tid; e < pen_offsets[r + 1]; e += blockDim.x) {
+      int tok = pen_tokens[e];
+      if (tok < 0 || tok >= V) continue;
+      float v = w[tok];
+      for (int c = 0; c < pen_counts[e]; ++c) v = v > 0.f ? v / rp : v * rp;
+      w[tok] = v;
+    }
+  }
+  __syncthreads();
+
+  // max and argmax (ties: lowest index)
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int i = tid; i < V; i += blockDim.x) {
+    float v = w[i];
+    if (v > best) {
+      best = v;
+      best_i = i;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    float ob = __shfl_xor(best, off, 64);
+    int oi = __shfl_xor(best_i, off, 64);
+    if (ob > best || (ob == best && oi < best_i)) {
+      best = ob;
+      best_i = oi;
+    }
+  }
+  if ((tid & 63) == 0) {
+    fred[tid >> 6] = best;
+    ired[tid >> 6] = best_i;
+  }
+  __syncthreads();
+  best = fred[0];
+  best_i = ired[0];
+  for (int i = 1; i < (int)(blockDim.x >> 6); ++i) {
+    if (fred[i] > best || (fred[i] == best && ired[i] < best_i)) {
+      best = fred[i];
+      best_i = ired[i];
+    }
+  }
+  if (!(temp > 0.f)) {
+    if (tid == 0) out[r] = best_i;
+    return;
+  }
+  __syncthreads();
+
+  const float inv_t = 1.f / temp;
+  const float m = best * inv_t;  // max of the scaled logits (temp > 0)
+  auto key = [&](int i) { return ordered_key(w[i] * inv_t); };
+
+  // top-k: keep keys >= the k-th largest
+  uint32_t floor_key = 0;
+  int k = top_k ? top_k[r] : 0;
+  if (k > 0 && k < V)
+    floor_key = radix_select(V, (unsigned long long)k, hist, sel, key,
+                             [](int, uint32_t) { return 1ull; });
+
+  // probabilities of the kept tokens as 32.32 fixed point
+  auto mass = [&](int i, uint32_t kk) -> unsigned long long {
+    if (kk < floor_key) return 0ull;
+    return (unsigned long long)(expf(w[i] * inv_t - m) * 4294967296.f);
+  };
+  auto block_total = [&](uint32_t lowest) {
+    unsigned long long s = 0;
+    for (int i = tid; i < V; i += blockDim.x) {
+      uint32_t kk = key(i);
+      if (kk >= lowest) s += mass(i, kk);
+    }
+    sums[tid] = s;
+    __syncthreads();
+    for (int off = kSampleThreads / 2; off > 0; off >>= 1) {
+      if (tid < off) sums[tid] += sums[tid + off];
+      __syncthreads();
+    }
+    unsigned long long t = sums[0];
+    __syncthreads();
+    return t;
+  };
+  unsigned long long total = block_total(floor_key);
+
+  // top-p: the smallest set of most probable tokens whose mass reaches top_p
+  float pp = top_p ? top_p[r] : 1.f;
+  if (pp < 1.f) {
+    unsigned long long target = (unsigned long long)((double)pp * (double)total);
+    if (target < 1) target = 1;
+    uint32_t pk = radix_select(V, target, hist, sel, key, mass);
+    if (pk > floor_key) {
+      floor_key = pk;
+      total = block_total(floor_key);
+    }
+  }
+
+  // inverse CDF over the kept tokens in index order
+  unsigned long long goal = (unsigned long long)((double)uniform[r] * (double)total);
+  if (goal >= total) goal = total - 1;
+  const int chunk = (V + blockDim.x - 1) / blockDim.x;
+  const int c0 = tid * chunk, c1 = min(V, c0 + chunk);
+  unsigned long long mine = 0;
+  for (int i = c0; i < c1; ++i) {
+    uint32_t kk = key(i);
+    if (kk >= floor_key) mine += mass(i, kk);
+  }
+  sums[tid] = mine;
+  __syncthreads();
+  if (tid == 0) {
+    unsigned long long run = 0;
+    for (int i = 0; i < (int)blockDim.x; ++i) {
+      unsigned long long s = sums[i];
+      sums[i] = run;
+      run += s;
+    }
+
+  }
+  __syncthreads();
+  unsigned long long before = sums[tid];
+  if (mine > 0 && goal >= before && goal < before + mine) {
+    unsigned long long run = before;
+    int pick = c1 - 1;
+    for (int i = c0; i < c1; ++i) {
+      uint32_t kk = key(i);
+      unsigned long long ms = kk >= floor_key ? mass(i, kk) : 0ull;
+      if (ms && goal < run + ms) {
+        pick = i;
+        break;
+      }
+      run += ms;
+    }
+    out[r] = pick;
+  }
+}
+
+}  // namespace ninfer
+
+using namespace ninfer;
+
+// logits [R, ld] (V used); work [R, V] scratch; per-row temperature, top_k,
+// top_p, rep_penalty, uniform; penalties as (token, count) pairs in
+// pen_tokens/pen_counts[pen_offsets[r] .. pen_offsets[r+1]) (null: none);
+// out [R] token ids.
+extern "C" int ninfer_sample(const float* logits, int ld, int V, int R, float* work,
+                             const float* temperature, const int* top_k, const float* top_p,
+                             const float* rep_penalty, const int* pen_tokens,
+                             const int* pen_counts, const int* pen_offsets, const float* uniform,
+                             int* out, hipStream_t stream) {
+  NINFER_REQUIRE(R > 0 && V > 0, "sample: R=%d V=%d must be positive", R, V);
+  NINFER_REQUIRE(ld >= V, "sample: row stride %d < vocabulary %d", ld, V);
+  NINFER_REQUIRE(temperature && uniform && work && out, "sample: a required array is null");
+  sample_kernel<<<R, kSampleThreads, 0, stream>>>(logits, ld, V, work, temperature, top_k, top_p,
+                                                  rep_penalty, pen_tokens, pen_counts, pen_offsets,
+                                                  uniform, out);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,163 @@
+"""The step function: one batch of (request, its next tokens) through the
+model, from the cache, to logits at the wanted rows.
+
+A batch may hold portions of prompts beside single decoded tokens, cut
+anywhere. Only the tokens given are run; everything earlier comes from the
+cache. The reference's counterpart is `Model::forward_batch`
+(src/models/model.hip:994-1065): rows = (token, position, sequence slot),
+groups = runs of equal slots (:950-961), logits for the last row of each group
+only (:727-755), and a host sync per sparse layer (src/ops/moe.hip:53). Here
+positions come from the cache manager, logits are returned for any asked
+rows, and nothing inside a step waits for the device.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..config.options import EngineOptions
+from ..models.spec import ModelSpec
+from ..parts.base import CacheView, CallInfo, StepContext, WeightBinder
+from ..weights.source import check_tensors
+
+_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+@dataclass
+class Chunk:
+    """The next tokens of one request in a step and the rows (indices into
+    `tokens`) whose logits are wanted."""
+    slot: int
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=list)
+
+
+class ModelRunner:
+    """Owns the bound model, the cache manager and the step function."""
+
+    def __init__(self, spec: ModelSpec, source, options: EngineOptions, ops=None,
+                 where: str = "model"):
+        options.validate()
+        self.spec = spec
+        self.options = options
+        self.device = torch.device(options.device)
+        self.act_dtype = _DTYPES[options.dtype]
+        if ops is None:
+            from ..kernels import load_ops
+            ops = load_ops()
+        self.ops = ops
+        check_tensors(source.shapes(), spec.tensor_specs(), where)
+        spec.bind(WeightBinder(source, self.device, self.act_dtype))
+
+        # one cache instance per plan entry that writes keys and values
+        needs = []
+        self._state_range: List[Optional[slice]] = []
+        floats = 0
+        for call in spec.plan:
+            mixer = spec.blocks[call.layer].mixer
+            needs.append(mixer.cache_need() if call.cache_from is None else None)
+            n = mixer.state_floats()
+            self._state_range.append(slice(floats, floats + n) if n else None)
+            floats += n
+        self.cache = CacheManager(needs, options.page_size, options.pool_pages(),
+                                  options.num_sequences, options.max_context, floats)
+        self.cache.allocate_pools(self.device, self.act_dtype)
+        self.vocab_size = spec.vocab_size
+        self.steps_run = 0
+
+    # ---- requests --------------------------------------------------------------
+    def open(self) -> int:
+        return self.cache.acquire()
+
+    def close(self, slot: int) -> None:
+        self.cache.release(slot)
+
+    # ---- the step ----------------------------------------------------------------
+    def step(self, chunks: Sequence[Chunk]) -> Optional[torch.Tensor]:
+        """Run one batch. Returns 32-bit logits [R, vocab] on the device for
+        the wanted rows, in the order of the chunks and of their `want`, or
+        None if none are wanted. Raises OutOfPages (nothing run, nothing
+        reserved beyond what fits) when pages do not suffice."""
+        if not chunks:
+            return None
+        cache = self.cache
+        slots = [c.slot for c in chunks]
+        if len(set(slots)) != len(slots):
+            raise ValueError("a request may appear once in a step")
+        pos0 = [cache.length(c.slot) for c in chunks]
+        for c in chunks:
+            if len(c.tokens) < 1:
+                raise ValueError("a request in a step brings at least one token")
+        # pages for all requests of the step, or for none
+        cache.reserve_all([(c.slot, p + len(c.tokens)) for c, p in zip(chunks, pos0)])
+        T = sum(len(c.tokens) for c in chunks)
+        S = len(chunks)
+        tokens = np.empty(T, np.int32)
+        positions = np.empty(T, np.int32)
+        row_seq = np.empty(T, np.int32)
+        row_start = np.empty(S, np.int32)
+        qlen = np.empty(S, np.int32)
+        want_rows: List[int] = []
+        r = 0
+        for i, (c, p) in enumerate(zip(chunks, pos0)):
+            n = len(c.tokens)
+            tokens[r:r + n] = np.asarray(c.tokens, dtype=np.int64)
+            positions[r:r + n] = np.arange(p, p + n)
+            row_seq[r:r + n] = i
+            row_start[i] = r
+            qlen[i] = n
+            for w in c.want:
+                if not 0 <= w < n:
+                    raise ValueError(f"wanted row {w} is outside the request's {n} tokens")
+                want_rows.append(r + w)
+            r += n
+        if tokens.min() < 0 or tokens.max() >= self.vocab_size:
+            raise ValueError(f"token id outside [0, {self.vocab_size})")
+        tables = [cache.block_table(g, slots) for g in range(len(cache.groups))]
+        parts = [tokens, positions, row_seq, np.asarray(slots, np.int32), row_start, qlen,
+                 np.asarray(pos0, np.int32), np.asarray(want_rows, np.int32)]
+        parts += [t.reshape(-1) for t in tables]
+        sizes = [x.size for x in parts]
+        host = torch.from_numpy(np.concatenate(parts)).pin_memory() \
+            if self.device.type == "cuda" else torch.from_numpy(np.concatenate(parts))
+        dev = host.to(self.device, non_blocking=True)
+        views = []
+        o = 0
+        for n in sizes:
+            views.append(dev[o:o + n])
+            o += n
+        d_tables = [v.view(S, t.shape[1]) for v, t in zip(views[8:], tables)]
+        ctx = StepContext(
+            ops=self.ops, act_dtype=self.act_dtype, device=self.device, T=T, S=S,
+            tokens=views[0], positions=views[1], row_seq=views[2], seq_slots=views[3],
+            seq_row_start=views[4], seq_qlen=views[5], seq_pos0=views[6],
+            max_qlen=int(qlen.max()), max_kv_len=int(max(p + len(c.tokens)
+                                                         for c, p in zip(chunks, pos0))),
+            all_decode=bool(qlen.max() == 1))
+        ctx.scratch["host_qlen"] = qlen
+        ctx.scratch["host_pos0"] = np.asarray(pos0, np.int32)
+        logits = self.spec.forward(ctx, self._call_infos(d_tables), views[7] if want_rows else None)
+        for c, p in zip(chunks, pos0):
+            cache.commit(c.slot, p + len(c.tokens))
+        self.steps_run += 1
+        return logits
+
+    def _call_infos(self, d_tables: List[torch.Tensor]) -> List[CallInfo]:
+        cache = self.cache
+        infos = []
+        for i, call in enumerate(self.spec.plan):
+            owner = i if call.cache_from is None else call.cache_from
+            view = None
+            if owner in cache.pools:
+                g = cache.group_of_instance[owner]
+                k_pool, v_pool = cache.pools[owner]
+                view = CacheView(k_pool, v_pool, d_tables[g], cache.page_size,
+                                 cache.groups[g].window)
+            rng = self._state_range[i]
+            state = cache.state[:, rng] if rng is not None else None
+            infos.append(CallInfo(cache=view, writes_cache=call.cache_from is None, state=state))
+        return infos

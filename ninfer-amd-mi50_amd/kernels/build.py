@@ -1,0 +1,124 @@
+"""Compiles the HIP sources under csrc/ for gfx950 into one shared library.
+
+The library is built in-tree (csrc/_build/) when the tree is writable, else in
+a per-user temporary folder. `ensure_built()` loads nothing and compiles only
+when no library matches the current sources (a hash of the sources and flags
+is kept beside it); `build(force=True)` always compiles.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import glob
+import hashlib
+import os
+import subprocess
+import sys
+import tempfile
+import time
+from typing import List, Optional
+
+CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
+LIB_NAME = "libninfer_hip.so"
+ARCH = "gfx950"
+FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC",
+         # packed 32-bit float instructions are kept out of all device code
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.isfile(cand):
+            return cand
+    return "hipcc"
+
+
+def sources() -> List[str]:
+    return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+
+
+def _fingerprint() -> str:
+    h = hashlib.sha256(" ".join(FLAGS).encode())
+    for path in sources() + sorted(glob.glob(os.path.join(CSRC, "*.h"))):
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def _build_dirs() -> List[str]:
+    uid = os.getuid() if hasattr(os, "getuid") else 0
+    return [os.path.join(CSRC, "_build"),
+            os.path.join(tempfile.gettempdir(), f"ninfer_hip_build_{uid}")]
+
+
+def _matching_library() -> Optional[str]:
+    want = _fingerprint()
+    for d in _build_dirs():
+        lib, stamp = os.path.join(d, LIB_NAME), os.path.join(d, "fingerprint")
+        if os.path.isfile(lib) and os.path.isfile(stamp):
+            with open(stamp) as f:
+                if f.read().strip() == want:
+                    return lib
+    return None
+
+
+def _say(msg: str) -> None:
+    print(f"[ninfer build] {msg}", file=sys.stderr, flush=True)
+
+
+def _run(cmd: List[str]) -> None:
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    noise = "is not a recognized feature for this target"
+    out = "\n".join(l for l in p.stdout.splitlines() if noise not in l)
+    if p.returncode != 0:
+        raise RuntimeError(f"command failed ({p.returncode}): {' '.join(cmd)}\n{out}")
+    if out.strip():
+        _say(out)
+
+
+def build(force: bool = True, jobs: int = 8) -> str:
+    """Compile every source and link the library; returns its path."""
+    if not force:
+        lib = _matching_library()
+        if lib:
+            return lib
+    out_dir = None
+    for d in _build_dirs():
+        try:
+            os.makedirs(d, exist_ok=True)
+            with open(os.path.join(d, ".probe"), "w"):
+                pass
+            os.remove(os.path.join(d, ".probe"))
+            out_dir = d
+            break
+        except OSError:
+            continue
+    if out_dir is None:
+        raise RuntimeError("no writable folder to build the HIP library in")
+    srcs = sources()
+    if not srcs:
+        raise RuntimeError(f"no HIP sources under {CSRC}")
+    hipcc = _hipcc()
+    _say(f"compiling {len(srcs)} HIP sources for {ARCH} into {out_dir}")
+    t0 = time.time()
+    objs = [os.path.join(out_dir, os.path.basename(s)[:-4] + ".o") for s in srcs]
+
+    def one(pair):
+        src, obj = pair
+        _run([hipcc, *FLAGS, "-I", CSRC, "-c", src, "-o", obj])
+        _say(f"  {os.path.basename(src)} done ({time.time() - t0:.0f} s)")
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(one, zip(srcs, objs)))
+    lib = os.path.join(out_dir, LIB_NAME)
+    _run([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", lib + ".tmp", *objs])
+    os.replace(lib + ".tmp", lib)
+    with open(os.path.join(out_dir, "fingerprint"), "w") as f:
+        f.write(_fingerprint())
+    _say(f"built {lib} in {time.time() - t0:.0f} s")
+    return lib
+
+
+def ensure_built() -> str:
+    """Path of a library that matches the sources; compiles if there is none."""
+    return build(force=False)

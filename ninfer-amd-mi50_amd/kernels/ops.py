@@ -1,0 +1,306 @@
+"""The kernel library as Python calls on torch tensors.
+
+Every method checks shapes and dtypes on the host, then enqueues hand-written
+gfx950 kernels from the HIP library on torch's current stream. There is no
+other implementation behind these calls: if the library cannot be built or
+loaded, `load_ops` raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .build import ensure_built
+
+_c_int_p = ctypes.c_void_p
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    """The kernel library refused a call (bad size, dtype or launch)."""
+
+
+class _GemmArgs(ctypes.Structure):
+    _fields_ = [("A", ctypes.c_void_p), ("W", ctypes.c_void_p), ("C", ctypes.c_void_p),
+                ("bias", ctypes.c_void_p), ("offsets", ctypes.c_void_p),
+                ("a_index", ctypes.c_void_p), ("c_index", ctypes.c_void_p),
+                ("w_group_stride", ctypes.c_int64),
+                ("M", ctypes.c_int), ("N", ctypes.c_int), ("K", ctypes.c_int),
+                ("lda", ctypes.c_int), ("ldc", ctypes.c_int), ("groups", ctypes.c_int),
+                ("a_div", ctypes.c_int), ("in_dtype", ctypes.c_int), ("out_dtype", ctypes.c_int),
+                ("epilogue", ctypes.c_int)]
+
+
+class _AttnArgs(ctypes.Structure):
+    _fields_ = [("q", ctypes.c_void_p), ("kpool", ctypes.c_void_p), ("vpool", ctypes.c_void_p),
+                ("out", ctypes.c_void_p), ("block_table", ctypes.c_void_p),
+                ("positions", ctypes.c_void_p), ("row_seq", ctypes.c_void_p),
+                ("seq_row_start", ctypes.c_void_p), ("seq_qlen", ctypes.c_void_p),
+                ("seq_pos0", ctypes.c_void_p), ("workspace", ctypes.c_void_p),
+                ("workspace_floats", ctypes.c_int64),
+                ("q_stride", ctypes.c_int), ("bt_stride", ctypes.c_int), ("T", ctypes.c_int),
+                ("S", ctypes.c_int), ("Hq", ctypes.c_int), ("Hkv", ctypes.c_int),
+                ("D", ctypes.c_int), ("page_size", ctypes.c_int), ("window", ctypes.c_int),
+                ("scale", ctypes.c_float), ("dtype", ctypes.c_int), ("max_qlen", ctypes.c_int),
+                ("max_kv_len", ctypes.c_int)]
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(t: torch.Tensor, name: str, dtype=None, dims: Optional[int] = None) -> None:
+    _need(t.is_cuda, f"{name} must be on the GPU")
+    _need(t.is_contiguous(), f"{name} must be contiguous")
+    if dtype is not None:
+        _need(t.dtype == dtype, f"{name} must be {dtype}, is {t.dtype}")
+    if dims is not None:
+        _need(t.dim() == dims, f"{name} must have {dims} dimensions, has {t.dim()}")
+
+
+class HipOps:
+    def __init__(self, lib_path: Optional[str] = None):
+        self.lib_path = lib_path or ensure_built()
+        self.lib = ctypes.CDLL(self.lib_path)
+        self.lib.ninfer_last_error.restype = ctypes.c_char_p
+        self.force_generic = False  # tests: run the plain kernels whatever the shape
+        self._attn_ws = None
+
+    # ---- helpers ----------------------------------------------------------------
+    def _stream(self) -> ctypes.c_void_p:
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def _ok(self, rc: int) -> None:
+        if rc != 0:
+            raise KernelError(self.lib.ninfer_last_error().decode())
+
+    def device_info(self):
+        cu, lds = ctypes.c_int(), ctypes.c_int()
+        arch = ctypes.create_string_buffer(128)
+        self._ok(self.lib.ninfer_device_info(ctypes.byref(cu), ctypes.byref(lds), arch, 128))
+        return {"cu_count": cu.value, "lds_bytes": lds.value, "arch": arch.value.decode()}
+
+    # ---- row-wise ---------------------------------------------------------------
+    def embed(self, tokens, table, out):
+        _dev(tokens, "tokens", torch.int32, 1)
+        _dev(table, "table", dims=2)
+        _dev(out, "out", torch.float32, 2)
+        _need(out.shape == (tokens.shape[0], table.shape[1]), "embed: out has the wrong shape")
+        self._ok(self.lib.ninfer_embed(
+            ctypes.c_void_p(tokens.data_ptr()), ctypes.c_void_p(table.data_ptr()),
+            ctypes.c_void_p(out.data_ptr()), tokens.shape[0], table.shape[1], _DT[table.dtype],
+            self._stream()))
+
+    def rmsnorm(self, x, gain, eps, out, delta=None, rows=None):
+        _dev(x, "x", torch.float32, 2)
+        _dev(gain, "gain", torch.float32, 1)
+        _dev(out, "out", dims=2)
+        h = x.shape[1]
+        _need(gain.shape[0] == h and out.shape[1] == h, "rmsnorm: widths differ")
+        if delta is not None:
+            _dev(delta, "delta", out.dtype, 2)
+            _need(delta.shape == x.shape, "rmsnorm: delta has the wrong shape")
+        if rows is not None:
+            _dev(rows, "rows", torch.int32, 1)
+            _need(out.shape[0] == rows.shape[0], "rmsnorm: out has the wrong number of rows")
+        else:
+            _need(out.shape[0] == x.shape[0], "rmsnorm: out has the wrong number of rows")
+        self._ok(self.lib.ninfer_rmsnorm(
+            ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(_ptr(delta)),
+            ctypes.c_void_p(gain.data_ptr()), ctypes.c_void_p(out.data_ptr()),
+            ctypes.c_void_p(_ptr(rows)), out.shape[0], h, ctypes.c_float(eps), _DT[out.dtype],
+            self._stream()))
+
+    def rope_kv_write(self, qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv, head_dim,
+                      k_pool, v_pool, block_table, page_size, write_kv=True):
+        _dev(qkv, "qkv", dims=2)
+        t = qkv.shape[0]
+        width = (n_q + 2 * n_kv) * head_dim
+        _need(qkv.shape[1] == width, f"rope_kv_write: qkv width {qkv.shape[1]} != {width}")
+        if bias is not None:
+            _dev(bias, "bias", torch.float32, 1)
+            _need(bias.shape[0] == width, "rope_kv_write: bias has the wrong size")
+        _dev(positions, "positions", torch.int32, 1)
+        _dev(row_seq, "row_seq", torch.int32, 1)
+        _need(positions.shape[0] == t and row_seq.shape[0] == t, "rope_kv_write: index sizes")
+        if rot_dim:
+            _dev(inv_freq, "inv_freq", torch.float32, 1)
+            _need(inv_freq.shape[0] == rot_dim // 2, "rope_kv_write: table size != rot_dim / 2")
+        _dev(k_pool, "k_pool", qkv.dtype, 4)
+        _dev(v_pool, "v_pool", qkv.dtype, 4)
+        _need(k_pool.shape == v_pool.shape and k_pool.shape[1:] == (n_kv, page_size, head_dim),
+              f"rope_kv_write: pools {tuple(k_pool.shape)} do not fit (kv heads {n_kv}, page "
+              f"{page_size}, head {head_dim})")
+        _dev(block_table, "block_table", torch.int32, 2)
+        self._ok(self.lib.ninfer_rope_kv_write(
+            ctypes.c_void_p(qkv.data_ptr()), ctypes.c_void_p(_ptr(bias)),
+            ctypes.c_void_p(positions.data_ptr()), ctypes.c_void_p(row_seq.data_ptr()),
+            ctypes.c_void_p(_ptr(inv_freq) if rot_dim else None), rot_dim, n_q, n_kv, head_dim,
+            ctypes.c_void_p(k_pool.data_ptr()), ctypes.c_void_p(v_pool.data_ptr()),
+            ctypes.c_void_p(block_table.data_ptr()), block_table.shape[1], page_size,
+            1 if write_kv else 0, t, _DT[qkv.dtype], self._stream()))
+
+    def moe_combine(self, residual, y, wts, shared=None, gate=None):
+        _dev(residual, "residual", torch.float32, 2)
+        _dev(y, "y", dims=2)
+        _dev(wts, "wts", torch.float32, 2)
+        t, h = residual.shape
+        k = wts.shape[1]
+        _need(wts.shape[0] == t and y.shape == (t * k, h), "moe_combine: shapes differ")
+        if shared is not None:
+            _dev(shared, "shared", y.dtype, 2)
+            _need(shared.shape == (t, h), "moe_combine: shared has the wrong shape")
+        if gate is not None:
+            _dev(gate, "gate", torch.float32)
+            _need(gate.numel() == t, "moe_combine: gate has the wrong size")
+        self._ok(self.lib.ninfer_moe_combine(
+            ctypes.c_void_p(residual.data_ptr()), ctypes.c_void_p(y.data_ptr()),
+            ctypes.c_void_p(wts.data_ptr()), ctypes.c_void_p(_ptr(shared)),
+            ctypes.c_void_p(_ptr(gate)), t, h, k, _DT[y.dtype], self._stream()))
+
+    # ---- products ---------------------------------------------------------------
+    def _gemm(self, a, w, c, *, n, k, m, bias=None, offsets=None, a_index=None, c_index=None,
+              a_div=1, groups=1, epilogue=0, w_group_stride=0):
+        args = _GemmArgs(a.data_ptr(), w.data_ptr(), c.data_ptr(), _ptr(bias), _ptr(offsets),
+                         _ptr(a_index), _ptr(c_index), w_group_stride, m, n, k, a.shape[1],
+                         c.shape[1], groups, a_div, _DT[a.dtype], _DT[c.dtype], epilogue)
+        self._ok(self.lib.ninfer_gemm(ctypes.byref(args), 1 if self.force_generic else 0,
+                                      self._stream()))
+
+    def linear(self, x, w, out, bias=None):
+        """out = x w^T (+ bias); out may be 32-bit whatever the inputs are."""
+        _dev(x, "x", dims=2)
+        _dev(w, "w", x.dtype, 2)
+        _dev(out, "out", dims=2)
+        _need(x.shape[1] == w.shape[1], f"linear: x has {x.shape[1]} columns, w has {w.shape[1]}")
+        _need(out.shape == (x.shape[0], w.shape[0]), "linear: out has the wrong shape")
+        _need(out.dtype in (x.dtype, torch.float32), "linear: bad out dtype")
+        if bias is not None:
+            _dev(bias, "bias", torch.float32, 1)
+            _need(bias.shape[0] == w.shape[0], "linear: bias has the wrong size")
+        self._gemm(x, w, out, m=x.shape[0], n=w.shape[0], k=x.shape[1], bias=bias)
+
+    def swiglu_linear(self, x, w_gate_up, out):
+        """out = silu(x Wg^T) * (x Wu^T), Wg = rows [0, I), Wu = rows [I, 2I)."""
+        _dev(x, "x", dims=2)
+        _dev(w_gate_up, "w_gate_up", x.dtype, 2)
+        _dev(out, "out", x.dtype, 2)
+        inner = w_gate_up.shape[0] // 2
+        _need(w_gate_up.shape == (2 * inner, x.shape[1]), "swiglu_linear: weight shape")
+        _need(out.shape == (x.shape[0], inner), "swiglu_linear: out has the wrong shape")
+        self._gemm(x, w_gate_up, out, m=x.shape[0], n=inner, k=x.shape[1], epilogue=1)
+
+    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out):
+        """out[r] = swiglu of row order[r] // top_k of x by the expert that owns
+        sorted position r."""
+        _dev(x, "x", dims=2)
+        _dev(w_gate_up, "w_gate_up", x.dtype, 3)
+        _dev(out, "out", x.dtype, 2)
+        _dev(offsets, "offsets", torch.int32, 1)
+        _dev(order, "order", torch.int32, 1)
+        e, two_i, h = w_gate_up.shape
+        inner = two_i // 2
+        n = order.shape[0]
+        _need(h == x.shape[1] and two_i == 2 * inner, "grouped_swiglu: weight shape")
+        _need(offsets.shape[0] == e + 1, "grouped_swiglu: offsets size")
+        _need(n == x.shape[0] * top_k and out.shape == (n, inner), "grouped_swiglu: row counts")
+        self._gemm(x, w_gate_up, out, m=n, n=inner, k=h, offsets=offsets, a_index=order,
+                   a_div=top_k, groups=e, epilogue=1, w_group_stride=two_i * h)
+
+    def grouped_down(self, h, w_down, offsets, order, out):
+        """out[order[r]] = h[r] Wd_e^T for the expert e that owns sorted position r."""
+        _dev(h, "h", dims=2)
+        _dev(w_down, "w_down", h.dtype, 3)
+        _dev(out, "out", h.dtype, 2)
+        _dev(offsets, "offsets", torch.int32, 1)
+        _dev(order, "order", torch.int32, 1)
+        e, hidden, inner = w_down.shape
+        n = order.shape[0]
+        _need(inner == h.shape[1] and h.shape[0] == n, "grouped_down: input shape")
+        _need(out.shape == (n, hidden) and offsets.shape[0] == e + 1, "grouped_down: shapes")
+        self._gemm(h, w_down, out, m=n, n=hidden, k=inner, offsets=offsets, c_index=order,
+                   groups=e, w_group_stride=hidden * inner)
+
+    # ---- routing ------------------------------------------------------------------
+    def router_topk(self, logits, experts, top_k, renorm, ids, wts):
+        _dev(logits, "logits", torch.float32, 2)
+        _dev(ids, "ids", torch.int32, 2)
+        _dev(wts, "wts", torch.float32, 2)
+        t = logits.shape[0]
+        _need(ids.shape == (t, top_k) and wts.shape == (t, top_k), "router_topk: output shapes")
+        self._ok(self.lib.ninfer_router_topk(
+            ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, experts, top_k,
+            1 if renorm else 0, ctypes.c_void_p(ids.data_ptr()), ctypes.c_void_p(wts.data_ptr()),
+            self._stream()))
+
+    def moe_align(self, ids, experts, offsets, order):
+        _dev(ids, "ids", torch.int32)
+        _dev(offsets, "offsets", torch.int32, 1)
+        _dev(order, "order", torch.int32, 1)
+        _need(offsets.shape[0] == experts + 1 and order.shape[0] == ids.numel(),
+              "moe_align: output sizes")
+        self._ok(self.lib.ninfer_moe_align(
+            ctypes.c_void_p(ids.data_ptr()), ids.numel(), experts,
+            ctypes.c_void_p(offsets.data_ptr()), ctypes.c_void_p(order.data_ptr()),
+            self._stream()))
+
+    # ---- attention ------------------------------------------------------------------
+    def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,
+                        page_size, window, scale, out):
+        """Attention of the rows' query heads (the first n_q * head_dim columns
+        of `qkv`) over their requests' cached keys and values."""
+        _dev(qkv, "qkv", dims=2)
+        _dev(k_pool, "k_pool", qkv.dtype, 4)
+        _dev(v_pool, "v_pool", qkv.dtype, 4)
+        _dev(out, "out", qkv.dtype, 2)
+        _dev(block_table, "block_table", torch.int32, 2)
+        t = qkv.shape[0]
+        _need(out.shape == (t, n_q * head_dim), "paged_attention: out has the wrong shape")
+        _need(k_pool.shape == v_pool.shape and k_pool.shape[1:] == (n_kv, page_size, head_dim),
+              "paged_attention: pools do not fit the head layout")
+        _need(block_table.shape[0] == ctx.S, "paged_attention: block table rows != requests")
+        _need(ctx.positions.shape[0] == t, "paged_attention: positions size")
+        args = _AttnArgs(
+            qkv.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), out.data_ptr(),
+            block_table.data_ptr(), ctx.positions.data_ptr(), ctx.row_seq.data_ptr(),
+            ctx.seq_row_start.data_ptr(), ctx.seq_qlen.data_ptr(), ctx.seq_pos0.data_ptr(),
+            None, 0, qkv.shape[1], block_table.shape[1], t, ctx.S, n_q, n_kv, head_dim, page_size,
+            int(window or 0), float(scale), _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len)
+        self._ok(self.lib.ninfer_paged_attention(ctypes.byref(args),
+                                                 1 if self.force_generic else 0, self._stream()))
+
+    # ---- sampling -------------------------------------------------------------------
+    def sample(self, logits, temperature, uniform, out, top_k=None, top_p=None, rep_penalty=None,
+               pen_tokens=None, pen_counts=None, pen_offsets=None):
+        _dev(logits, "logits", torch.float32, 2)
+        r, v = logits.shape
+        _dev(temperature, "temperature", torch.float32, 1)
+        _dev(uniform, "uniform", torch.float32, 1)
+        _dev(out, "out", torch.int32, 1)
+        _need(temperature.shape[0] == r and uniform.shape[0] == r and out.shape[0] == r,
+              "sample: per-row arrays have the wrong size")
+        for name, t, dt in (("top_k", top_k, torch.int32), ("top_p", top_p, torch.float32),
+                            ("rep_penalty", rep_penalty, torch.float32)):
+            if t is not None:
+                _dev(t, name, dt, 1)
+                _need(t.shape[0] == r, f"sample: {name} has the wrong size")
+        if pen_offsets is not None:
+            _dev(pen_offsets, "pen_offsets", torch.int32, 1)
+            _dev(pen_tokens, "pen_tokens", torch.int32, 1)
+            _dev(pen_counts, "pen_counts", torch.int32, 1)
+            _need(pen_offsets.shape[0] == r + 1, "sample: pen_offsets has the wrong size")
+        work = torch.empty((r, v), dtype=torch.float32, device=logits.device)
+        self._ok(self.lib.ninfer_sample(
+            ctypes.c_void_p(logits.data_ptr()), logits.stride(0), v, r,
+            ctypes.c_void_p(work.data_ptr()), ctypes.c_void_p(temperature.data_ptr()),
+            ctypes.c_void_p(_ptr(top_k)), ctypes.c_void_p(_ptr(top_p)),
+            ctypes.c_void_p(_ptr(rep_penalty)), ctypes.c_void_p(_ptr(pen_tokens)),
+            ctypes.c_void_p(_ptr(pen_counts)), ctypes.c_void_p(_ptr(pen_offsets)),
+            ctypes.c_void_p(uniform.data_ptr()), ctypes.c_void_p(out.data_ptr()), self._stream()))

@@ -1,0 +1,14 @@
+from .attention import Attention
+from .base import (Block, CacheNeed, CacheView, CallInfo, FeedForward, Mixer, Norm, Part,
+                   PositionEncoding, StepContext, WeightBinder)
+from .block import PreNormBlock
+from .embedding import LMHead, TokenEmbedding
+from .mlp import SwiGLU
+from .moe import RoutedExperts, SoftmaxTopKRouter, SparseMoE
+from .norm import RMSNorm
+from .rotary import NoPosition, Rotary
+
+__all__ = ["Attention", "Block", "CacheNeed", "CacheView", "CallInfo", "FeedForward", "Mixer",
+           "Norm", "Part", "PositionEncoding", "StepContext", "WeightBinder", "PreNormBlock",
+           "LMHead", "TokenEmbedding", "SwiGLU", "RoutedExperts", "SoftmaxTopKRouter",
+           "SparseMoE", "RMSNorm", "NoPosition", "Rotary"]

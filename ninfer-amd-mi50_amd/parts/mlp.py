@@ -1,0 +1,53 @@
+"""Dense SwiGLU feed-forward: (silu(x Wg^T) * (x Wu^T)) Wd^T, no biases.
+
+Gate and up weights are stacked into one [2 I, hidden] matrix, rows [0, I)
+gate and [I, 2I) up (reference src/models/model.hip:585-617); the activation
+runs in the product's epilogue (the reference does so only for one row,
+src/ops/gemv.hip:103-166, and otherwise in a kernel of its own,
+src/ops/kernels.hip:131-140).
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..registry import register_part
+from ..weights.source import TensorSpec
+from .base import FeedForward, StepContext, WeightBinder
+
+
+class SwiGLU(FeedForward):
+    def __init__(self, prefix: str, hidden: int, inner: int):
+        self.prefix = prefix
+        self.hidden = hidden
+        self.inner = inner
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        p = self.prefix
+        return {p + "gate_proj.weight": TensorSpec((self.inner, self.hidden)),
+                p + "up_proj.weight": TensorSpec((self.inner, self.hidden)),
+                p + "down_proj.weight": TensorSpec((self.hidden, self.inner))}
+
+    def bind(self, w: WeightBinder) -> None:
+        p = self.prefix
+        self.w_gate_up = torch.empty((2 * self.inner, self.hidden), dtype=w.act_dtype,
+                                     device=w.device)
+        w.matrix_into(p + "gate_proj.weight", self.w_gate_up[:self.inner])
+        w.matrix_into(p + "up_proj.weight", self.w_gate_up[self.inner:])
+        self.w_down = w.matrix(p + "down_proj.weight")
+
+    def run(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
+        h = ctx.empty((x.shape[0], self.inner))
+        ctx.ops.swiglu_linear(x, self.w_gate_up, h)
+        out = ctx.empty((x.shape[0], self.hidden))
+        ctx.ops.linear(h, self.w_down, out)
+        return out
+
+    def forward(self, ctx: StepContext, x, residual):
+        return self.run(ctx, x)
+
+
+register_part("feed_forward", "swiglu", SwiGLU)

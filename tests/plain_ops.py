@@ -1,0 +1,166 @@
+"""A plain PyTorch twin of every kernel of the HIP library, with the same call
+signatures, computing in 32-bit with elementary torch operations.
+
+Used two ways: on the GPU, each HIP kernel is compared with its twin here on
+random inputs; on the CPU, the engine's host logic (batch building, cache
+manager, block tables, plan, scheduler) is run end to end with these twins in
+place of the kernels, which have no CPU form. Formula sources are the same
+reference lines that tests/plain_model.py cites.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+
+def _f(t):
+    return t.to(torch.float32)
+
+
+class PlainOps:
+    force_generic = False
+
+    def embed(self, tokens, table, out):
+        out.copy_(_f(table[tokens.long()]))
+
+    def rmsnorm(self, x, gain, eps, out, delta=None, rows=None):
+        if rows is None:
+            if delta is not None:
+                x += _f(delta)
+            v = x
+        else:
+            v = x[rows.long()]
+            if delta is not None:
+                v = v + _f(delta[rows.long()])
+        ms = (v * v).sum(-1, keepdim=True) / v.shape[-1]
+        out.copy_((v * torch.rsqrt(ms + eps) * gain).to(out.dtype))
+
+    def rope_kv_write(self, qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv, head_dim,
+                      k_pool, v_pool, block_table, page_size, write_kv=True):
+        t = qkv.shape[0]
+        x = _f(qkv)
+        if bias is not None:
+            x = x + bias
+        x = x.view(t, n_q + 2 * n_kv, head_dim).clone()
+        if rot_dim:
+            half = rot_dim // 2
+            phi = positions.to(torch.float32)[:, None] * inv_freq[None, :]
+            c, s = torch.cos(phi)[:, None, :], torch.sin(phi)[:, None, :]
+            qk = x[:, :n_q + n_kv, :]
+            x1, x2 = qk[..., :half].clone(), qk[..., half:rot_dim].clone()
+            qk[..., :half] = x1 * c - x2 * s
+            qk[..., half:rot_dim] = x1 * s + x2 * c
+        qkv.view(t, n_q + 2 * n_kv, head_dim)[:, :n_q] = x[:, :n_q].to(qkv.dtype)
+        if not write_kv:
+            return
+        pos = positions.long()
+        page = block_table[row_seq.long(), pos // page_size].long()
+        assert (page >= 0).all(), "write into a page that is not held"
+        slot = pos % page_size
+        k_pool[page, :, slot, :] = x[:, n_q:n_q + n_kv].to(k_pool.dtype)
+        v_pool[page, :, slot, :] = x[:, n_q + n_kv:].to(v_pool.dtype)
+
+    def moe_combine(self, residual, y, wts, shared=None, gate=None):
+        t, h = residual.shape
+        k = wts.shape[1]
+        acc = (_f(y).view(t, k, h) * wts[:, :, None]).sum(1)
+        if shared is not None:
+            g = torch.sigmoid(gate.reshape(t, 1)) if gate is not None else 1.0
+            acc = acc + g * _f(shared)
+        residual += acc
+
+    def linear(self, x, w, out, bias=None):
+        r = _f(x) @ _f(w).T
+        if bias is not None:
+            r = r + bias
+        out.copy_(r.to(out.dtype))
+
+    def swiglu_linear(self, x, w_gate_up, out):
+        inner = w_gate_up.shape[0] // 2
+        g = _f(x) @ _f(w_gate_up[:inner]).T
+        u = _f(x) @ _f(w_gate_up[inner:]).T
+        out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
+
+    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out):
+        e, two_i, _ = w_gate_up.shape
+        inner = two_i // 2
+        off = offsets.tolist()
+        for g in range(e):
+            rows = order[off[g]:off[g + 1]].long()
+            if rows.numel() == 0:
+                continue
+            xs = _f(x[rows // top_k])
+            gg = xs @ _f(w_gate_up[g, :inner]).T
+            uu = xs @ _f(w_gate_up[g, inner:]).T
+            out[off[g]:off[g + 1]] = (gg / (1 + torch.exp(-gg)) * uu).to(out.dtype)
+
+    def grouped_down(self, h, w_down, offsets, order, out):
+        e = w_down.shape[0]
+        off = offsets.tolist()
+        for g in range(e):
+            rows = order[off[g]:off[g + 1]].long()
+            if rows.numel() == 0:
+                continue
+            out[rows] = (_f(h[off[g]:off[g + 1]]) @ _f(w_down[g]).T).to(out.dtype)
+
+    def router_topk(self, logits, experts, top_k, renorm, ids, wts):
+        l = logits[:, :experts]
+        p = torch.exp(l - l.max(-1, keepdim=True).values)
+        p = p / p.sum(-1, keepdim=True)
+        work = p.clone()
+        for j in range(top_k):
+            best = work.max(-1).values
+            # lowest index among the maxima
+            idx = torch.argmax((work == best[:, None]).to(torch.int32), dim=-1)
+            ids[:, j] = idx.to(torch.int32)
+            wts[:, j] = best
+            work[torch.arange(work.shape[0]), idx] = -1.0
+        if renorm:
+            wts /= wts.sum(-1, keepdim=True)
+
+    def moe_align(self, ids, experts, offsets, order):
+        flat = ids.reshape(-1).long()
+        counts = torch.bincount(flat, minlength=experts)
+        offsets[0] = 0
+        offsets[1:] = torch.cumsum(counts, 0).to(torch.int32)
+        order.copy_(torch.sort(flat, stable=True).indices.to(torch.int32))
+
+    def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,
+                        page_size, window, scale, out):
+        t = qkv.shape[0]
+        q = _f(qkv[:, :n_q * head_dim]).view(t, n_q, head_dim)
+        group = n_q // n_kv
+        pos = ctx.positions.tolist()
+        seq = ctx.row_seq.tolist()
+        for r in range(t):
+            lo = max(0, pos[r] - window + 1) if window else 0
+            js = torch.arange(lo, pos[r] + 1)
+            pages = block_table[seq[r], js // page_size].long()
+            assert (pages >= 0).all(), "read of a page that is not held"
+            k = _f(k_pool[pages, :, js % page_size, :])  # [n, n_kv, D]
+            v = _f(v_pool[pages, :, js % page_size, :])
+            for h in range(n_q):
+                g = h // group
+                s = (k[:, g, :] @ q[r, h]) * scale
+                p = torch.exp(s - s.max())
+                p = p / p.sum()
+                out[r, h * head_dim:(h + 1) * head_dim] = (p @ v[:, g, :]).to(out.dtype)
+
+    def sample(self, logits, temperature, uniform, out, top_k=None, top_p=None, rep_penalty=None,
+               pen_tokens=None, pen_counts=None, pen_offsets=None):
+        from plain_model import sample_distribution
+        r, v = logits.shape
+        for i in range(r):
+            recent = []
+            if pen_offsets is not None:
+                for e in range(int(pen_offsets[i]), int(pen_offsets[i + 1])):
+                    recent += [int(pen_tokens[e])] * int(pen_counts[e])
+            p = sample_distribution(
+                logits[i].cpu(), float(temperature[i]), int(top_k[i]) if top_k is not None else 0,
+                float(top_p[i]) if top_p is not None else 1.0,
+                float(rep_penalty[i]) if rep_penalty is not None else 1.0, recent)
+            cdf = torch.cumsum(p.double(), 0)
+            idx = int(torch.searchsorted(cdf, torch.tensor(float(uniform[i]) * float(cdf[-1]),
+                                                           dtype=torch.float64), right=True))
+            out[i] = min(idx, v - 1)

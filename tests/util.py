@@ -1,0 +1,129 @@
+"""Helpers shared by the tests: reading a model folder for the plain
+implementation, seeded token ids, and the replay schedules (whole, tail,
+portions, mixed) expressed as steps of (request, tokens, wanted rows)."""
+from __future__ import annotations
+
+import json
+import os
+import random
+from typing import Dict, List, Sequence, Tuple
+
+import torch
+
+
+def read_folder(model_dir: str) -> Tuple[dict, Dict[str, torch.Tensor]]:
+    """config dictionary and name -> 32-bit tensor, read with the safetensors
+    package (independent of the engine's own reader)."""
+    from safetensors import safe_open
+    with open(os.path.join(model_dir, "config.json")) as f:
+        cfg = json.load(f)
+    tensors = {}
+    with safe_open(os.path.join(model_dir, "model.safetensors"), framework="pt") as f:
+        for k in f.keys():
+            tensors[k] = f.get_tensor(k).to(torch.float32)
+    return cfg, tensors
+
+
+def random_tokens(n: int, vocab: int, seed: int) -> List[int]:
+    rng = random.Random(seed)
+    return [rng.randrange(vocab) for _ in range(n)]
+
+
+# A schedule is a list of steps; a step is (entries, end) with entries
+# [(request id, tokens, want rows)] and end = ids finished after the step.
+Step = Tuple[List[Tuple[str, List[int], List[int]]], List[str]]
+
+
+def schedule_whole(rid: str, tokens: Sequence[int]) -> List[Step]:
+    return [([(rid, list(tokens), list(range(len(tokens))))], [rid])]
+
+
+def schedule_tail(rid: str, tokens: Sequence[int], tail: int = 32) -> List[Step]:
+    """All but the last min(tail, n-1) tokens in one step, then one by one."""
+    n = len(tokens)
+    tail = min(tail, n - 1)
+    head = n - tail
+    steps: List[Step] = [([(rid, list(tokens[:head]), list(range(head)))], [])]
+    for i in range(head, n):
+        steps.append(([(rid, [tokens[i]], [0])], [rid] if i == n - 1 else []))
+    return steps
+
+
+def schedule_portions(rid: str, tokens: Sequence[int], seed: int = 0) -> List[Step]:
+    """Portions of changing size, down to two tokens."""
+    sizes = [7, 2, 5, 3, 2, 11, 4, 2, 9]
+    rng = random.Random(seed)
+    rng.shuffle(sizes)
+    steps: List[Step] = []
+    i, j, n = 0, 0, len(tokens)
+    while i < n:
+        m = min(sizes[j % len(sizes)], n - i)
+        if n - i - m == 1:   # never leave a single token for the last portion
+            m += 1
+        j += 1
+        steps.append(([(rid, list(tokens[i:i + m]), list(range(m)))], [rid] if i + m == n else []))
+        i += m
+    return steps
+
+
+def schedule_mixed(requests: Dict[str, Sequence[int]], seed: int = 0, max_live: int = 4,
+                   decode_tail: int = 6) -> List[Step]:
+    """Up to `max_live` live requests with staggered starts: prompt portions of
+    some beside single tokens of others in the same step. Each request is fed
+    in portions (>= 2 tokens) until `decode_tail` tokens remain, which then
+    come one per step. Requests start two steps apart; when one ends the next
+    waiting one starts, so pages given back are used again."""
+    rng = random.Random(seed)
+    waiting = list(requests)
+    live: Dict[str, int] = {}
+    steps: List[Step] = []
+    step_no = 0
+    while waiting or live:
+        if waiting and len(live) < max_live and step_no % 2 == 0:
+            live[waiting.pop(0)] = 0
+        entries, end = [], []
+        for rid in list(live):
+            toks = requests[rid]
+            done = live[rid]
+            left = len(toks) - done
+            if left > decode_tail + 1:
+                m = min(rng.choice([2, 3, 5, 8, 13]), left - decode_tail)
+                if m < 2:
+                    m = left - decode_tail
+            else:
+                m = 1
+            if rng.random() < 0.15 and len(live) > 1:
+                continue  # a request may be left out of a step and go on later
+            entries.append((rid, list(toks[done:done + m]), list(range(m))))
+            live[rid] = done + m
+            if live[rid] == len(toks):
+                end.append(rid)
+                del live[rid]
+        if entries:
+            steps.append((entries, end))
+        step_no += 1
+    return steps
+
+
+def run_schedule(runner, steps: List[Step]) -> Dict[str, torch.Tensor]:
+    """Feed a schedule through a ModelRunner; returns id -> logits [n, vocab]
+    (rows in position order) on the CPU."""
+    from ninfer_amd.engine import Chunk
+    slots: Dict[str, int] = {}
+    rows: Dict[str, List[torch.Tensor]] = {}
+    for entries, end in steps:
+        chunks = []
+        for rid, toks, want in entries:
+            if rid not in slots:
+                slots[rid] = runner.open()
+                rows[rid] = []
+            chunks.append(Chunk(slots[rid], toks, want))
+        logits = runner.step(chunks)
+        o = 0
+        for rid, toks, want in entries:
+            if want:
+                rows[rid].append(logits[o:o + len(want)].float().cpu())
+                o += len(want)
+        for rid in end:
+            runner.close(slots.pop(rid))
+    return {rid: torch.cat(v) for rid, v in rows.items()}
