@@ -1,0 +1,82 @@
+"""The engine on the GPU against the plain implementation: every request
+alone and whole; most of it in one step and the last 32 tokens one by one; in
+portions of changing size; and mixed, up to four live requests with so few
+pages that they are used again. In 32-bit and in bfloat16, for both tiny
+configurations. The 32-bit bound is never widened; bfloat16 is compared with
+the plain implementation run on the bfloat16-rounded weights."""
+import pytest
+import torch
+
+import plain_model
+import util
+from conftest import TINY
+
+pytestmark = pytest.mark.gpu
+
+PROMPTS = {"A": [5, 11, 17, 60], "B": [3, 20, 33, 40, 75]}
+
+
+def bound(dtype):
+    return dict(atol=2e-5, rtol=1e-4) if dtype == "float32" else dict(atol=6e-2, rtol=5e-2)
+
+
+@pytest.fixture(scope="module", params=["A", "B"])
+def case(request, model_dirs):
+    name = request.param
+    cfg = TINY[name][0]
+    out = {"name": name, "cfg": cfg, "dirs": model_dirs[name], "ref": {}, "reqs": {}}
+    for i, n in enumerate(PROMPTS[name]):
+        out["reqs"][f"r{i}"] = util.random_tokens(n + 12, cfg["vocab_size"], 100 + i)
+    for dtype, d in model_dirs[name].items():
+        rcfg, w = util.read_folder(d)
+        out["ref"][dtype] = {k: plain_model.forward(w, rcfg, v) for k, v in out["reqs"].items()}
+    return out
+
+
+def make_runner(case, dtype, page_size=8, num_pages=40):
+    from ninfer_amd import EngineOptions, load_model
+    opt = EngineOptions(dtype=dtype, max_context=128, num_sequences=4, page_size=page_size,
+                        num_pages=num_pages)
+    return load_model(case["dirs"][dtype], opt)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_tail_portions(case, dtype):
+    runner = make_runner(case, dtype)
+    for rid, toks in case["reqs"].items():
+        ref = case["ref"][dtype][rid]
+        for name, sched in (("whole", util.schedule_whole(rid, toks)),
+                            ("tail", util.schedule_tail(rid, toks, 32)),
+                            ("portions", util.schedule_portions(rid, toks, seed=len(toks)))):
+            got = util.run_schedule(runner, sched)[rid]
+            torch.testing.assert_close(got, ref, **bound(dtype),
+                                       msg=lambda m: f"{case['name']} {rid} {name}: {m}")
+    runner.cache.check()
+    assert all(g.allocator.in_use == 0 for g in runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page_size,num_pages", [(4, 60), (16, 16)])
+def test_mixed_with_page_reuse(case, dtype, page_size, num_pages):
+    runner = make_runner(case, dtype, page_size, num_pages)
+    reqs = dict(case["reqs"])
+    sched = util.schedule_mixed(reqs, seed=7)
+    got = util.run_schedule(runner, sched)
+    for rid in reqs:
+        torch.testing.assert_close(got[rid], case["ref"][dtype][rid], **bound(dtype),
+                                   msg=lambda m: f"{case['name']} {rid} mixed: {m}")
+    runner.cache.check()
+    assert runner.cache.pages_reused() > 0, "the pool is small enough that pages are used again"
+    if case["name"] == "B":
+        assert any(g.window_freed > 0 for g in runner.cache.groups)
+
+
+def test_32bit_does_not_depend_on_the_cut(case):
+    """In 32-bit every way of cutting gives the same logits to the last bit or
+    nearly so (far inside the bound against the plain implementation)."""
+    runner = make_runner(case, "float32")
+    rid, toks = "r3", case["reqs"]["r3"]
+    a = util.run_schedule(runner, util.schedule_whole(rid, toks))[rid]
+    b = util.run_schedule(runner, util.schedule_tail(rid, toks, 32))[rid]
+    c = util.run_schedule(runner, util.schedule_portions(rid, toks, 1))[rid]
+    assert torch.equal(a, b) and torch.equal(a, c)

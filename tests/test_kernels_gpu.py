@@ -1,0 +1,314 @@
+"""Each HIP kernel alone against its plain twin (tests/plain_ops.py), in 32-bit
+and in bfloat16, at sizes other than the engine's tiny models: widths and
+vocabularies that are no power of two, odd row counts, experts without rows,
+contexts that end inside a page."""
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from plain_ops import PlainOps
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from ninfer_amd.kernels import load_ops
+    return load_ops()
+
+
+@pytest.fixture(scope="module", params=[False, True], ids=["fast", "generic"])
+def ops_mode(ops, request):
+    ops.force_generic = request.param
+    yield ops
+    ops.force_generic = False
+
+
+def tol(dtype, scale=1.0):
+    return (2e-5 * scale, 1e-4) if dtype == torch.float32 else (2e-2 * scale, 2e-2)
+
+
+def close(a, b, dtype, scale=1.0):
+    atol, rtol = tol(dtype, scale)
+    torch.testing.assert_close(a.float().cpu(), b.float().cpu(), atol=atol, rtol=rtol)
+
+
+def rnd(shape, dtype, gen, scale=1.0):
+    return (torch.randn(shape, generator=gen, device="cuda") * scale).to(dtype)
+
+
+@pytest.fixture()
+def gen():
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1234)
+    return g
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(ops, gen, dtype):
+    table = rnd((301, 72), dtype, gen)
+    tokens = torch.randint(0, 301, (19,), generator=gen, device="cuda", dtype=torch.int32)
+    out, ref = torch.empty(19, 72, device="cuda"), torch.empty(19, 72, device="cuda")
+    ops.embed(tokens, table, out)
+    PlainOps().embed(tokens, table, ref)
+    assert torch.equal(out, ref)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,h", [(1, 64), (7, 200), (33, 2048), (3, 3584)])
+def test_rmsnorm(ops, gen, dtype, rows, h):
+    gain = 1 + 0.1 * torch.randn(h, generator=gen, device="cuda")
+    x = torch.randn(rows, h, generator=gen, device="cuda") * 3
+    delta = rnd((rows, h), dtype, gen)
+    for d in (None, delta):
+        x1, x2 = x.clone(), x.clone()
+        o1, o2 = torch.empty(rows, h, device="cuda", dtype=dtype), torch.empty(
+            rows, h, device="cuda", dtype=dtype)
+        ops.rmsnorm(x1, gain, 1e-5, o1, delta=d)
+        PlainOps().rmsnorm(x2, gain, 1e-5, o2, delta=d)
+        close(o1, o2, dtype)
+        close(x1, x2, torch.float32)
+    sel = torch.tensor([rows - 1, 0], device="cuda", dtype=torch.int32)
+    o1 = torch.empty(2, h, device="cuda", dtype=dtype)
+    o2 = torch.empty_like(o1)
+    x1 = x.clone()
+    ops.rmsnorm(x1, gain, 1e-6, o1, delta=delta, rows=sel)
+    PlainOps().rmsnorm(x.clone(), gain, 1e-6, o2, delta=delta, rows=sel)
+    close(o1, o2, dtype)
+    assert torch.equal(x1, x), "the rows form must leave the residual alone"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 48, 40), (3, 130, 72), (17, 64, 200), (70, 200, 136),
+                                   (129, 96, 64)])
+def test_linear(ops_mode, gen, dtype, m, n, k):
+    ops = ops_mode
+    x, w = rnd((m, k), dtype, gen), rnd((n, k), dtype, gen)
+    bias = torch.randn(n, generator=gen, device="cuda")
+    for out_dtype in {dtype, torch.float32}:
+        for b in (None, bias):
+            o1 = torch.empty(m, n, device="cuda", dtype=out_dtype)
+            o2 = torch.empty_like(o1)
+            ops.linear(x, w, o1, bias=b)
+            PlainOps().linear(x, w, o2, bias=b)
+            close(o1, o2, out_dtype, scale=math.sqrt(k))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,inner,k", [(1, 48, 64), (5, 80, 96), (66, 176, 72)])
+def test_swiglu_linear(ops_mode, gen, dtype, m, inner, k):
+    ops = ops_mode
+    x, w = rnd((m, k), dtype, gen), rnd((2 * inner, k), dtype, gen, 0.3)
+    o1 = torch.empty(m, inner, device="cuda", dtype=dtype)
+    o2 = torch.empty_like(o1)
+    ops.swiglu_linear(x, w, o1)
+    PlainOps().swiglu_linear(x, w, o2)
+    close(o1, o2, dtype, scale=k * 0.3)
+
+
+def test_linear_row_result_does_not_depend_on_batch(ops, gen):
+    """32-bit: a row's product is bit-identical alone and inside a batch."""
+    x, w = rnd((70, 136), torch.float32, gen), rnd((200, 136), torch.float32, gen)
+    full = torch.empty(70, 200, device="cuda")
+    ops.linear(x, w, full)
+    for r in (0, 63, 64, 69):
+        one = torch.empty(1, 200, device="cuda")
+        ops.linear(x[r:r + 1].contiguous(), w, one)
+        assert torch.equal(one[0], full[r])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("t,e,k,h,inner", [(1, 4, 2, 64, 32), (17, 8, 3, 96, 48),
+                                           (150, 60, 4, 128, 80), (3, 6, 6, 72, 40)])
+def test_router_align_experts_combine(ops_mode, gen, dtype, t, e, k, h, inner):
+    """The whole sparse feed-forward chain, kernel by kernel, against the twins;
+    with few rows most experts get none."""
+    ops = ops_mode
+    plain = PlainOps()
+    x = rnd((t, h), dtype, gen)
+    logits = torch.randn(t, e, generator=gen, device="cuda") * 2
+    for renorm in (False, True):
+        ids1 = torch.empty(t, k, device="cuda", dtype=torch.int32)
+        ids2 = torch.empty_like(ids1)
+        w1 = torch.empty(t, k, device="cuda")
+        w2 = torch.empty_like(w1)
+        ops.router_topk(logits, e, k, renorm, ids1, w1)
+        plain.router_topk(logits, e, k, renorm, ids2, w2)
+        assert torch.equal(ids1, ids2)
+        close(w1, w2, torch.float32)
+    off1 = torch.empty(e + 1, device="cuda", dtype=torch.int32)
+    off2 = torch.empty_like(off1)
+    ord1 = torch.empty(t * k, device="cuda", dtype=torch.int32)
+    ord2 = torch.empty_like(ord1)
+    ops.moe_align(ids1, e, off1, ord1)
+    plain.moe_align(ids1, e, off2, ord2)
+    assert torch.equal(off1, off2)
+    # the order inside an expert is free: compare as sets per expert
+    o = off1.tolist()
+    for g in range(e):
+        assert sorted(ord1[o[g]:o[g + 1]].tolist()) == sorted(ord2[o[g]:o[g + 1]].tolist())
+        assert all(int(ids1.reshape(-1)[i]) == g for i in ord1[o[g]:o[g + 1]].tolist())
+    wgu = rnd((e, 2 * inner, h), dtype, gen, 0.3)
+    wd = rnd((e, h, inner), dtype, gen, 0.3)
+    h1 = torch.zeros(t * k, inner, device="cuda", dtype=dtype)
+    h2 = torch.zeros_like(h1)
+    ops.grouped_swiglu(x, wgu, off1, ord1, k, h1)
+    plain.grouped_swiglu(x, wgu, off1, ord1, k, h2)
+    close(h1, h2, dtype, scale=h * 0.3)
+    y1 = torch.zeros(t * k, h, device="cuda", dtype=dtype)
+    y2 = torch.zeros_like(y1)
+    ops.grouped_down(h2, wd, off1, ord1, y1)
+    plain.grouped_down(h2, wd, off1, ord1, y2)
+    close(y1, y2, dtype, scale=h2.float().abs().max().item() * math.sqrt(inner) * 0.3)
+    shared = rnd((t, h), dtype, gen)
+    gate = torch.randn(t, 1, generator=gen, device="cuda")
+    r1 = torch.randn(t, h, generator=gen, device="cuda")
+    r2 = r1.clone()
+    ops.moe_combine(r1, y2, w1, shared, gate)
+    plain.moe_combine(r2, y2, w1, shared, gate)
+    close(r1, r2, torch.float32, scale=y2.float().abs().max().item())
+    r1, r2 = torch.zeros(t, h, device="cuda"), torch.zeros(t, h, device="cuda")
+    ops.moe_combine(r1, y2, w1)
+    plain.moe_combine(r2, y2, w1)
+    close(r1, r2, torch.float32, scale=y2.float().abs().max().item())
+
+
+def test_router_ties_go_to_the_lower_index(ops):
+    logits = torch.zeros(2, 8, device="cuda")
+    logits[1, 5] = 1.0
+    ids = torch.empty(2, 3, device="cuda", dtype=torch.int32)
+    w = torch.empty(2, 3, device="cuda")
+    ops.router_topk(logits, 8, 3, False, ids, w)
+    assert ids.tolist() == [[0, 1, 2], [5, 0, 1]]
+
+
+def _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, n_pages):
+    """seqs: list of (pos0, qlen). Builds shuffled block tables and pools filled
+    with random keys and values for every position < pos0 + qlen."""
+    s = len(seqs)
+    t = sum(q for _, q in seqs)
+    max_pages = max(-(-(p + q) // page_size) for p, q in seqs)
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(5)).tolist()
+    bt = torch.full((s, max_pages), -1, dtype=torch.int32)
+    for i, (p, q) in enumerate(seqs):
+        for lp in range(-(-(p + q) // page_size)):
+            bt[i, lp] = perm.pop()
+    k_pool = rnd((n_pages, n_kv, page_size, d), dtype, gen)
+    v_pool = rnd((n_pages, n_kv, page_size, d), dtype, gen)
+    positions, row_seq, row_start = [], [], []
+    for i, (p, q) in enumerate(seqs):
+        row_start.append(len(positions))
+        positions += list(range(p, p + q))
+        row_seq += [i] * q
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    ctx = SimpleNamespace(S=s, T=t, positions=dev(positions), row_seq=dev(row_seq),
+                          seq_row_start=dev(row_start), seq_qlen=dev([q for _, q in seqs]),
+                          seq_pos0=dev([p for p, _ in seqs]),
+                          max_qlen=max(q for _, q in seqs),
+                          max_kv_len=max(p + q for p, q in seqs))
+    qkv = rnd((t, (n_q + 2 * n_kv) * d), dtype, gen)
+    return ctx, qkv, k_pool, v_pool, bt.cuda()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_q,n_kv,d,page_size,window", [
+    (4, 2, 16, 4, 0), (3, 1, 32, 8, 24), (16, 16, 128, 16, 0), (28, 4, 128, 16, 0),
+    (6, 3, 48, 16, 37), (8, 2, 64, 32, 0), (2, 2, 80, 16, 0)])
+def test_paged_attention(ops_mode, gen, dtype, n_q, n_kv, d, page_size, window):
+    ops = ops_mode
+    seqs = [(0, 1), (0, 37), (130, 1), (61, 5), (17, 70), (255, 1)]
+    ctx, qkv, k_pool, v_pool, bt = _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, 80)
+    o1 = torch.empty(ctx.T, n_q * d, device="cuda", dtype=dtype)
+    o2 = torch.empty_like(o1)
+    scale = 1 / math.sqrt(d)
+    ops.paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, page_size, window, scale, o1)
+    PlainOps().paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, page_size, window,
+                               scale, o2)
+    close(o1, o2, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_finds_a_far_key(ops_mode, gen, dtype):
+    """One key among hundreds is made to dominate: the output must be its
+    value, wherever it lies (a page's first or last slot, far back)."""
+    ops = ops_mode
+    n_q, n_kv, d, ps = 4, 2, 64, 16
+    for far in (0, 15, 16, 255, 300, 511):
+        seqs = [(511, 1), (480, 32)]
+        ctx, qkv, k_pool, v_pool, bt = _attention_case(gen, dtype, seqs, n_q, n_kv, d, ps, 80)
+        page = int(bt[0, far // ps])
+        # every query of request 0 equals 8 * (the far key)
+        k_pool[page, :, far % ps, :] = torch.sign(k_pool[page, :, far % ps, :].float()).to(dtype)
+        for h in range(n_q):
+            qkv[0, h * d:(h + 1) * d] = (8 * k_pool[page, h // 2, far % ps, :].float()).to(dtype)
+        out = torch.empty(ctx.T, n_q * d, device="cuda", dtype=dtype)
+        ops.paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, ps, 0, 1 / math.sqrt(d),
+                            out)
+        for h in range(n_q):
+            torch.testing.assert_close(out[0, h * d:(h + 1) * d].float(),
+                                       v_pool[page, h // 2, far % ps, :].float(),
+                                       atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_q,n_kv,d,rot", [(4, 2, 16, 16), (3, 1, 32, 32), (16, 16, 128, 128),
+                                            (5, 5, 48, 24), (2, 1, 64, 0)])
+def test_rope_kv_write(ops, gen, dtype, n_q, n_kv, d, rot):
+    from ninfer_amd.parts.rotary import Rotary
+    ps = 8
+    seqs = [(0, 9), (1000, 1), (30, 3)]
+    ctx, qkv, k_pool, v_pool, bt = _attention_case(gen, dtype, seqs, n_q, n_kv, d, ps, 200)
+    table = Rotary(rot, 1e4).inv_freq().cuda() if rot else None
+    bias = torch.randn(qkv.shape[1], generator=gen, device="cuda")
+    for b in (None, bias):
+        for write in (True, False):
+            q1, q2 = qkv.clone(), qkv.clone()
+            k1, k2, v1, v2 = k_pool.clone(), k_pool.clone(), v_pool.clone(), v_pool.clone()
+            ops.rope_kv_write(q1, b, ctx.positions, ctx.row_seq, table, rot, n_q, n_kv, d, k1, v1,
+                              bt, ps, write_kv=write)
+            PlainOps().rope_kv_write(q2, b, ctx.positions, ctx.row_seq, table, rot, n_q, n_kv, d,
+                                     k2, v2, bt, ps, write_kv=write)
+            close(q1[:, :n_q * d], q2[:, :n_q * d], dtype, scale=4)
+            close(k1, k2, dtype, scale=4)
+            close(v1, v2, dtype, scale=4)
+            if not write:
+                assert torch.equal(k1, k_pool) and torch.equal(v1, v_pool)
+
+
+def test_sample_greedy_and_distribution(ops, gen):
+    import plain_model
+    v = 1000
+    logits = torch.randn(6, v, generator=gen, device="cuda") * 3
+    logits[0, 17] = 50.0
+    logits[1, 400] = logits[1, 3] = 60.0  # a tie: the lower id wins
+    temp = torch.tensor([0.0, 0.0, 0.7, 1.0, 1.3, 0.7], device="cuda")
+    top_k = torch.tensor([0, 0, 0, 50, 7, 1], device="cuda", dtype=torch.int32)
+    top_p = torch.tensor([1.0, 1.0, 1.0, 0.9, 0.5, 1.0], device="cuda")
+    rp = torch.tensor([1.0, 1.0, 1.0, 1.3, 1.0, 1.0], device="cuda")
+    pen_tokens = torch.tensor([5, 9], device="cuda", dtype=torch.int32)
+    pen_counts = torch.tensor([1, 2], device="cuda", dtype=torch.int32)
+    pen_offsets = torch.tensor([0, 0, 0, 0, 2, 2, 2], device="cuda", dtype=torch.int32)
+    out = torch.empty(6, device="cuda", dtype=torch.int32)
+    draws = {i: [] for i in range(6)}
+    us = torch.linspace(0.0005, 0.9995, 400)
+    for u in us.tolist():
+        uniform = torch.full((6,), u, device="cuda")
+        ops.sample(logits, temp, uniform, out, top_k=top_k, top_p=top_p, rep_penalty=rp,
+                   pen_tokens=pen_tokens, pen_counts=pen_counts, pen_offsets=pen_offsets)
+        for i, tkn in enumerate(out.tolist()):
+            draws[i].append(tkn)
+    assert set(draws[0]) == {17} and set(draws[1]) == {3}
+    assert set(draws[5]) == {int(torch.argmax(logits[5]))}, "top_k = 1 is greedy"
+    for i in (2, 3, 4):
+        recent = [5, 9, 9] if i == 3 else []
+        p = plain_model.sample_distribution(logits[i].cpu(), float(temp[i]), int(top_k[i]),
+                                            float(top_p[i]), float(rp[i]), recent)
+        support = set(torch.nonzero(p).flatten().tolist())
+        assert set(draws[i]) <= support
+        # a grid of u's samples the inverse CDF: frequencies follow p
+        freq = torch.bincount(torch.tensor(draws[i]), minlength=v).float() / len(us)
+        assert (freq - p).abs().max() < 3.0 / len(us) + 1e-3
