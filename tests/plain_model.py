@@ -203,11 +203,14 @@ def layer_window(cfg: dict, layer: int) -> Optional[int]:
     return None
 
 
-def feed_forward(x: Tensor, w: Dict[str, Tensor], cfg: dict, layer: int) -> Tensor:
+def feed_forward(x: Tensor, w: Dict[str, Tensor], cfg: dict, layer: int,
+                 probe: Optional[dict] = None) -> Tensor:
     p = f"model.layers.{layer}.mlp."
     if not layer_is_sparse(cfg, layer):
         return swiglu_mlp(x, w[p + "gate_proj.weight"], w[p + "up_proj.weight"],
                           w[p + "down_proj.weight"])
+    if probe is not None:
+        probe.setdefault("router_logits", {})[layer] = x @ w[p + "gate.weight"].float().T
     ids, wts = router(x, w[p + "gate.weight"], cfg["num_experts_per_tok"],
                       cfg.get("norm_topk_prob", False))
     return routed_experts(x, ids, wts, w, p) + shared_expert(x, w, p)
@@ -218,7 +221,7 @@ def feed_forward(x: Tensor, w: Dict[str, Tensor], cfg: dict, layer: int) -> Tens
 # --------------------------------------------------------------------------
 def forward(w: Dict[str, Tensor], cfg: dict, tokens: Sequence[int],
             plan: Optional[List[Tuple[int, Optional[int]]]] = None,
-            first_position: int = 0) -> Tensor:
+            first_position: int = 0, probe: Optional[dict] = None) -> Tensor:
     """Logits [T, V] of one whole sequence.
 
     Layer order (pre-norm residual decoder): reference src/models/model.hip:
@@ -227,6 +230,7 @@ def forward(w: Dict[str, Tensor], cfg: dict, tokens: Sequence[int],
     call computes its own keys and values; an integer names an earlier entry of
     the plan whose keys and values it reads instead. Default: each layer once.
     `first_position` shifts all positions (only distances may matter).
+    `probe`, if given, receives the router logits of every sparse layer.
     """
     tok = torch.tensor(list(tokens), dtype=torch.long)
     t = tok.shape[0]
@@ -250,7 +254,7 @@ def forward(w: Dict[str, Tensor], cfg: dict, tokens: Sequence[int],
         o = attention_core(q, k, v, pos, pos, layer_window(cfg, layer))
         x = x + o.reshape(t, hq * d) @ w[lp + "self_attn.o_proj.weight"].float().T
         m = rms_norm(x, w[lp + "post_attention_layernorm.weight"], eps)
-        x = x + feed_forward(m, w, cfg, layer)
+        x = x + feed_forward(m, w, cfg, layer, probe)
     n = rms_norm(x, w["model.norm.weight"], eps)
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) \
         else w["lm_head.weight"]

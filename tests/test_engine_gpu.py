@@ -25,10 +25,14 @@ def case(request, model_dirs):
     name = request.param
     cfg = TINY[name][0]
     out = {"name": name, "cfg": cfg, "dirs": model_dirs[name], "ref": {}, "reqs": {}}
+    rcfg, w16 = util.read_folder(model_dirs[name]["bfloat16"])
     for i, n in enumerate(PROMPTS[name]):
-        out["reqs"][f"r{i}"] = util.random_tokens(n + 12, cfg["vocab_size"], 100 + i)
+        # routing must be clear in both weight sets (they differ by rounding only)
+        out["reqs"][f"r{i}"] = util.safe_prompt(w16, rcfg, n + 12, 100 + i)
     for dtype, d in model_dirs[name].items():
         rcfg, w = util.read_folder(d)
+        for v in out["reqs"].values():
+            assert util.routing_margins(w, rcfg, v).min() > 0.03
         out["ref"][dtype] = {k: plain_model.forward(w, rcfg, v) for k, v in out["reqs"].items()}
     return out
 

@@ -192,6 +192,7 @@ def _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, n_pages):
     s = len(seqs)
     t = sum(q for _, q in seqs)
     max_pages = max(-(-(p + q) // page_size) for p, q in seqs)
+    n_pages = max(n_pages, sum(-(-(p + q) // page_size) for p, q in seqs) + 3)
     perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(5)).tolist()
     bt = torch.full((s, max_pages), -1, dtype=torch.int32)
     for i, (p, q) in enumerate(seqs):

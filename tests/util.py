@@ -29,6 +29,39 @@ def random_tokens(n: int, vocab: int, seed: int) -> List[int]:
     return [rng.randrange(vocab) for _ in range(n)]
 
 
+def routing_margins(w, cfg, tokens) -> torch.Tensor:
+    """Per row, the smallest gap between the k-th and (k+1)-th router logit over
+    the sparse layers, relative to the largest |logit| of that row and layer."""
+    import plain_model
+    probe: dict = {}
+    plain_model.forward(w, cfg, tokens, probe=probe)
+    k = cfg["num_experts_per_tok"]
+    worst = torch.full((len(tokens),), float("inf"))
+    for logits in probe.get("router_logits", {}).values():
+        if logits.shape[1] <= k:
+            continue
+        top = torch.sort(logits, dim=-1, descending=True).values
+        gap = (top[:, k - 1] - top[:, k]) / logits.abs().max(dim=-1).values
+        worst = torch.minimum(worst, gap)
+    return worst
+
+
+def safe_prompt(w, cfg, n: int, seed: int, rel_margin: float = 0.06) -> List[int]:
+    """Seeded random token ids, redrawn where the plain model's routing would
+    be nearly tied: top-k routing is discontinuous, so a row whose k-th and
+    (k+1)-th experts are within rounding noise of each other may legitimately
+    pick either in reduced precision, and no bound on logits could hold there.
+    A row's routing depends only on its prefix, so rows are fixed left to right."""
+    rng = random.Random(seed)
+    toks = [rng.randrange(cfg["vocab_size"]) for _ in range(n)]
+    for _ in range(20 * n):
+        bad = torch.nonzero(routing_margins(w, cfg, toks) < rel_margin).flatten()
+        if bad.numel() == 0:
+            return toks
+        toks[int(bad[0])] = rng.randrange(cfg["vocab_size"])
+    raise RuntimeError("no prompt with clear routing found")
+
+
 # A schedule is a list of steps; a step is (entries, end) with entries
 # [(request id, tokens, want rows)] and end = ids finished after the step.
 Step = Tuple[List[Tuple[str, List[int], List[int]]], List[str]]
