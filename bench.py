@@ -1,0 +1,170 @@
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+The default run has the layer sizes of Qwen1.5-MoE-A2.7B (24 layers, hidden
+2048, 16 heads of 128, 60 experts top-4 of 1408, shared expert 5632, vocabulary
+151936) with random bf16 weights generated on the device, a batch of 8
+requests and a context of 8192 tokens each (the cache is filled with random
+keys and values; token ids are seeded random). A step is one decode step: one
+new token for every request of the batch through the engine's step function
+and its device sampler. One JSON line is printed: decoded tokens a second as
+`value`; the 2,048-token prefill under "prefill"; the decode step's memory
+roofline under "roofline"; decode at batch 1 and 64 under "points".
+Peaks: HBM 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s (fp32 157.3 TFLOP/s).
+"""
+import argparse
+import json
+import sys
+import time
+
+HBM_PEAK = 8.0e12
+FLOP_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+CONFIG_C = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe",
+    "num_hidden_layers": 24, "hidden_size": 2048, "num_attention_heads": 16,
+    "num_key_value_heads": 16, "head_dim": 128, "intermediate_size": 5632,
+    "moe_intermediate_size": 1408, "shared_expert_intermediate_size": 5632,
+    "num_experts": 60, "num_experts_per_tok": 4, "norm_topk_prob": False,
+    "decoder_sparse_step": 1, "mlp_only_layers": [], "vocab_size": 151936,
+    "rope_theta": 1000000.0, "use_sliding_window": False, "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False, "hidden_act": "silu",
+}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=8192)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--graph", action="store_true", help="decode through a captured HIP graph")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    import ninfer_amd
+    from ninfer_amd import Chunk, EngineOptions, random_model
+    from ninfer_amd.parts.moe import SparseMoE
+    from ninfer_amd.sampling import SampleRow, Sampler, SamplingParams
+    from collections import Counter
+
+    raw = dict(CONFIG_C)
+    layers_full = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    L = raw["num_hidden_layers"]
+    H, Hq, Hkv, D = raw["hidden_size"], raw["num_attention_heads"], raw["num_key_value_heads"], \
+        raw["head_dim"]
+    Im, Is, E, k, V = raw["moe_intermediate_size"], raw["shared_expert_intermediate_size"], \
+        raw["num_experts"], raw["num_experts_per_tok"], raw["vocab_size"]
+    esize = 2 if args.dtype == "bfloat16" else 4
+    page = 16
+    max_b = args.batch if args.no_points else max(args.batch, 64)
+    ctx = args.context
+    opt = EngineOptions(dtype=args.dtype, max_context=ctx, prefill_chunk=max(2048, max_b),
+                        num_sequences=max_b, page_size=page, use_graph=args.graph)
+    t0 = time.time()
+    runner = random_model(raw, 1234, opt)
+    torch.cuda.synchronize()
+    print(f"[bench] model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    for kp, vp in runner.cache.pools.values():   # a cache full of synthetic keys and values
+        kp.normal_()
+        vp.normal_()
+    sampler = Sampler(runner.ops, runner.device)
+    gen = torch.Generator().manual_seed(7)
+    greedy = SamplingParams.greedy()
+    moes = [b.feed_forward for b in runner.spec.blocks if isinstance(b.feed_forward, SparseMoE)]
+
+    def decode_run(batch: int, steps: int, warmup: int):
+        start = ctx - (steps + warmup) - 1
+        slots = [runner.open() for _ in range(batch)]
+        for s in slots:                       # positions 0..start-1 count as cached
+            runner.cache.reserve(s, start)
+            runner.cache.commit(s, start)
+        toks = torch.randint(0, V, (batch,), generator=gen).tolist()
+        rows = [SampleRow(greedy, Counter(), i, 0, 1) for i in range(batch)]
+
+        def one():
+            nonlocal toks
+            logits = runner.step([Chunk(s, [t], [0]) for s, t in zip(slots, toks)])
+            toks = sampler.sample(logits, rows)
+
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t) / steps
+        distinct = [int(torch.unique(m.last_ids).numel()) for m in moes if m.last_ids is not None]
+        for s in slots:
+            runner.close(s)
+        n_exp = sum(distinct) / max(len(distinct), 1)
+        per_layer = ((Hq + 2 * Hkv) * D * H + H * Hq * D + E * H + n_exp * 3 * Im * H
+                     + 3 * Is * H + H) * esize
+        kv = batch * 2 * L * Hkv * D * (ctx - steps / 2) * esize
+        nbytes = L * per_layer + V * H * esize + kv
+        return dt, nbytes, n_exp
+
+    def prefill_run(T: int, reps: int):
+        toks = torch.randint(0, V, (T,), generator=gen).tolist()
+        times = []
+        for _ in range(reps + 1):
+            s = runner.open()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            runner.step([Chunk(s, toks, [T - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            runner.close(s)
+        dt = sorted(times[1:])[len(times[1:]) // 2]
+        flops = T * 2 * L * ((Hq + 2 * Hkv) * D * H + Hq * D * H + E * H + k * 3 * Im * H
+                             + 3 * Is * H + H) + L * 2 * Hq * D * T * T + 2 * V * H
+        return dt, flops
+
+    dt, nbytes, n_exp = decode_run(args.batch, args.steps, args.warmup)
+    result = {
+        "metric": "decode tok/s at batch 8 (Qwen1.5-MoE-A2.7B shapes, context 8192)",
+        "value": round(args.batch / dt, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {"model": "Qwen1.5-MoE-A2.7B shapes, random weights", "global_batch": args.batch,
+                   "seq_len": ctx, "parallelism": "single GPU", "layers": L,
+                   "layers_full": layers_full, "hidden": H, "heads": Hq, "kv_heads": Hkv,
+                   "head_dim": D, "moe_intermediate": Im, "shared_intermediate": Is,
+                   "intermediate": raw["intermediate_size"], "experts": E, "top_k": k, "vocab": V,
+                   "page_size": page, "graph": bool(args.graph)},
+        "roofline": {"bound": "hbm", "achieved": round(nbytes / dt / 1e9, 1),
+                     "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(nbytes / dt / HBM_PEAK, 4),
+                     "distinct_experts_per_layer": round(n_exp, 1)},
+    }
+    if not args.no_prefill:
+        pdt, flops = prefill_run(2048, 3)
+        result["prefill"] = {"value": round(2048 / pdt, 1), "tokens": 2048,
+                             "ms": round(pdt * 1e3, 3),
+                             "frac": round(flops / pdt / FLOP_PEAK[args.dtype], 4)}
+    if not args.no_points:
+        points = {}
+        for b in (1, 64):
+            steps = max(8, args.steps // (4 if b == 64 else 1))
+            d, _, _ = decode_run(b, steps, max(2, args.warmup // 2))
+            points[f"decode_b{b}"] = round(b / d, 2)
+        result["points"] = points
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,102 @@
+"""Command line in the reference's manner: `ninfer <model_dir> [options]`
+(src/apps/ninfer.cpp:55-119). Option names and meanings are the reference's
+where it has them: --max-context, --prefill-chunk, --max-new, --temperature
+(0 = greedy), --top-k, --top-p, --repeat-penalty, --seed (0 = not fixed),
+--graph, --log-level. Prompts are token ids (there is no tokenizer here):
+--prompt-ids, --prompt-file, --random-prompts. Generated ids go to stdout, one
+line per request; diagnostics go to stderr (src/apps/ninfer.cpp:1-2). An
+unknown option is an error (:114-116).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import random
+import sys
+import time
+from typing import List, Optional
+
+
+def build_parser() -> argparse.ArgumentParser:
+    ap = argparse.ArgumentParser(prog="ninfer", description="Qwen2-MoE generation on one MI355X")
+    ap.add_argument("model_dir", help="folder with config.json (and model.safetensors)")
+    ap.add_argument("--prompt-ids", action="append", default=[],
+                    help="a prompt as comma-separated token ids (may be given several times)")
+    ap.add_argument("--prompt-file", help="JSON file: a list of lists of token ids")
+    ap.add_argument("--random-prompts", help="comma-separated lengths of seeded random prompts")
+    ap.add_argument("--max-context", type=int, default=32768, help="KV capacity in tokens per request")
+    ap.add_argument("--prefill-chunk", type=int, default=512, help="token budget of one step")
+    ap.add_argument("--max-new", type=int, default=512, help="new tokens per generation")
+    ap.add_argument("--temperature", type=float, default=0.7, help="sampling temperature (0 = greedy)")
+    ap.add_argument("--top-k", type=int, default=50)
+    ap.add_argument("--top-p", type=float, default=0.95)
+    ap.add_argument("--repeat-penalty", type=float, default=1.05)
+    ap.add_argument("--seed", type=int, default=0, help="sampling seed (0 = not fixed)")
+    ap.add_argument("--graph", action="store_true", help="replay decode steps from a HIP graph")
+    ap.add_argument("--log-level", choices=["debug", "info", "warn", "error"], default="info")
+    ap.add_argument("--dtype", choices=["bf16", "fp32", "bfloat16", "float32"], default="bf16")
+    ap.add_argument("--random-weights", type=int, metavar="SEED",
+                    help="fill the model with seeded random weights (needs only config.json)")
+    ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--kv-pages", type=int, help="pages per cache group")
+    ap.add_argument("--max-seqs", type=int, default=8, help="most live requests")
+    ap.add_argument("--eos-id", type=int, help="stop token (default: config.json eos_token_id)")
+    return ap
+
+
+def main(argv: Optional[List[str]] = None) -> int:
+    args = build_parser().parse_args(argv)
+    quiet = args.log_level in ("warn", "error")
+
+    def log(msg: str) -> None:
+        if not quiet:
+            print(f"[ninfer] {msg}", file=sys.stderr, flush=True)
+
+    from .api.ninfer import Ninfer
+    from .config.base import read_config_json
+    from .sampling.params import SamplingParams
+
+    dtype = {"bf16": "bfloat16", "fp32": "float32"}.get(args.dtype, args.dtype)
+    raw = read_config_json(args.model_dir)
+    prompts: List[List[int]] = [[int(x) for x in p.split(",") if x.strip()]
+                                for p in args.prompt_ids]
+    if args.prompt_file:
+        with open(args.prompt_file) as f:
+            prompts += [list(map(int, p)) for p in json.load(f)]
+    if args.random_prompts:
+        rng = random.Random(args.seed or 1234)
+        for n in args.random_prompts.split(","):
+            prompts.append([rng.randrange(raw["vocab_size"]) for _ in range(int(n))])
+    if not prompts:
+        print("ninfer: no prompt given (--prompt-ids, --prompt-file or --random-prompts)",
+              file=sys.stderr)
+        return 2
+    t0 = time.time()
+    common = dict(max_context=args.max_context, prefill_chunk=args.prefill_chunk,
+                  num_sequences=args.max_seqs, dtype=dtype, page_size=args.page_size,
+                  num_pages=args.kv_pages, use_graph=args.graph)
+    try:
+        if args.random_weights is not None:
+            eng = Ninfer(random_config=raw, random_seed=args.random_weights, **common)
+        else:
+            eng = Ninfer(args.model_dir, **common)
+        log(f"engine ready in {time.time() - t0:.1f} s: vocab={eng.vocab} ctx={args.max_context} "
+            f"chunk={args.prefill_chunk} seqs={args.max_seqs} dtype={dtype}")
+        params = SamplingParams(args.temperature, args.top_k, args.top_p, args.repeat_penalty,
+                                args.seed, args.max_new)
+        stop = [args.eos_id] if args.eos_id is not None else None
+        t1 = time.time()
+        outs = eng.generate(prompts, params, stop)
+        dt = time.time() - t1
+        for o in outs:
+            print(",".join(map(str, o)))
+        n = sum(len(o) for o in outs)
+        log(f"{n} tokens in {dt:.2f} s ({n / max(dt, 1e-9):.1f} tok/s)")
+    except Exception as e:  # the reference exits 1 with the message (src/apps/ninfer.cpp:234-237)
+        print(f"ninfer: error: {e}", file=sys.stderr)
+        return 1
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

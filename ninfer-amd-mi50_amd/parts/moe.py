@@ -105,6 +105,7 @@ class SparseMoE(FeedForward):
         self.experts = RoutedExperts(prefix + "experts.", hidden, inner, experts)
         self.shared: Optional[SwiGLU] = None
         self.shared_gate: Optional[torch.Tensor] = None
+        self.last_ids: Optional[torch.Tensor] = None   # routing of the last step (for statistics)
         if shared_inner > 0:
             self.shared = SwiGLU(prefix + "shared_expert.", hidden, shared_inner)
 
@@ -122,6 +123,7 @@ class SparseMoE(FeedForward):
 
     def forward(self, ctx: StepContext, x, residual):
         ids, wts = self.router.route(ctx, x)
+        self.last_ids = ids
         y = self.experts.run(ctx, x, ids)
         shared = gate = None
         if self.shared is not None:

@@ -1,0 +1,165 @@
+"""The scheduler's decisions, on the CPU: the engine's host logic runs with the
+plain twins of the kernels (tests/plain_ops.py) in place of the HIP library."""
+import random
+
+import pytest
+import torch
+
+import plain_model
+import util
+from conftest import TINY
+from plain_ops import PlainOps
+
+
+@pytest.fixture(scope="module")
+def setup(model_dirs):
+    cfg, w = util.read_folder(model_dirs["A"]["float32"])
+    return model_dirs["A"]["float32"], cfg, w
+
+
+def make(setup, num_pages, page_size=4, chunk=16, seqs=4, max_context=96):
+    from ninfer_amd import EngineOptions, Sampler, Scheduler, load_model
+    opt = EngineOptions(dtype="float32", max_context=max_context, prefill_chunk=chunk,
+                        num_sequences=seqs, page_size=page_size, num_pages=num_pages, device="cpu")
+    runner = load_model(setup[0], opt, ops=PlainOps())
+    return runner, Scheduler(runner, Sampler(PlainOps(), runner.device))
+
+
+class Spy:
+    """Wraps a runner's step to record the shape of every batch."""
+
+    def __init__(self, runner):
+        self.runner, self.batches = runner, []
+        self._step = runner.step
+        runner.step = self.step
+
+    def step(self, chunks):
+        self.batches.append([(c.slot, len(c.tokens), list(c.want)) for c in chunks])
+        return self._step(chunks)
+
+
+def requests(cfg, lens, max_new, **kw):
+    from ninfer_amd import Request, SamplingParams
+    params = SamplingParams(max_new_tokens=max_new, **kw)
+    return [Request(f"q{i}", util.random_tokens(n, cfg["vocab_size"], 50 + i), params)
+            for i, n in enumerate(lens)]
+
+
+def test_greedy_matches_plain_and_budgets_hold(setup):
+    _, cfg, w = setup
+    runner, sched = make(setup, num_pages=200)
+    spy = Spy(runner)
+    reqs = requests(cfg, [5, 11, 17, 30, 3, 23], 8, temperature=0.0, top_k=0, top_p=1.0,
+                    repetition_penalty=1.0)
+    for r in reqs:
+        sched.add(r)
+    sched.run()
+    for r in reqs:
+        assert r.status == "finished" and len(r.output) == 8
+        assert r.output == plain_model.greedy_generate(w, cfg, r.prompt, 8)
+    for b in spy.batches:
+        assert sum(n for _, n, _ in b) <= 16 and len(b) <= 4
+        assert len({s for s, _, _ in b}) == len(b)
+    # prompts longer than the budget were cut; some steps mix portions and decode tokens
+    assert any(len(b) > 1 and any(n > 1 for _, n, _ in b) and any(n == 1 for _, n, _ in b)
+               for b in spy.batches)
+    runner.cache.check()
+    assert all(g.allocator.in_use == 0 for g in runner.cache.groups)
+    assert runner.cache.free_slots == 4
+
+
+def test_preemption_gives_the_same_tokens(setup):
+    _, cfg, w = setup
+    lens = [20, 18, 22, 16]
+    runner, sched = make(setup, num_pages=200)
+    ref = requests(cfg, lens, 12, temperature=0.8, top_k=20, top_p=0.9, seed=77)
+    for r in ref:
+        sched.add(r)
+    sched.run()
+    # 22 pages of 4 tokens cannot hold four requests of ~30 tokens: some are preempted
+    runner2, sched2 = make(setup, num_pages=22)
+    again = requests(cfg, lens, 12, temperature=0.8, top_k=20, top_p=0.9, seed=77)
+    for r in again:
+        sched2.add(r)
+    sched2.run()
+    assert sched2.preemptions > 0
+    for a, b in zip(ref, again):
+        assert b.status == "finished" and a.output == b.output
+    runner2.cache.check()
+    assert all(g.allocator.in_use == 0 for g in runner2.cache.groups)
+
+
+def test_request_that_cannot_fit_fails_alone(setup):
+    _, cfg, _ = setup
+    runner, sched = make(setup, num_pages=6)       # 24 tokens of cache
+    big, small = requests(cfg, [40, 6], 4, temperature=0.0)
+    sched.add(big)
+    sched.add(small)
+    sched.run()
+    assert big.status == "failed" and "fit" in big.error
+    assert small.status == "finished" and len(small.output) == 4
+    assert all(g.allocator.in_use == 0 for g in runner.cache.groups)
+    # a request that grows beyond the pool while decoding, alone, fails too
+    runner, sched = make(setup, num_pages=6)
+    (grow,) = requests(cfg, [20], 30, temperature=0.0)
+    sched.add(grow)
+    sched.run()
+    assert grow.status == "failed" and len(grow.output) > 0
+    assert all(g.allocator.in_use == 0 for g in runner.cache.groups)
+
+
+def test_reference_rule_prompt_plus_new_tokens(setup):
+    _, cfg, _ = setup
+    runner, sched = make(setup, num_pages=200, max_context=32)
+    (r,) = requests(cfg, [30], 8, temperature=0.0)
+    sched.add(r)
+    assert r.status == "failed" and "max_context" in r.error
+
+
+def test_stop_token_ends_a_request(setup):
+    _, cfg, w = setup
+    runner, sched = make(setup, num_pages=200)
+    (r,) = requests(cfg, [9], 10, temperature=0.0)
+    full = plain_model.greedy_generate(w, cfg, r.prompt, 10)
+    r.stop_ids = [full[4]]
+    sched.add(r)
+    sched.run()
+    assert r.status == "finished" and r.output == full[:full.index(full[4])]
+
+
+def test_seeded_sampling_does_not_depend_on_the_crowd(setup):
+    _, cfg, _ = setup
+    lens = [7, 13, 9]
+    outs = []
+    for crowd in (False, True):
+        runner, sched = make(setup, num_pages=200)
+        reqs = requests(cfg, lens if crowd else lens[:1], 10, temperature=1.0, top_k=0, top_p=1.0,
+                        repetition_penalty=1.0, seed=5)
+        for r in reqs:
+            sched.add(r)
+        sched.run()
+        outs.append(reqs[0].output)
+    assert outs[0] == outs[1]
+    # and another seed gives another continuation
+    runner, sched = make(setup, num_pages=200)
+    (r,) = requests(cfg, lens[:1], 10, temperature=1.0, top_k=0, top_p=1.0,
+                    repetition_penalty=1.0, seed=6)
+    sched.add(r)
+    sched.run()
+    assert r.output != outs[0]
+
+
+def test_random_arrivals_never_leak(setup):
+    _, cfg, _ = setup
+    rng = random.Random(3)
+    runner, sched = make(setup, num_pages=40, chunk=12, seqs=3)
+    pending = requests(cfg, [rng.randrange(2, 30) for _ in range(14)], 5, temperature=0.0)
+    done = 0
+    while pending or sched.has_work():
+        while pending and rng.random() < 0.4:
+            sched.add(pending.pop())
+        if sched.has_work():
+            done += len(sched.step())
+            runner.cache.check()
+    assert done == 14 and all(r.status == "finished" for r in sched.finished)
+    assert all(g.allocator.in_use == 0 for g in runner.cache.groups)
