@@ -38,4 +38,8 @@ int attention_generic(const void* q, int q_stride, const void* kpool, const void
                       const int* row_seq, void* out, int T, int Hq, int Hkv, int D, int page_size,
                       int window, float scale, int dtype, hipStream_t stream);
 
+int64_t attention_decode_workspace_floats(int T, int Hq, int D, int max_kv_len);
+bool attention_decode_takes(const AttnArgs& a);
+int attention_decode(const AttnArgs& a, hipStream_t stream);
+
 }  // namespace ninfer

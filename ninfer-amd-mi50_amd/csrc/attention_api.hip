@@ -18,8 +18,15 @@ extern "C" int ninfer_paged_attention(const AttnArgs* a, int force_generic, hipS
                  a->dtype);
   NINFER_REQUIRE(a->q_stride >= a->Hq * a->D, "paged_attention: row stride %d < %d", a->q_stride,
                  a->Hq * a->D);
-  (void)force_generic;
+  NINFER_REQUIRE(a->max_qlen >= 1 && a->max_kv_len >= 1, "paged_attention: bad size hints");
+  if (!force_generic && a->max_qlen == 1 && attention_decode_takes(*a))
+    return attention_decode(*a, stream);
   return attention_generic(a->q, a->q_stride, a->kpool, a->vpool, a->block_table, a->bt_stride,
                            a->positions, a->row_seq, a->out, a->T, a->Hq, a->Hkv, a->D,
                            a->page_size, a->window, a->scale, a->dtype, stream);
+}
+
+// 32-bit floats of workspace the split-KV decode kernel needs for this shape.
+extern "C" long long ninfer_attention_workspace_floats(int T, int Hq, int D, int max_kv_len) {
+  return attention_decode_workspace_floats(T, Hq, D, max_kv_len);
 }

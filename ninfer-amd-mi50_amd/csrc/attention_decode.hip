@@ -1,0 +1,241 @@
+// Paged attention for decode rows (bf16): the context of every row is split
+// into chunks of keys that different blocks walk at the same time
+// (flash-decoding), then a second kernel merges the chunks. The reference
+// walks the whole context in one block per head with a serial softmax tail
+// (src/ops/attention.hip:14-94); at long context and small batch that leaves
+// most of the GPU idle.
+//
+// Pass 1, grid (chunks, kv heads x head groups, rows), 4 waves per block. A
+// key row of D = 8 LPK elements is read by LPK adjacent lanes, 16 bytes each,
+// so one wave instruction fetches 64 / LPK whole keys, contiguous in the page.
+// The dot product is reduced over those LPK lanes; each lane group keeps its
+// own online softmax (m, l, acc) over the keys it sees, for up to GQ query
+// heads that share the kv head, so keys and values are read once for all of
+// them. Lane groups, then waves, are merged by the usual log-sum-exp rule and
+// the chunk's (m, l, acc) goes to the workspace.
+// Pass 2, grid (rows, query heads): merges the chunks of a row in chunk order.
+//
+// Scores, softmax and sums are 32-bit. A row sees keys lo..pos with
+// lo = max(0, pos - window + 1); chunks are aligned to absolute positions.
+#include "attention.h"
+
+namespace ninfer {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kChunk = 256;      // keys per block
+constexpr int kDecWaves = 4;
+
+__device__ __forceinline__ void cvt8(const bf16x8& v, float* f) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
+}
+
+template <int LPK, int GQ>
+__global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a, int head_groups) {
+  constexpr int D = 8 * LPK;
+  constexpr int KPI = 64 / LPK;             // keys per wave instruction
+  constexpr int KEYS_PER_WAVE = kChunk / kDecWaves;
+  constexpr int ITERS = KEYS_PER_WAVE / KPI;
+  constexpr int UNROLL = ITERS >= 4 ? 4 : ITERS;
+  __shared__ float merge[kDecWaves][GQ][D + 2];
+
+  const int t = blockIdx.z;
+  const int g = blockIdx.y / head_groups;            // kv head
+  const int hg = blockIdx.y % head_groups;           // which GQ-group of its query heads
+  const int group = a.Hq / a.Hkv;
+  const int h0 = g * group + hg * GQ;                // first query head of this block
+  const int n_heads = min(GQ, group - hg * GQ);
+  const int pos = a.positions[t];
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int c0 = blockIdx.x * kChunk;
+  if (c0 > pos || c0 + kChunk <= lo) return;          // chunk outside the row's keys
+  const int n_chunks = gridDim.x;
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane % LPK, kslot = lane / LPK;
+  const int* bt = a.block_table + (int64_t)a.row_seq[t] * a.bt_stride;
+  const bf16* kpool = (const bf16*)a.kpool;
+  const bf16* vpool = (const bf16*)a.vpool;
+  const int ps = a.page_size, Hkv = a.Hkv;
+
+  float q[GQ][8];
+#pragma unroll
+  for (int i = 0; i < GQ; ++i) {
+    if (i < n_heads) {
+      bf16x8 v = *(const bf16x8*)((const bf16*)a.q + (int64_t)t * a.q_stride + (h0 + i) * D + 8 * sub);
+      cvt8(v, q[i]);
+#pragma unroll
+      for (int d = 0; d < 8; ++d) q[i][d] *= a.scale;
+    } else {
+#pragma unroll
+      for (int d = 0; d < 8; ++d) q[i][d] = 0.f;
+    }
+  }
+  float m[GQ], l[GQ], acc[GQ][8];
+#pragma unroll
+  for (int i = 0; i < GQ; ++i) {
+    m[i] = -1e30f;
+    l[i] = 0.f;
+#pragma unroll
+    for (int d = 0; d < 8; ++d) acc[i][d] = 0.f;
+  }
+
+  const int wbase = c0 + wave * KEYS_PER_WAVE;
+  for (int it0 = 0; it0 < ITERS; it0 += UNROLL) {
+    bf16x8 kf[UNROLL], vf[UNROLL];
+    bool ok[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      int j = wbase + (it0 + u) * KPI + kslot;
+      ok[u] = j >= lo && j <= pos;
+      if (ok[u]) {
+        int page = bt[j / ps];
+        int64_t off = (((int64_t)page * Hkv + g) * ps + (j % ps)) * D + 8 * sub;
+        kf[u] = *(const bf16x8*)(kpool + off);
+        vf[u] = *(const bf16x8*)(vpool + off);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      float kk[8], vv[8];
+      if (ok[u]) {
+        cvt8(kf[u], kk);
+        cvt8(vf[u], vv);
+      } else {
+#pragma unroll
+        for (int d = 0; d < 8; ++d) kk[d] = vv[d] = 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < GQ; ++i) {
+        float s = 0.f;
+#pragma unroll
+        for (int d = 0; d < 8; ++d) s = fmaf(q[i][d], kk[d], s);
+#pragma unroll
+        for (int off = LPK / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+        if (ok[u]) {
+          float m_new = fmaxf(m[i], s);
+          float alpha = __expf(m[i] - m_new);
+          float p = __expf(s - m_new);
+          l[i] = l[i] * alpha + p;
+#pragma unroll
+          for (int d = 0; d < 8; ++d) acc[i][d] = fmaf(p, vv[d], acc[i][d] * alpha);
+          m[i] = m_new;
+        }
+      }
+    }
+  }
+
+  // merge the KPI lane groups of the wave
+#pragma unroll
+  for (int i = 0; i < GQ; ++i) {
+#pragma unroll
+    for (int off = LPK; off < 64; off <<= 1) {
+      float om = __shfl_xor(m[i], off, 64);
+      float ol = __shfl_xor(l[i], off, 64);
+      float m_new = fmaxf(m[i], om);
+      float sa = __expf(m[i] - m_new), sb = __expf(om - m_new);
+      l[i] = l[i] * sa + ol * sb;
+#pragma unroll
+      for (int d = 0; d < 8; ++d) {
+        float oa = __shfl_xor(acc[i][d], off, 64);
+        acc[i][d] = acc[i][d] * sa + oa * sb;
+      }
+      m[i] = m_new;
+    }
+    if (kslot == 0) {
+#pragma unroll
+      for (int d = 0; d < 8; ++d) merge[wave][i][8 * sub + d] = acc[i][d];
+      if (sub == 0) {
+        merge[wave][i][D] = m[i];
+        merge[wave][i][D + 1] = l[i];
+      }
+    }
+  }
+  __syncthreads();
+  // merge the waves; one thread per (head, dim)
+  for (int e = threadIdx.x; e < n_heads * D; e += blockDim.x) {
+    int i = e / D, d = e % D;
+    float mm = merge[0][i][D];
+#pragma unroll
+    for (int w = 1; w < kDecWaves; ++w) mm = fmaxf(mm, merge[w][i][D]);
+    float ll = 0.f, aa = 0.f;
+#pragma unroll
+    for (int w = 0; w < kDecWaves; ++w) {
+      float sc = __expf(merge[w][i][D] - mm);
+      ll += merge[w][i][D + 1] * sc;
+      aa += merge[w][i][d] * sc;
+    }
+    float* ws = a.workspace + (((int64_t)t * a.Hq + h0 + i) * n_chunks + blockIdx.x) * (D + 2);
+    ws[d] = aa;
+    if (d == 0) {
+      ws[D] = mm;
+      ws[D + 1] = ll;
+    }
+  }
+}
+
+// out[t, h, :] = sum_c acc_c exp(m_c - M) / sum_c l_c exp(m_c - M), chunks in order.
+__global__ void attn_decode_merge_kernel(AttnArgs a, int n_chunks) {
+  const int t = blockIdx.x, h = blockIdx.y, D = a.D;
+  const int pos = a.positions[t];
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int c_lo = lo / kChunk, c_hi = pos / kChunk;
+  const float* ws = a.workspace + ((int64_t)t * a.Hq + h) * n_chunks * (D + 2);
+  float M = -1e30f;
+  for (int c = c_lo; c <= c_hi; ++c) M = fmaxf(M, ws[c * (D + 2) + D]);
+  float L = 0.f;
+  for (int c = c_lo; c <= c_hi; ++c) L += ws[c * (D + 2) + D + 1] * __expf(ws[c * (D + 2) + D] - M);
+  const float inv = 1.f / L;
+  bf16* out = (bf16*)a.out + ((int64_t)t * a.Hq + h) * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float acc = 0.f;
+    for (int c = c_lo; c <= c_hi; ++c)
+      acc += ws[c * (D + 2) + d] * __expf(ws[c * (D + 2) + D] - M);
+    out[d] = __float2bfloat16(acc * inv);
+  }
+}
+
+int64_t attention_decode_workspace_floats(int T, int Hq, int D, int max_kv_len) {
+  int n_chunks = (max_kv_len + kChunk - 1) / kChunk;
+  return (int64_t)T * Hq * n_chunks * (D + 2);
+}
+
+bool attention_decode_takes(const AttnArgs& a) {
+  int d = a.D;
+  bool d_ok = d == 16 || d == 32 || d == 64 || d == 128 || d == 256;
+  return a.dtype == kBF16 && d_ok && a.q_stride % 8 == 0 && a.workspace != nullptr;
+}
+
+template <int LPK>
+static void launch_decode(const AttnArgs& a, int n_chunks, hipStream_t stream) {
+  int group = a.Hq / a.Hkv;
+  if (group == 1) {
+    attn_decode_kernel<LPK, 1><<<dim3(n_chunks, a.Hkv, a.T), kDecWaves * 64, 0, stream>>>(a, 1);
+  } else if (group == 2) {
+    attn_decode_kernel<LPK, 2><<<dim3(n_chunks, a.Hkv, a.T), kDecWaves * 64, 0, stream>>>(a, 1);
+  } else {
+    int hg = (group + 3) / 4;
+    attn_decode_kernel<LPK, 4><<<dim3(n_chunks, a.Hkv * hg, a.T), kDecWaves * 64, 0, stream>>>(a, hg);
+  }
+}
+
+int attention_decode(const AttnArgs& a, hipStream_t stream) {
+  int n_chunks = (a.max_kv_len + kChunk - 1) / kChunk;
+  NINFER_REQUIRE(a.workspace_floats >= attention_decode_workspace_floats(a.T, a.Hq, a.D, a.max_kv_len),
+                 "paged_attention: workspace of %lld floats is too small", (long long)a.workspace_floats);
+  switch (a.D) {
+    case 16: launch_decode<2>(a, n_chunks, stream); break;
+    case 32: launch_decode<4>(a, n_chunks, stream); break;
+    case 64: launch_decode<8>(a, n_chunks, stream); break;
+    case 128: launch_decode<16>(a, n_chunks, stream); break;
+    case 256: launch_decode<32>(a, n_chunks, stream); break;
+    default: return set_error(-1, "paged_attention: decode kernel does not take head size %d", a.D);
+  }
+  NINFER_LAUNCH_CHECK();
+  attn_decode_merge_kernel<<<dim3(a.T, a.Hq), a.D >= 128 ? 128 : 64, 0, stream>>>(a, n_chunks);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace ninfer

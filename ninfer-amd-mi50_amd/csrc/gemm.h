@@ -29,7 +29,50 @@ struct GemmArgs {
   int epilogue;
 };
 
+// Which rows does tile `ti` of the grouped enumeration cover? Tiles of
+// `tile_rows` sorted rows are counted expert by expert from the device-side
+// offsets. Called by every thread of the block; the first wave scans 64 groups
+// at a time. info (LDS, 3 ints) receives {first row, end row of the expert,
+// expert}; returns false when the tile does not exist.
+__device__ inline bool find_tile(const int* __restrict__ offsets, int groups, int tile_rows,
+                                 int ti, int* info) {
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    int base = 0, found = 0;
+    for (int g0 = 0; g0 < groups && !found; g0 += 64) {
+      int g = g0 + lane, b = 0, e = 0;
+      if (g < groups) {
+        b = offsets[g];
+        e = offsets[g + 1];
+      }
+      int nt = (e - b + tile_rows - 1) / tile_rows;
+      int incl = nt;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        int v = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += v;
+      }
+      int lo = base + incl - nt, hi = base + incl;
+      bool mine = ti >= lo && ti < hi;
+      if (__ballot(mine)) {
+        found = 1;
+        if (mine) {
+          info[0] = b + (ti - lo) * tile_rows;
+          info[1] = e;
+          info[2] = g;
+        }
+      }
+      base += __shfl(incl, 63, 64);
+    }
+    if (!found && lane == 0) info[2] = -1;
+  }
+  __syncthreads();
+  return info[2] >= 0;
+}
+
 int gemm_check(const GemmArgs& a);
+bool gemm_skinny_takes(const GemmArgs& a);
+int gemm_skinny(const GemmArgs& a, hipStream_t stream);
 int gemm_generic(const GemmArgs& a, hipStream_t stream);
 
 }  // namespace ninfer

@@ -8,6 +8,7 @@ using namespace ninfer;
 extern "C" int ninfer_gemm(const GemmArgs* args, int force_generic, hipStream_t stream) {
   int rc = gemm_check(*args);
   if (rc) return rc;
-  (void)force_generic;
-  return gemm_generic(*args, stream);
+  const GemmArgs& a = *args;
+  if (!force_generic && gemm_skinny_takes(a)) return gemm_skinny(a, stream);
+  return gemm_generic(a, stream);
 }

@@ -27,25 +27,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs a) {
   // which rows: dense, or the tile `blockIdx.y` of the grouped enumeration
   int row0, row_end, group = 0;
   if (a.offsets) {
-    if (threadIdx.x == 0) {
-      int ti = blockIdx.y, g = 0, found = 0;
-      for (; g < a.groups; ++g) {
-        int b = a.offsets[g], e = a.offsets[g + 1];
-        int nt = (e - b + BM - 1) / BM;
-        if (ti < nt) {
-          tile_info[0] = b + ti * BM;
-          tile_info[1] = e;
-          tile_info[2] = g;
-          found = 1;
-          break;
-        }
-        ti -= nt;
-      }
-      if (!found) tile_info[2] = -1;
-    }
-    __syncthreads();
+    if (!find_tile(a.offsets, a.groups, BM, blockIdx.y, tile_info)) return;
     group = tile_info[2];
-    if (group < 0) return;
     row0 = tile_info[0];
     row_end = tile_info[1];
   } else {

@@ -1,0 +1,166 @@
+// C = A W^T for few rows (decode): every weight is read once from HBM and
+// multiplied on the matrix cores.
+//
+// One block owns 16 output features (16 rows of W; with the SwiGLU epilogue
+// the 16 gate rows and their 16 up rows) and up to 16 rows of A. The weight
+// rows are the A operand of v_mfma_f32_16x16x32_bf16 (lane l supplies row
+// l % 16, k = 8 (l / 16) .. +7, i.e. 16 contiguous bytes), the activations are
+// the B operand (lane l supplies token l % 16, same k), so the accumulator
+// holds a 16 x 16 tile out[feature 4 (l / 16) + v][token l % 16]. The K range is
+// split over the waves of the block in chunks of 128; partial tiles meet in LDS
+// and are summed in wave order, so the result does not depend on timing.
+// Activations are read straight from global memory (they stay in cache: few
+// rows), weights stream through registers with four 16-byte loads in flight
+// per lane and chunk.
+//
+// Grouped form as in the plain kernel: tiles of 16 sorted rows per expert are
+// enumerated from the device-side offsets; a block whose tile does not exist
+// exits. The reference runs these products as one GEMV per row (decode,
+// src/ops/gemv.hip:52-93) or one library call per expert
+// (src/models/model.hip:355-427).
+#include "gemm.h"
+
+namespace ninfer {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int SM = 16;  // rows of A per tile
+
+template <int WAVES, bool SWIGLU, typename TC>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a) {
+  __shared__ float red[WAVES][SWIGLU ? 2 : 1][256];
+  __shared__ int tile_info[3];
+
+  int row0, row_end, group = 0;
+  if (a.offsets) {
+    if (!find_tile(a.offsets, a.groups, SM, blockIdx.y, tile_info)) return;
+    group = tile_info[2];
+    row0 = tile_info[0];
+    row_end = tile_info[1];
+  } else {
+    row0 = blockIdx.y * SM;
+    row_end = a.M;
+    if (row0 >= row_end) return;
+  }
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, j = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int K = a.K;
+
+  const bf16* W = (const bf16*)a.W + (int64_t)group * a.w_group_stride;
+  const int n = min(n0 + r, a.N - 1);
+  const bf16* wrow = W + (int64_t)n * K + 8 * j;
+  const bf16* urow = SWIGLU ? wrow + (int64_t)a.N * K : nullptr;
+
+  const int mrow = row0 + r;
+  const bool m_valid = mrow < row_end;
+  int64_t a_row = 0;
+  if (m_valid) a_row = a.a_index ? a.a_index[mrow] / a.a_div : mrow;
+  const bf16* xrow = (const bf16*)a.A + a_row * a.lda + 8 * j;
+
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  f32x4 accu = {0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  const int steps = K / 32;
+  for (int c = wave; c * 4 < steps; c += WAVES) {
+    const int s0 = c * 4;
+    if (s0 + 4 <= steps) {
+      bf16x8 w[4], u[4], x[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        w[i] = *(const bf16x8*)(wrow + (s0 + i) * 32);
+        if (SWIGLU) u[i] = *(const bf16x8*)(urow + (s0 + i) * 32);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] = m_valid ? *(const bf16x8*)(xrow + (s0 + i) * 32) : zero;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[i], x[i], acc, 0, 0, 0);
+        if (SWIGLU) accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u[i], x[i], accu, 0, 0, 0);
+      }
+    } else {
+      for (int s = s0; s < steps; ++s) {
+        bf16x8 w = *(const bf16x8*)(wrow + s * 32);
+        bf16x8 x = m_valid ? *(const bf16x8*)(xrow + s * 32) : zero;
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, x, acc, 0, 0, 0);
+        if (SWIGLU) {
+          bf16x8 u = *(const bf16x8*)(urow + s * 32);
+          accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u, x, accu, 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // partial tiles -> LDS, element (feature f, token m) at [m * 16 + f]
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    int f = 4 * j + v;
+    red[wave][0][r * 16 + f] = acc[v];
+    if (SWIGLU) red[wave][1][r * 16 + f] = accu[v];
+  }
+  __syncthreads();
+  if (threadIdx.x < 256) {
+    const int m = threadIdx.x >> 4, f = threadIdx.x & 15;
+    const int row = row0 + m, col = n0 + f;
+    if (row < row_end && col < a.N) {
+      float v = 0.f, up = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) {
+        v += red[w][0][threadIdx.x];
+        if (SWIGLU) up += red[w][1][threadIdx.x];
+      }
+      if (SWIGLU) {
+        v = v / (1.f + __expf(-v)) * up;
+      } else if (a.bias) {
+        v += a.bias[col];
+      }
+      int64_t c_row = a.c_index ? a.c_index[row] : row;
+      ((TC*)a.C)[c_row * a.ldc + col] = from_f32<TC>(v);
+    }
+  }
+}
+
+template <int WAVES>
+static void launch_skinny(const GemmArgs& a, hipStream_t stream) {
+  int m_tiles = a.offsets ? min((a.M + SM - 1) / SM + a.groups, a.M) : (a.M + SM - 1) / SM;
+  dim3 grid((a.N + 15) / 16, m_tiles);
+  dim3 block(WAVES * 64);
+  bool swiglu = a.epilogue == kEpilogueSwiGLU;
+  if (a.out_dtype == kF32) {
+    if (swiglu)
+      gemm_skinny_kernel<WAVES, true, float><<<grid, block, 0, stream>>>(a);
+    else
+      gemm_skinny_kernel<WAVES, false, float><<<grid, block, 0, stream>>>(a);
+  } else {
+    if (swiglu)
+      gemm_skinny_kernel<WAVES, true, bf16><<<grid, block, 0, stream>>>(a);
+    else
+      gemm_skinny_kernel<WAVES, false, bf16><<<grid, block, 0, stream>>>(a);
+  }
+}
+
+// Shapes the kernel takes: bf16 inputs, K a multiple of 32, rows 16-byte aligned.
+bool gemm_skinny_takes(const GemmArgs& a) {
+  return a.in_dtype == kBF16 && a.K % 32 == 0 && a.lda % 8 == 0 &&
+         ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0) && a.w_group_stride % 8 == 0;
+}
+
+int gemm_skinny(const GemmArgs& a, hipStream_t stream) {
+  // more waves per block when the grid alone would leave CUs idle
+  int m_tiles = a.offsets ? a.groups : (a.M + SM - 1) / SM;
+  long blocks = (long)((a.N + 15) / 16) * m_tiles;
+  int chunks = a.K / 128;
+  if (blocks < 512 && chunks >= 16)
+    launch_skinny<16>(a, stream);
+  else if (blocks < 2048 && chunks >= 8)
+    launch_skinny<8>(a, stream);
+  else
+    launch_skinny<4>(a, stream);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace ninfer

@@ -70,7 +70,9 @@ class HipOps:
         self.lib_path = lib_path or ensure_built()
         self.lib = ctypes.CDLL(self.lib_path)
         self.lib.ninfer_last_error.restype = ctypes.c_char_p
+        self.lib.ninfer_attention_workspace_floats.restype = ctypes.c_longlong
         self.force_generic = False  # tests: run the plain kernels whatever the shape
+        self.library_min_rows = 32  # dense bf16 products with more rows go to the library
         self._attn_ws = None
 
     # ---- helpers ----------------------------------------------------------------
@@ -185,7 +187,26 @@ class HipOps:
         if bias is not None:
             _dev(bias, "bias", torch.float32, 1)
             _need(bias.shape[0] == w.shape[0], "linear: bias has the wrong size")
+        if self._use_library(x, out) and bias is None:
+            torch.matmul(x, w.t(), out=out)
+            return
         self._gemm(x, w, out, m=x.shape[0], n=w.shape[0], k=x.shape[1], bias=bias)
+
+    def _use_library(self, x, out) -> bool:
+        """Plain dense products of many bf16 rows go to the vendor library, as
+        the reference sends every multi-row product to rocBLAS
+        (src/ops/linear.hip:21-35); few rows, 32-bit, grouped and fused products
+        run on the hand-written kernels."""
+        return (not self.force_generic and x.dtype == torch.bfloat16 and out.dtype == x.dtype
+                and x.shape[0] > self.library_min_rows)
+
+    def silu_mul(self, x, out):
+        _dev(x, "x", dims=2)
+        _dev(out, "out", x.dtype, 2)
+        _need(x.shape[1] == 2 * out.shape[1] and x.shape[0] == out.shape[0], "silu_mul: shapes")
+        self._ok(self.lib.ninfer_silu_mul(ctypes.c_void_p(x.data_ptr()),
+                                          ctypes.c_void_p(out.data_ptr()), x.shape[0],
+                                          out.shape[1], _DT[x.dtype], self._stream()))
 
     def swiglu_linear(self, x, w_gate_up, out):
         """out = silu(x Wg^T) * (x Wu^T), Wg = rows [0, I), Wu = rows [I, 2I)."""
@@ -195,6 +216,11 @@ class HipOps:
         inner = w_gate_up.shape[0] // 2
         _need(w_gate_up.shape == (2 * inner, x.shape[1]), "swiglu_linear: weight shape")
         _need(out.shape == (x.shape[0], inner), "swiglu_linear: out has the wrong shape")
+        if self._use_library(x, out):
+            gu = torch.empty((x.shape[0], 2 * inner), dtype=x.dtype, device=x.device)
+            torch.matmul(x, w_gate_up.t(), out=gu)
+            self.silu_mul(gu, out)
+            return
         self._gemm(x, w_gate_up, out, m=x.shape[0], n=inner, k=x.shape[1], epilogue=1)
 
     def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out):
@@ -267,11 +293,18 @@ class HipOps:
               "paged_attention: pools do not fit the head layout")
         _need(block_table.shape[0] == ctx.S, "paged_attention: block table rows != requests")
         _need(ctx.positions.shape[0] == t, "paged_attention: positions size")
+        ws, ws_floats = None, 0
+        if ctx.max_qlen == 1 and qkv.dtype == torch.bfloat16 and not self.force_generic:
+            ws_floats = int(self.lib.ninfer_attention_workspace_floats(t, n_q, head_dim,
+                                                                       ctx.max_kv_len))
+            if self._attn_ws is None or self._attn_ws.numel() < ws_floats:
+                self._attn_ws = torch.empty(ws_floats, dtype=torch.float32, device=qkv.device)
+            ws = self._attn_ws.data_ptr()
         args = _AttnArgs(
             qkv.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), out.data_ptr(),
             block_table.data_ptr(), ctx.positions.data_ptr(), ctx.row_seq.data_ptr(),
             ctx.seq_row_start.data_ptr(), ctx.seq_qlen.data_ptr(), ctx.seq_pos0.data_ptr(),
-            None, 0, qkv.shape[1], block_table.shape[1], t, ctx.S, n_q, n_kv, head_dim, page_size,
+            ws, ws_floats, qkv.shape[1], block_table.shape[1], t, ctx.S, n_q, n_kv, head_dim, page_size,
             int(window or 0), float(scale), _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len)
         self._ok(self.lib.ninfer_paged_attention(ctypes.byref(args),
                                                  1 if self.force_generic else 0, self._stream()))

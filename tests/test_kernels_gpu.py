@@ -84,7 +84,8 @@ def test_rmsnorm(ops, gen, dtype, rows, h):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(1, 48, 40), (3, 130, 72), (17, 64, 200), (70, 200, 136),
-                                   (129, 96, 64)])
+                                   (129, 96, 64), (5, 130, 256), (16, 48, 2048), (33, 100, 128),
+                                   (8, 2048, 1408), (1, 300, 5632), (2, 61, 96)])
 def test_linear(ops_mode, gen, dtype, m, n, k):
     ops = ops_mode
     x, w = rnd((m, k), dtype, gen), rnd((n, k), dtype, gen)
@@ -99,7 +100,8 @@ def test_linear(ops_mode, gen, dtype, m, n, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("m,inner,k", [(1, 48, 64), (5, 80, 96), (66, 176, 72)])
+@pytest.mark.parametrize("m,inner,k", [(1, 48, 64), (5, 80, 96), (66, 176, 72), (20, 1408, 256),
+                                       (3, 100, 2048)])
 def test_swiglu_linear(ops_mode, gen, dtype, m, inner, k):
     ops = ops_mode
     x, w = rnd((m, k), dtype, gen), rnd((2 * inner, k), dtype, gen, 0.3)
@@ -123,7 +125,9 @@ def test_linear_row_result_does_not_depend_on_batch(ops, gen):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("t,e,k,h,inner", [(1, 4, 2, 64, 32), (17, 8, 3, 96, 48),
-                                           (150, 60, 4, 128, 80), (3, 6, 6, 72, 40)])
+                                           (150, 60, 4, 128, 80), (3, 6, 6, 72, 40),
+                                           (40, 6, 2, 128, 64), (300, 4, 2, 64, 96),
+                                           (8, 60, 4, 256, 160)])
 def test_router_align_experts_combine(ops_mode, gen, dtype, t, e, k, h, inner):
     """The whole sparse feed-forward chain, kernel by kernel, against the twins;
     with few rows most experts get none."""
@@ -222,6 +226,25 @@ def _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, n_pages):
 def test_paged_attention(ops_mode, gen, dtype, n_q, n_kv, d, page_size, window):
     ops = ops_mode
     seqs = [(0, 1), (0, 37), (130, 1), (61, 5), (17, 70), (255, 1)]
+    ctx, qkv, k_pool, v_pool, bt = _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, 80)
+    o1 = torch.empty(ctx.T, n_q * d, device="cuda", dtype=dtype)
+    o2 = torch.empty_like(o1)
+    scale = 1 / math.sqrt(d)
+    ops.paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, page_size, window, scale, o1)
+    PlainOps().paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, page_size, window,
+                               scale, o2)
+    close(o1, o2, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_q,n_kv,d,page_size,window", [
+    (4, 2, 16, 4, 0), (3, 1, 32, 8, 24), (16, 16, 128, 16, 0), (28, 4, 128, 16, 0),
+    (8, 8, 64, 16, 300), (10, 2, 64, 64, 0), (2, 2, 80, 16, 0), (4, 1, 256, 16, 0)])
+def test_paged_attention_decode_rows(ops_mode, gen, dtype, n_q, n_kv, d, page_size, window):
+    """Single-token rows only: the split-context kernel's case. Contexts end at
+    chunk and page edges and inside them."""
+    ops = ops_mode
+    seqs = [(0, 1), (15, 1), (16, 1), (255, 1), (256, 1), (700, 1), (1023, 1), (511, 1)]
     ctx, qkv, k_pool, v_pool, bt = _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, 80)
     o1 = torch.empty(ctx.T, n_q * d, device="cuda", dtype=dtype)
     o2 = torch.empty_like(o1)
