@@ -176,22 +176,40 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
 }
 
 // out[t, h, :] = sum_c acc_c exp(m_c - M) / sum_c l_c exp(m_c - M), chunks in order.
-__global__ void attn_decode_merge_kernel(AttnArgs a, int n_chunks) {
-  const int t = blockIdx.x, h = blockIdx.y, D = a.D;
+// Block of 128 threads; LDS holds one scale per chunk.
+__global__ __launch_bounds__(128) void attn_decode_merge_kernel(AttnArgs a, int n_chunks) {
+  extern __shared__ float scale_s[];   // [n_chunks]
+  __shared__ float red[4];
+  const int t = blockIdx.x, h = blockIdx.y, D = a.D, tid = threadIdx.x;
   const int pos = a.positions[t];
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int c_lo = lo / kChunk, c_hi = pos / kChunk;
   const float* ws = a.workspace + ((int64_t)t * a.Hq + h) * n_chunks * (D + 2);
-  float M = -1e30f;
-  for (int c = c_lo; c <= c_hi; ++c) M = fmaxf(M, ws[c * (D + 2) + D]);
-  float L = 0.f;
-  for (int c = c_lo; c <= c_hi; ++c) L += ws[c * (D + 2) + D + 1] * __expf(ws[c * (D + 2) + D] - M);
-  const float inv = 1.f / L;
+  float mx = -1e30f;
+  for (int c = c_lo + tid; c <= c_hi; c += 128) {
+    float m = ws[c * (D + 2) + D];
+    scale_s[c] = m;
+    mx = fmaxf(mx, m);
+  }
+  mx = wave_max(mx);
+  if ((tid & 63) == 0) red[tid >> 6] = mx;
+  __syncthreads();
+  const float M = fmaxf(red[0], red[1]);
+  float lsum = 0.f;
+  for (int c = c_lo + tid; c <= c_hi; c += 128) {
+    float sc = __expf(scale_s[c] - M);
+    scale_s[c] = sc;
+    lsum += ws[c * (D + 2) + D + 1] * sc;
+  }
+  lsum = wave_sum(lsum);
+  if ((tid & 63) == 0) red[2 + (tid >> 6)] = lsum;
+  __syncthreads();
+  const float inv = 1.f / (red[2] + red[3]);
   bf16* out = (bf16*)a.out + ((int64_t)t * a.Hq + h) * D;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+  for (int d = tid; d < D; d += 128) {
     float acc = 0.f;
-    for (int c = c_lo; c <= c_hi; ++c)
-      acc += ws[c * (D + 2) + d] * __expf(ws[c * (D + 2) + D] - M);
+#pragma unroll 4
+    for (int c = c_lo; c <= c_hi; ++c) acc = fmaf(ws[c * (D + 2) + d], scale_s[c], acc);
     out[d] = __float2bfloat16(acc * inv);
   }
 }
@@ -233,7 +251,7 @@ int attention_decode(const AttnArgs& a, hipStream_t stream) {
     default: return set_error(-1, "paged_attention: decode kernel does not take head size %d", a.D);
   }
   NINFER_LAUNCH_CHECK();
-  attn_decode_merge_kernel<<<dim3(a.T, a.Hq), a.D >= 128 ? 128 : 64, 0, stream>>>(a, n_chunks);
+  attn_decode_merge_kernel<<<dim3(a.T, a.Hq), 128, n_chunks * sizeof(float), stream>>>(a, n_chunks);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

@@ -110,15 +110,16 @@ template <typename T>
 __global__ void moe_combine_kernel(float* __restrict__ residual, const T* __restrict__ y,
                                    const float* __restrict__ w, const T* __restrict__ shared,
                                    const float* __restrict__ gate, int H, int k) {
-  int64_t t = blockIdx.x;
-  float g = 0.f;
-  if (shared) g = gate ? 1.f / (1.f + expf(-gate[t])) : 1.f;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    float acc = 0.f;
-    for (int j = 0; j < k; ++j) acc += w[t * k + j] * to_f32(y[(t * k + j) * H + i]);
-    if (shared) acc += g * to_f32(shared[t * H + i]);
-    residual[t * H + i] += acc;
+  const int64_t t = blockIdx.x;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i >= H) return;
+  float acc = 0.f;
+  for (int j = 0; j < k; ++j) acc += w[t * k + j] * to_f32(y[(t * k + j) * H + i]);
+  if (shared) {
+    float g = gate ? 1.f / (1.f + expf(-gate[t])) : 1.f;
+    acc += g * to_f32(shared[t * H + i]);
   }
+  residual[t * H + i] += acc;
 }
 
 // out[r, i] = silu(x[r, i]) * x[r, I + i]   (reference src/ops/kernels.hip:131-140)
@@ -209,10 +210,10 @@ extern "C" int ninfer_moe_combine(float* residual, const void* y, const float* w
   NINFER_REQUIRE(T > 0 && H > 0 && k > 0, "moe_combine: T=%d H=%d k=%d must be positive", T, H, k);
   NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "moe_combine: unknown dtype %d", dtype);
   if (dtype == kF32)
-    moe_combine_kernel<float><<<T, 256, 0, stream>>>(residual, (const float*)y, w,
+    moe_combine_kernel<float><<<dim3(T, (H + 255) / 256), 256, 0, stream>>>(residual, (const float*)y, w,
                                                     (const float*)shared, gate, H, k);
   else
-    moe_combine_kernel<bf16><<<T, 256, 0, stream>>>(residual, (const bf16*)y, w,
+    moe_combine_kernel<bf16><<<dim3(T, (H + 255) / 256), 256, 0, stream>>>(residual, (const bf16*)y, w,
                                                    (const bf16*)shared, gate, H, k);
   NINFER_LAUNCH_CHECK();
   return 0;

@@ -68,6 +68,8 @@ class ModelRunner:
         self.cache.allocate_pools(self.device, self.act_dtype)
         self.vocab_size = spec.vocab_size
         self.steps_run = 0
+        self._graphs: Dict[tuple, dict] = {}
+        self.graph_context_step = 1024   # a graph serves contexts up to the next multiple
 
     # ---- requests --------------------------------------------------------------
     def open(self) -> int:
@@ -117,34 +119,87 @@ class ModelRunner:
             r += n
         if tokens.min() < 0 or tokens.max() >= self.vocab_size:
             raise ValueError(f"token id outside [0, {self.vocab_size})")
-        tables = [cache.block_table(g, slots) for g in range(len(cache.groups))]
+        max_kv_len = int(max(p + len(c.tokens) for c, p in zip(chunks, pos0)))
+        graph = (self.options.use_graph and self.device.type == "cuda" and int(qlen.max()) == 1
+                 and want_rows == list(range(T)))
+        # a graph is replayed for many steps: fixed table width, context rounded up
+        width = cache.max_pages_per_request if graph else None
+        if graph:
+            max_kv_len = min(-(-max_kv_len // self.graph_context_step) * self.graph_context_step,
+                             cache.max_pages_per_request * cache.page_size)
+        tables = [cache.block_table(g, slots, width) for g in range(len(cache.groups))]
         parts = [tokens, positions, row_seq, np.asarray(slots, np.int32), row_start, qlen,
                  np.asarray(pos0, np.int32), np.asarray(want_rows, np.int32)]
         parts += [t.reshape(-1) for t in tables]
         sizes = [x.size for x in parts]
-        host = torch.from_numpy(np.concatenate(parts)).pin_memory() \
-            if self.device.type == "cuda" else torch.from_numpy(np.concatenate(parts))
-        dev = host.to(self.device, non_blocking=True)
-        views = []
-        o = 0
-        for n in sizes:
-            views.append(dev[o:o + n])
-            o += n
-        d_tables = [v.view(S, t.shape[1]) for v, t in zip(views[8:], tables)]
-        ctx = StepContext(
-            ops=self.ops, act_dtype=self.act_dtype, device=self.device, T=T, S=S,
-            tokens=views[0], positions=views[1], row_seq=views[2], seq_slots=views[3],
-            seq_row_start=views[4], seq_qlen=views[5], seq_pos0=views[6],
-            max_qlen=int(qlen.max()), max_kv_len=int(max(p + len(c.tokens)
-                                                         for c, p in zip(chunks, pos0))),
-            all_decode=bool(qlen.max() == 1))
-        ctx.scratch["host_qlen"] = qlen
-        ctx.scratch["host_pos0"] = np.asarray(pos0, np.int32)
-        logits = self.spec.forward(ctx, self._call_infos(d_tables), views[7] if want_rows else None)
+        host = torch.from_numpy(np.concatenate(parts))
+        shape = dict(T=T, S=S, sizes=sizes, widths=[t.shape[1] for t in tables],
+                     max_qlen=int(qlen.max()), max_kv_len=max_kv_len, wants=bool(want_rows))
+        if graph:
+            logits = self._step_graph(host, shape)
+        else:
+            if self.device.type == "cuda":
+                host = host.pin_memory()
+            logits = self._forward(host.to(self.device, non_blocking=True), shape)
         for c, p in zip(chunks, pos0):
             cache.commit(c.slot, p + len(c.tokens))
         self.steps_run += 1
         return logits
+
+    def _forward(self, dev: torch.Tensor, shape: dict) -> Optional[torch.Tensor]:
+        """Run the model on the step described by the packed index buffer `dev`
+        (tokens, positions, row_seq, slots, row_start, qlen, pos0, wanted rows,
+        then one block table per cache group)."""
+        views = []
+        o = 0
+        for n in shape["sizes"]:
+            views.append(dev[o:o + n])
+            o += n
+        S = shape["S"]
+        d_tables = [v.view(S, w) for v, w in zip(views[8:], shape["widths"])]
+        ctx = StepContext(
+            ops=self.ops, act_dtype=self.act_dtype, device=self.device, T=shape["T"], S=S,
+            tokens=views[0], positions=views[1], row_seq=views[2], seq_slots=views[3],
+            seq_row_start=views[4], seq_qlen=views[5], seq_pos0=views[6],
+            max_qlen=shape["max_qlen"], max_kv_len=shape["max_kv_len"],
+            all_decode=shape["max_qlen"] == 1)
+        return self.spec.forward(ctx, self._call_infos(d_tables),
+                                 views[7] if shape["wants"] else None)
+
+    def _step_graph(self, host: torch.Tensor, shape: dict) -> torch.Tensor:
+        """Decode-only steps replayed from a captured HIP graph: one graph per
+        (requests in the step, context bound). The index buffer is the graph's
+        only input; it is refreshed by one copy before every replay. The first
+        step of a shape runs eagerly (it also sizes every workspace), the
+        second is captured. The reference captures its single-token dense
+        decode the same way (src/models/model.hip:786-830). The returned logits
+        live in the graph's memory and are valid until the next step."""
+        key = (shape["S"], shape["max_kv_len"])
+        entry = self._graphs.get(key)
+        if entry is None:
+            self._graphs[key] = {"pinned": torch.empty(host.numel(), dtype=torch.int32).pin_memory(),
+                                 "meta": torch.empty(host.numel(), dtype=torch.int32,
+                                                     device=self.device), "graph": None}
+            entry = self._graphs[key]
+            entry["pinned"].copy_(host)
+            entry["meta"].copy_(entry["pinned"], non_blocking=True)
+            return self._forward(entry["meta"], shape)
+        # the pinned staging buffer is reused: wait until the last copy from it is done
+        if entry.get("copied") is not None:
+            entry["copied"].synchronize()
+        entry["pinned"].copy_(host)
+        entry["meta"].copy_(entry["pinned"], non_blocking=True)
+        if entry.get("copied") is None:
+            entry["copied"] = torch.cuda.Event()
+        entry["copied"].record()
+        if entry["graph"] is None:
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                entry["logits"] = self._forward(entry["meta"], shape)
+            entry["graph"] = g
+        entry["graph"].replay()
+        return entry["logits"]
 
     def _call_infos(self, d_tables: List[torch.Tensor]) -> List[CallInfo]:
         cache = self.cache

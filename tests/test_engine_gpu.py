@@ -84,3 +84,36 @@ def test_32bit_does_not_depend_on_the_cut(case):
     b = util.run_schedule(runner, util.schedule_tail(rid, toks, 32))[rid]
     c = util.run_schedule(runner, util.schedule_portions(rid, toks, 1))[rid]
     assert torch.equal(a, b) and torch.equal(a, c)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replay_equals_eager(case, dtype):
+    """Decode-only steps replayed from a HIP graph give the logits of the same
+    steps run eagerly, replay after replay, with eager steps (other shapes,
+    prompts of new requests) in between."""
+    from ninfer_amd import Chunk, EngineOptions, load_model
+    runners = []
+    for use_graph in (False, True):
+        opt = EngineOptions(dtype=dtype, max_context=128, num_sequences=4, page_size=8,
+                            num_pages=64, use_graph=use_graph)
+        runners.append(load_model(case["dirs"][dtype], opt))
+    reqs = list(case["reqs"].values())[:3]
+    outs = [[], []]
+    for which, runner in enumerate(runners):
+        slots = [runner.open() for _ in reqs]
+        for s, toks in zip(slots, reqs):
+            runner.step([Chunk(s, toks[:5], [])])
+        for i in range(5, 15):
+            logits = runner.step([Chunk(s, [toks[i]], [0]) for s, toks in zip(slots, reqs)])
+            outs[which].append(logits.float().cpu().clone())
+            if i == 9:   # an eager step of another shape between replays
+                extra = runner.open()
+                runner.step([Chunk(extra, reqs[0][:7], [6])])
+                runner.close(extra)
+            if i == 11:  # fewer requests: another graph
+                runner.close(slots.pop())
+        for s in slots:
+            runner.close(s)
+    assert runners[1]._graphs and any(e["graph"] is not None for e in runners[1]._graphs.values())
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
