@@ -13,7 +13,7 @@ struct AttnArgs {
   const int* block_table;   // [S, bt_stride] page of each logical page, -1 when given back
   const int* positions;     // [T] absolute position of each row
   const int* row_seq;       // [T] request (index in this step) of each row
-  const int* seq_row_start; // [S]
+  const int* seq_row_start; // [S + 1] first row of each request, then T
   const int* seq_qlen;      // [S]
   const int* seq_pos0;      // [S]
   float* workspace;         // split-KV partial results, or null
@@ -41,5 +41,7 @@ int attention_generic(const void* q, int q_stride, const void* kpool, const void
 int64_t attention_decode_workspace_floats(int T, int Hq, int D, int max_kv_len);
 bool attention_decode_takes(const AttnArgs& a);
 int attention_decode(const AttnArgs& a, hipStream_t stream);
+bool attention_prefill_takes(const AttnArgs& a);
+int attention_prefill(const AttnArgs& a, hipStream_t stream);
 
 }  // namespace ninfer

@@ -21,6 +21,7 @@ extern "C" int ninfer_paged_attention(const AttnArgs* a, int force_generic, hipS
   NINFER_REQUIRE(a->max_qlen >= 1 && a->max_kv_len >= 1, "paged_attention: bad size hints");
   if (!force_generic && a->max_qlen == 1 && attention_decode_takes(*a))
     return attention_decode(*a, stream);
+  if (!force_generic && attention_prefill_takes(*a)) return attention_prefill(*a, stream);
   return attention_generic(a->q, a->q_stride, a->kpool, a->vpool, a->block_table, a->bt_stride,
                            a->positions, a->row_seq, a->out, a->T, a->Hq, a->Hkv, a->D,
                            a->page_size, a->window, a->scale, a->dtype, stream);

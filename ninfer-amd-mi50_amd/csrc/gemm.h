@@ -73,6 +73,8 @@ __device__ inline bool find_tile(const int* __restrict__ offsets, int groups, in
 int gemm_check(const GemmArgs& a);
 bool gemm_skinny_takes(const GemmArgs& a);
 int gemm_skinny(const GemmArgs& a, hipStream_t stream);
+bool gemm_tile_takes(const GemmArgs& a);
+int gemm_tile(const GemmArgs& a, hipStream_t stream);
 int gemm_generic(const GemmArgs& a, hipStream_t stream);
 
 }  // namespace ninfer

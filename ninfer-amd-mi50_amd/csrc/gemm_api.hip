@@ -9,6 +9,11 @@ extern "C" int ninfer_gemm(const GemmArgs* args, int force_generic, hipStream_t 
   int rc = gemm_check(*args);
   if (rc) return rc;
   const GemmArgs& a = *args;
-  if (!force_generic && gemm_skinny_takes(a)) return gemm_skinny(a, stream);
+  if (!force_generic) {
+    // many rows per weight matrix: 64-row tiles; few: 16-row tiles that stream the weights
+    bool many = a.offsets ? a.M >= 16 * a.groups : a.M > 32;
+    if (many && gemm_tile_takes(a)) return gemm_tile(a, stream);
+    if (gemm_skinny_takes(a)) return gemm_skinny(a, stream);
+  }
   return gemm_generic(a, stream);
 }

@@ -101,7 +101,7 @@ class ModelRunner:
         tokens = np.empty(T, np.int32)
         positions = np.empty(T, np.int32)
         row_seq = np.empty(T, np.int32)
-        row_start = np.empty(S, np.int32)
+        row_start = np.empty(S + 1, np.int32)
         qlen = np.empty(S, np.int32)
         want_rows: List[int] = []
         r = 0
@@ -117,6 +117,7 @@ class ModelRunner:
                     raise ValueError(f"wanted row {w} is outside the request's {n} tokens")
                 want_rows.append(r + w)
             r += n
+        row_start[S] = T
         if tokens.min() < 0 or tokens.max() >= self.vocab_size:
             raise ValueError(f"token id outside [0, {self.vocab_size})")
         max_kv_len = int(max(p + len(c.tokens) for c, p in zip(chunks, pos0)))

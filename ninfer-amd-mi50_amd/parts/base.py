@@ -66,7 +66,7 @@ class StepContext:
     positions: torch.Tensor       # [T] absolute position of each row in its request
     row_seq: torch.Tensor         # [T] index (within this step) of the row's request
     seq_slots: torch.Tensor       # [S] slot of each request (index into state)
-    seq_row_start: torch.Tensor   # [S]
+    seq_row_start: torch.Tensor   # [S + 1] first row of each request, then T
     seq_qlen: torch.Tensor        # [S]
     seq_pos0: torch.Tensor        # [S] position of the request's first row
     max_qlen: int = 1

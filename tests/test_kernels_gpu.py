@@ -85,7 +85,8 @@ def test_rmsnorm(ops, gen, dtype, rows, h):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(1, 48, 40), (3, 130, 72), (17, 64, 200), (70, 200, 136),
                                    (129, 96, 64), (5, 130, 256), (16, 48, 2048), (33, 100, 128),
-                                   (8, 2048, 1408), (1, 300, 5632), (2, 61, 96)])
+                                   (8, 2048, 1408), (1, 300, 5632), (2, 61, 96), (200, 60, 128),
+                                   (333, 700, 256), (64, 256, 32)])
 def test_linear(ops_mode, gen, dtype, m, n, k):
     ops = ops_mode
     x, w = rnd((m, k), dtype, gen), rnd((n, k), dtype, gen)
@@ -101,7 +102,7 @@ def test_linear(ops_mode, gen, dtype, m, n, k):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,inner,k", [(1, 48, 64), (5, 80, 96), (66, 176, 72), (20, 1408, 256),
-                                       (3, 100, 2048)])
+                                       (3, 100, 2048), (130, 300, 128), (64, 128, 64)])
 def test_swiglu_linear(ops_mode, gen, dtype, m, inner, k):
     ops = ops_mode
     x, w = rnd((m, k), dtype, gen), rnd((2 * inner, k), dtype, gen, 0.3)
@@ -127,7 +128,8 @@ def test_linear_row_result_does_not_depend_on_batch(ops, gen):
 @pytest.mark.parametrize("t,e,k,h,inner", [(1, 4, 2, 64, 32), (17, 8, 3, 96, 48),
                                            (150, 60, 4, 128, 80), (3, 6, 6, 72, 40),
                                            (40, 6, 2, 128, 64), (300, 4, 2, 64, 96),
-                                           (8, 60, 4, 256, 160)])
+                                           (8, 60, 4, 256, 160), (700, 5, 3, 128, 192),
+                                           (512, 8, 2, 64, 96)])
 def test_router_align_experts_combine(ops_mode, gen, dtype, t, e, k, h, inner):
     """The whole sparse feed-forward chain, kernel by kernel, against the twins;
     with few rows most experts get none."""
@@ -209,6 +211,7 @@ def _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, n_pages):
         row_start.append(len(positions))
         positions += list(range(p, p + q))
         row_seq += [i] * q
+    row_start.append(len(positions))
     dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
     ctx = SimpleNamespace(S=s, T=t, positions=dev(positions), row_seq=dev(row_seq),
                           seq_row_start=dev(row_start), seq_qlen=dev([q for _, q in seqs]),
@@ -222,11 +225,18 @@ def _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, n_pages):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_q,n_kv,d,page_size,window", [
     (4, 2, 16, 4, 0), (3, 1, 32, 8, 24), (16, 16, 128, 16, 0), (28, 4, 128, 16, 0),
-    (6, 3, 48, 16, 37), (8, 2, 64, 32, 0), (2, 2, 80, 16, 0)])
+    (6, 3, 48, 16, 37), (8, 2, 64, 32, 0), (2, 2, 80, 16, 0), (4, 2, 64, 16, 50),
+    (14, 2, 128, 64, 100)])
 def test_paged_attention(ops_mode, gen, dtype, n_q, n_kv, d, page_size, window):
     ops = ops_mode
-    seqs = [(0, 1), (0, 37), (130, 1), (61, 5), (17, 70), (255, 1)]
+    seqs = [(0, 1), (0, 37), (130, 1), (61, 5), (17, 70), (255, 1), (3, 200), (64, 64)]
     ctx, qkv, k_pool, v_pool, bt = _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, 80)
+    if window:
+        # pages a window has wholly passed are given back: the kernel must not need them
+        for i, (p, q) in enumerate(seqs):
+            dead = (p - window + 1) // page_size
+            if dead > 0:
+                bt[i, :dead] = -1
     o1 = torch.empty(ctx.T, n_q * d, device="cuda", dtype=dtype)
     o2 = torch.empty_like(o1)
     scale = 1 / math.sqrt(d)
