@@ -94,8 +94,6 @@ class ModelRunner:
         for c in chunks:
             if len(c.tokens) < 1:
                 raise ValueError("a request in a step brings at least one token")
-        # pages for all requests of the step, or for none
-        cache.reserve_all([(c.slot, p + len(c.tokens)) for c, p in zip(chunks, pos0)])
         T = sum(len(c.tokens) for c in chunks)
         S = len(chunks)
         tokens = np.empty(T, np.int32)
@@ -120,6 +118,8 @@ class ModelRunner:
         row_start[S] = T
         if tokens.min() < 0 or tokens.max() >= self.vocab_size:
             raise ValueError(f"token id outside [0, {self.vocab_size})")
+        # the batch is well formed: now pages for all its requests, or for none
+        cache.reserve_all([(c.slot, p + len(c.tokens)) for c, p in zip(chunks, pos0)])
         max_kv_len = int(max(p + len(c.tokens) for c, p in zip(chunks, pos0)))
         graph = (self.options.use_graph and self.device.type == "cuda" and int(qlen.max()) == 1
                  and want_rows == list(range(T)))

@@ -32,20 +32,27 @@ class ModelSpec:
         self.blocks = blocks
         self.final_norm = final_norm
         self.head = head
-        self.plan = plan if plan is not None else [LayerCall(i) for i in range(len(blocks))]
         self.vocab_size = vocab_size if vocab_size is not None else head.vocab
         self.eos_token_id = eos_token_id
-        for i, call in enumerate(self.plan):
-            if not 0 <= call.layer < len(blocks):
+        self.plan: List[LayerCall] = []
+        self.set_plan(plan if plan is not None else [LayerCall(i) for i in range(len(blocks))])
+
+    def set_plan(self, plan: List[LayerCall]) -> None:
+        """Replace the order the layers run in (before the model is bound to a
+        cache); refuses entries that name no layer or read a cache that is not
+        written earlier."""
+        for i, call in enumerate(plan):
+            if not 0 <= call.layer < len(self.blocks):
                 raise ValueError(f"plan entry {i} names layer {call.layer}; the model has "
-                                 f"{len(blocks)}")
+                                 f"{len(self.blocks)}")
             if call.cache_from is not None:
                 if not 0 <= call.cache_from < i:
                     raise ValueError(f"plan entry {i} reads the cache of entry "
                                      f"{call.cache_from}, which does not run before it")
-                if self.plan[call.cache_from].cache_from is not None:
+                if plan[call.cache_from].cache_from is not None:
                     raise ValueError(f"plan entry {i} reads the cache of entry "
                                      f"{call.cache_from}, which has no cache of its own")
+        self.plan = list(plan)
 
     def parts(self) -> List[Part]:
         return [self.embedding, *self.blocks, self.final_norm, self.head]

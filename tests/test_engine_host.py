@@ -1,0 +1,134 @@
+"""The engine's host logic on the CPU: batch building, block tables, cache
+manager, layer plan and state slots run end to end, with the plain twins of
+the kernels (tests/plain_ops.py) in place of the HIP library, against the
+plain implementation. The same replays run on the GPU with the real kernels in
+test_engine_gpu.py."""
+import pytest
+import torch
+
+import plain_model
+import toy
+import util
+from conftest import TINY
+from plain_ops import PlainOps
+
+
+def runner_for(model_dir, page_size=8, num_pages=24, seqs=4, plan=None):
+    from ninfer_amd import EngineOptions, load_model
+    from ninfer_amd.models.spec import LayerCall
+    opt = EngineOptions(dtype="float32", max_context=128, num_sequences=seqs, page_size=page_size,
+                        num_pages=num_pages, device="cpu")
+    if plan is None:
+        return load_model(model_dir, opt, ops=PlainOps())
+    # the order layers run in is data: rebuild the runner with another plan
+    from ninfer_amd.config import read_config_json
+    from ninfer_amd.engine import ModelRunner
+    from ninfer_amd.loading import build_spec
+    from ninfer_amd.weights import CheckpointSource
+    _, spec = build_spec(read_config_json(model_dir))
+    spec.set_plan([LayerCall(l, c) for l, c in plan])
+    return ModelRunner(spec, CheckpointSource(model_dir), opt, ops=PlainOps())
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_every_way_of_cutting_equals_the_plain_model(model_dirs, name):
+    d = model_dirs[name]["float32"]
+    cfg, w = util.read_folder(d)
+    runner = runner_for(d)
+    reqs = {f"r{i}": util.random_tokens(n, cfg["vocab_size"], 10 + i)
+            for i, n in enumerate([5, 40, 33, 20, 47, 17])}
+    ref = {k: plain_model.forward(w, cfg, v) for k, v in reqs.items()}
+    for k, v in reqs.items():
+        for sched in (util.schedule_whole(k, v), util.schedule_tail(k, v),
+                      util.schedule_portions(k, v, 3)):
+            torch.testing.assert_close(util.run_schedule(runner, sched)[k], ref[k],
+                                       atol=2e-5, rtol=1e-4)
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=5))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=2e-5, rtol=1e-4)
+    runner.cache.check()
+    assert runner.cache.pages_reused() > 0
+    assert all(g.allocator.in_use == 0 for g in runner.cache.groups)
+    if name == "B":
+        assert [g.window for g in runner.cache.groups] == [None, 24]
+        assert runner.cache.groups[1].window_freed > 0
+
+
+def test_mixed_schedule_has_portions_beside_single_tokens():
+    reqs = {f"r{i}": list(range(n)) for i, n in enumerate([5, 40, 33, 20, 47])}
+    steps = util.schedule_mixed(reqs, seed=5)
+    assert max(len(e) for e, _ in steps) == 4
+    assert any(any(len(t) > 1 for _, t, _ in e) and any(len(t) == 1 for _, t, _ in e)
+               for e, _ in steps)
+    assert min(len(t) for e, _ in steps for _, t, _ in e) == 1
+    fed = {k: sum(len(t) for e, _ in steps for r, t, _ in e if r == k) for k in reqs}
+    assert fed == {k: len(v) for k, v in reqs.items()}
+
+
+@pytest.mark.parametrize("plan", [[(0, None), (1, 0), (2, None)],
+                                  [(0, None), (1, None), (1, None), (2, None)],
+                                  [(2, None), (0, None)]])
+def test_layer_plan_is_data(model_dirs, plan):
+    """A layer named twice, a layer that reads another call's cache, layers in
+    another order: the same parts, another list."""
+    d = model_dirs["B"]["float32"]
+    cfg, w = util.read_folder(d)
+    runner = runner_for(d, plan=plan)
+    toks = util.random_tokens(45, cfg["vocab_size"], 77)
+    ref = plain_model.forward(w, cfg, toks, plan=plan)
+    for sched in (util.schedule_whole("x", toks), util.schedule_portions("x", toks, 2),
+                  util.schedule_tail("x", toks, 12)):
+        torch.testing.assert_close(util.run_schedule(runner, sched)["x"], ref, atol=2e-5, rtol=1e-4)
+    own_caches = sum(1 for _, src in plan if src is None)
+    assert len(runner.cache.pools) == own_caches
+
+
+def test_bad_plans_are_refused(model_dirs):
+    with pytest.raises(ValueError, match="does not run before"):
+        runner_for(model_dirs["B"]["float32"], plan=[(0, 1), (1, None)])
+    with pytest.raises(ValueError, match="names layer 7"):
+        runner_for(model_dirs["B"]["float32"], plan=[(7, None)])
+    with pytest.raises(ValueError, match="no cache of its own"):
+        runner_for(model_dirs["B"]["float32"], plan=[(0, None), (1, 0), (2, 1)])
+
+
+def test_step_refuses_bad_batches(model_dirs):
+    from ninfer_amd import Chunk
+    from ninfer_amd.cache import OutOfPages
+    runner = runner_for(model_dirs["A"]["float32"], num_pages=4)
+    s = runner.open()
+    with pytest.raises(ValueError, match="once in a step"):
+        runner.step([Chunk(s, [1], []), Chunk(s, [2], [])])
+    with pytest.raises(ValueError, match="token id"):
+        runner.step([Chunk(s, [99999], [])])
+    with pytest.raises(ValueError, match="at least one token"):
+        runner.step([Chunk(s, [], [])])
+    with pytest.raises(ValueError, match="wanted row"):
+        runner.step([Chunk(s, [1, 2], [2])])
+    with pytest.raises(OutOfPages):
+        runner.step([Chunk(s, list(range(40)), [])])
+    assert runner.cache.length(s) == 0 and runner.cache.pages_free(0) == 4
+    assert runner.step([Chunk(s, [1, 2, 3], [])]) is None      # nothing wanted: no logits
+
+
+def test_toy_mixer_with_state_of_its_own(tmp_path):
+    """Registered, written, loaded and stepped through the framework's own entry
+    points; its state lives in the request's slot, is carried across steps and
+    is zeroed when a slot is used again."""
+    import ninfer_amd
+    toy.register()
+    d = str(tmp_path / "toy")
+    ninfer_amd.write_random_model(d, toy.TOY_CONFIG, 5, std=0.2)
+    cfg, w = util.read_folder(d)
+    runner = runner_for(d, seqs=3)
+    assert runner.cache.state_floats == 2 * 40 and not runner.cache.pools
+    reqs = {f"t{i}": util.random_tokens(n, 97, 60 + i) for i, n in enumerate([9, 21, 14, 30, 6])}
+    ref = {k: toy.plain_forward(w, cfg, v) for k, v in reqs.items()}
+    for k, v in reqs.items():
+        for sched in (util.schedule_whole(k, v), util.schedule_tail(k, v, 5),
+                      util.schedule_portions(k, v, 1)):
+            torch.testing.assert_close(util.run_schedule(runner, sched)[k], ref[k],
+                                       atol=2e-5, rtol=1e-4)
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=3, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=2e-5, rtol=1e-4)
