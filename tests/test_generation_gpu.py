@@ -1,0 +1,129 @@
+"""Generation through the entry points on the GPU: greedy tokens equal the
+plain implementation's; long decoding; the first tokens of a sequence; the
+command line; the toy architecture and other layer plans with the real
+kernels."""
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_model
+import toy
+import util
+from conftest import ROOT, TINY
+
+pytestmark = pytest.mark.gpu
+
+
+def test_greedy_generation_through_the_entry_point(model_dirs):
+    import ninfer_amd
+    for name in ("A", "B"):
+        d = model_dirs[name]["float32"]
+        cfg, w = util.read_folder(d)
+        eng = ninfer_amd.Ninfer(d, max_context=96, prefill_chunk=16, num_sequences=3,
+                                dtype="float32", page_size=8)
+        prompts = [util.random_tokens(n, cfg["vocab_size"], 40 + n) for n in (5, 11, 17, 30)]
+        outs = eng.generate(prompts, ninfer_amd.SamplingParams.greedy(8), stop_ids=[])
+        for p, o in zip(prompts, outs):
+            assert o == plain_model.greedy_generate(w, cfg, p, 8)
+        assert eng.kv_pages()["free"] == eng.kv_pages()["total"]
+
+
+def test_sessions_like_the_reference_binding(model_dirs):
+    import ninfer_amd
+    d = model_dirs["A"]["float32"]
+    cfg, w = util.read_folder(d)
+    eng = ninfer_amd.Ninfer(d, max_context=64, prefill_chunk=4, num_sequences=2, dtype="float32")
+    toks = util.random_tokens(14, cfg["vocab_size"], 9)
+    ref = plain_model.forward(w, cfg, toks)
+    with eng.session() as s, eng.session() as t:
+        l1 = s.prefill(toks[:9])                       # cut into portions of 4 inside
+        assert s.length == 9 and l1.shape == (cfg["vocab_size"],)
+        torch.testing.assert_close(torch.from_numpy(l1), ref[8], atol=2e-5, rtol=1e-4)
+        t.prefill(toks[:3])
+        both = eng.decode_batch([s, t], [toks[9], toks[3]])
+        torch.testing.assert_close(torch.from_numpy(both[0]), ref[9], atol=2e-5, rtol=1e-4)
+        torch.testing.assert_close(torch.from_numpy(both[1]), ref[3], atol=2e-5, rtol=1e-4)
+        assert eng.sample(l1, temperature=0.0) == int(ref[8].argmax())
+        drawn = {eng.sample(l1, temperature=1.0, top_k=5, top_p=1.0, seed=sd) for sd in range(1, 40)}
+        assert drawn <= set(ref[8].topk(5).indices.tolist()) and len(drawn) > 1
+        s.reset()
+        assert s.length == 0
+    assert eng.vocab == cfg["vocab_size"] and eng.kv_bytes_per_token == 2 * 2 * 2 * 16 * 4
+
+
+def test_long_decoding_and_first_tokens(model_dirs):
+    """300 tokens decoded one by one after a one-token prompt (first tokens of a
+    sequence, many page edges, the window passing pages) equal the whole-sequence
+    logits of the plain implementation."""
+    from ninfer_amd import Chunk, EngineOptions, load_model
+    for dtype in ("float32", "bfloat16"):
+        d = model_dirs["B"][dtype]
+        cfg, w = util.read_folder(d)
+        _, w16 = util.read_folder(model_dirs["B"]["bfloat16"])
+        toks = util.safe_prompt(w16, cfg, 300, 4242)
+        ref = plain_model.forward(w, cfg, toks)
+        runner = load_model(d, EngineOptions(dtype=dtype, max_context=320, num_sequences=1,
+                                             page_size=16))
+        s = runner.open()
+        rows = [runner.step([Chunk(s, [t], [0])])[0].float().cpu() for t in toks]
+        got = torch.stack(rows)
+        bound = dict(atol=3e-5, rtol=1e-4) if dtype == "float32" else dict(atol=6e-2, rtol=5e-2)
+        torch.testing.assert_close(got, ref, **bound)
+        assert runner.cache.groups[1].window_freed >= (300 - 24) // 16
+
+
+def test_command_line(model_dirs):
+    d = model_dirs["A"]["float32"]
+    cfg, w = util.read_folder(d)
+    prompt = util.random_tokens(7, cfg["vocab_size"], 3)
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "ninfer"), d, "--prompt-ids",
+         ",".join(map(str, prompt)), "--random-prompts", "5,9", "--max-new", "6", "--temperature",
+         "0", "--dtype", "fp32", "--max-context", "64", "--prefill-chunk", "8", "--seed", "3"],
+        capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = proc.stdout.strip().splitlines()
+    assert len(lines) == 3
+    assert [int(x) for x in lines[0].split(",")] == plain_model.greedy_generate(w, cfg, prompt, 6)
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "ninfer"), d, "--no-such-flag"],
+                         capture_output=True, text=True, timeout=120)
+    assert bad.returncode != 0
+
+
+def test_toy_mixer_on_the_gpu(tmp_path):
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, load_model
+    toy.register()
+    d = str(tmp_path / "toy")
+    ninfer_amd.write_random_model(d, toy.TOY_CONFIG, 5, std=0.2)
+    cfg, w = util.read_folder(d)
+    runner = load_model(d, EngineOptions(dtype="float32", max_context=64, num_sequences=3))
+    reqs = {f"t{i}": util.random_tokens(n, 97, 60 + i) for i, n in enumerate([9, 21, 14, 30])}
+    ref = {k: toy.plain_forward(w, cfg, v) for k, v in reqs.items()}
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=3, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=2e-5, rtol=1e-4)
+
+
+@pytest.mark.parametrize("plan", [[(0, None), (1, 0), (2, None)],
+                                  [(0, None), (1, None), (1, None), (2, None)]])
+def test_layer_plan_on_the_gpu(model_dirs, plan):
+    from ninfer_amd import EngineOptions
+    from ninfer_amd.config import read_config_json
+    from ninfer_amd.engine import ModelRunner
+    from ninfer_amd.loading import build_spec
+    from ninfer_amd.models.spec import LayerCall
+    from ninfer_amd.weights import CheckpointSource
+    d = model_dirs["B"]["float32"]
+    cfg, w = util.read_folder(d)
+    _, spec = build_spec(read_config_json(d))
+    spec.set_plan([LayerCall(l, c) for l, c in plan])
+    runner = ModelRunner(spec, CheckpointSource(d),
+                         EngineOptions(dtype="float32", max_context=64, num_sequences=2, page_size=8))
+    toks = util.random_tokens(45, cfg["vocab_size"], 77)
+    ref = plain_model.forward(w, cfg, toks, plan=plan)
+    for sched in (util.schedule_whole("x", toks), util.schedule_portions("x", toks, 2)):
+        torch.testing.assert_close(util.run_schedule(runner, sched)["x"], ref, atol=2e-5, rtol=1e-4)

@@ -160,3 +160,71 @@ def run_schedule(runner, steps: List[Step]) -> Dict[str, torch.Tensor]:
         for rid in end:
             runner.close(slots.pop(rid))
     return {rid: torch.cat(v) for rid, v in rows.items()}
+
+
+class DictSource:
+    """A weight source over a dictionary of tensors (for parts built alone)."""
+
+    def __init__(self, tensors: Dict[str, torch.Tensor]):
+        self.tensors = tensors
+
+    def shapes(self):
+        return {k: tuple(v.shape) for k, v in self.tensors.items()}
+
+    def read(self, name: str) -> torch.Tensor:
+        return self.tensors[name]
+
+    def close(self) -> None:
+        pass
+
+
+def random_part_weights(part, seed: int, std: float = 0.2) -> Dict[str, torch.Tensor]:
+    """Random 32-bit tensors for everything a part (and its children) expects."""
+    from ninfer_amd.weights import RandomSource
+    src = RandomSource(part.all_tensor_specs(), seed, torch.float32, std=std)
+    return {n: src.read(n) for n in src.specs}
+
+
+def make_context(ops, act_dtype, seqs, device="cuda"):
+    """A StepContext for requests given as (first position, rows)."""
+    from ninfer_amd.parts import StepContext
+    positions, row_seq, row_start = [], [], []
+    for i, (p, q) in enumerate(seqs):
+        row_start.append(len(positions))
+        positions += list(range(p, p + q))
+        row_seq += [i] * q
+    row_start.append(len(positions))
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device=device)
+    return StepContext(
+        ops=ops, act_dtype=act_dtype, device=torch.device(device), T=len(positions), S=len(seqs),
+        tokens=dev([0] * len(positions)), positions=dev(positions), row_seq=dev(row_seq),
+        seq_slots=dev(list(range(len(seqs)))), seq_row_start=dev(row_start),
+        seq_qlen=dev([q for _, q in seqs]), seq_pos0=dev([p for p, _ in seqs]),
+        max_qlen=max(q for _, q in seqs), max_kv_len=max(p + q for p, q in seqs),
+        all_decode=all(q == 1 for _, q in seqs))
+
+
+def write_trace(steps: List[Step]) -> str:
+    """A schedule as the JSON lines bin/trace_run reads."""
+    lines = []
+    for i, (entries, end) in enumerate(steps):
+        lines.append(json.dumps({"step": i, "entries": [{"id": r, "tokens": t, "want": w}
+                                                        for r, t, w in entries], "end": end}))
+    return "\n".join(lines) + "\n"
+
+
+def read_trace_output(out_dir: str, steps: List[Step], vocab: int) -> Dict[str, torch.Tensor]:
+    """Logits per request (rows in position order) from the <step>.f32 files."""
+    import numpy as np
+    rows: Dict[str, List[torch.Tensor]] = {}
+    for i, (entries, _) in enumerate(steps):
+        wanted = sum(len(w) for _, _, w in entries)
+        if not wanted:
+            continue
+        arr = np.fromfile(os.path.join(out_dir, f"{i}.f32"), dtype="<f4").reshape(wanted, vocab)
+        o = 0
+        for r, _, w in entries:
+            if w:
+                rows.setdefault(r, []).append(torch.from_numpy(arr[o:o + len(w)].copy()))
+                o += len(w)
+    return {k: torch.cat(v) for k, v in rows.items()}
