@@ -18,13 +18,37 @@ __global__ void embed_kernel(const int* __restrict__ tokens, const T* __restrict
   for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_f32(src[i]);
 }
 
-// y = (x [+ delta]) * rsqrt(mean(.^2) + eps) * gain  (reference
+// A weighted sum of rows that a sparse feed-forward leaves to be added to the
+// residual: sum_j w[t,j] * y[t*k + j,:] + sigmoid(gate[t * gate_stride]) * shared[t,:]
+// (gate null: factor 1; shared null: no such term; y null: nothing).
+struct MoeSum {
+  const void* y;
+  const float* w;
+  const void* shared;
+  const float* gate;
+  int gate_stride;
+  int k;
+};
+
+template <typename T>
+__device__ __forceinline__ float moe_sum_at(const MoeSum& ms, int64_t t, int i, int H, float g) {
+  float acc = 0.f;
+  const T* y = (const T*)ms.y;
+  for (int j = 0; j < ms.k; ++j) acc += ms.w[t * ms.k + j] * to_f32(y[(t * ms.k + j) * H + i]);
+  if (ms.shared) acc += g * to_f32(((const T*)ms.shared)[t * H + i]);
+  return acc;
+}
+
+constexpr int kNormPerThread = 8;
+
+// y = (x [+ delta] [+ moe sum]) * rsqrt(mean(.^2) + eps) * gain  (reference
 // src/ops/kernels.hip:17-41 and :100-129). With rows == nullptr the sum is
 // written back to x; with rows the kernel reads row rows[i] and leaves x alone.
-// The reduction order depends only on H and the block size, never on the
-// number of rows.
+// Every thread keeps its (at most 8) elements in registers between the two
+// passes. The reduction order depends only on H and the block size, never on
+// the number of rows.
 template <typename T>
-__global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta,
+__global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta, MoeSum ms,
                                const float* __restrict__ gain, T* __restrict__ out,
                                const int* __restrict__ rows, int H, float eps) {
   __shared__ float red[16];
@@ -33,21 +57,32 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delt
   float* xr = x + r_in * H;
   const T* dr = delta ? delta + r_in * H : nullptr;
   T* orow = out + r_out * H;
+  float g = 1.f;
+  if (ms.y && ms.shared && ms.gate) g = 1.f / (1.f + expf(-ms.gate[r_in * ms.gate_stride]));
+  float vals[kNormPerThread];
   float acc = 0.f;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    float v = xr[i];
-    if (dr) v += to_f32(dr[i]);
+#pragma unroll
+  for (int c = 0; c < kNormPerThread; ++c) {
+    int i = threadIdx.x + c * blockDim.x;
+    float v = 0.f;
+    if (i < H) {
+      v = xr[i];
+      if (dr) v += to_f32(dr[i]);
+      if (ms.y) v += moe_sum_at<T>(ms, r_in, i, H, g);
+    }
+    vals[c] = v;
     acc += v * v;
   }
   float total = block_sum(acc, red);
   float inv = rsqrtf(total / (float)H + eps);
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    float v = xr[i];
-    if (dr) {
-      v += to_f32(dr[i]);
-      if (!rows) xr[i] = v;
+  const bool write_back = !rows && (dr || ms.y);
+#pragma unroll
+  for (int c = 0; c < kNormPerThread; ++c) {
+    int i = threadIdx.x + c * blockDim.x;
+    if (i < H) {
+      if (write_back) xr[i] = vals[c];
+      orow[i] = from_f32<T>(vals[c] * inv * gain[i]);
     }
-    orow[i] = from_f32<T>(v * inv * gain[i]);
   }
 }
 
@@ -109,14 +144,14 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
 template <typename T>
 __global__ void moe_combine_kernel(float* __restrict__ residual, const T* __restrict__ y,
                                    const float* __restrict__ w, const T* __restrict__ shared,
-                                   const float* __restrict__ gate, int H, int k) {
+                                   const float* __restrict__ gate, int gate_stride, int H, int k) {
   const int64_t t = blockIdx.x;
   const int i = blockIdx.y * blockDim.x + threadIdx.x;
   if (i >= H) return;
   float acc = 0.f;
   for (int j = 0; j < k; ++j) acc += w[t * k + j] * to_f32(y[(t * k + j) * H + i]);
   if (shared) {
-    float g = gate ? 1.f / (1.f + expf(-gate[t])) : 1.f;
+    float g = gate ? 1.f / (1.f + expf(-gate[t * gate_stride])) : 1.f;
     acc += g * to_f32(shared[t * H + i]);
   }
   residual[t * H + i] += acc;
@@ -162,17 +197,27 @@ extern "C" int ninfer_embed(const int* tokens, const void* table, float* out, in
   return 0;
 }
 
+// moe_* describe an optional weighted sum of rows added before the norm (all
+// null / 0: none): y [rows * k, H], w [rows, k], shared [rows, H], gate logits
+// with stride gate_stride.
 extern "C" int ninfer_rmsnorm(float* x, const void* delta, const float* gain, void* out,
                               const int* rows, int n_rows, int H, float eps, int dtype,
+                              const void* moe_y, const float* moe_w, const void* moe_shared,
+                              const float* moe_gate, int moe_gate_stride, int moe_k,
                               hipStream_t stream) {
   NINFER_REQUIRE(n_rows > 0 && H > 0, "rmsnorm: rows=%d H=%d must be positive", n_rows, H);
   NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "rmsnorm: unknown dtype %d", dtype);
-  int block = H >= 2048 ? 512 : 256;
+  NINFER_REQUIRE(H <= 1024 * kNormPerThread, "rmsnorm: width %d exceeds %d", H,
+                 1024 * kNormPerThread);
+  NINFER_REQUIRE(!moe_y || (moe_w && moe_k > 0), "rmsnorm: a row sum needs weights and k");
+  int block = ((H + kNormPerThread - 1) / kNormPerThread + 63) / 64 * 64;
+  if (block < 128) block = 128;
+  MoeSum ms{moe_y, moe_w, moe_shared, moe_gate, moe_gate_stride, moe_k};
   if (dtype == kF32)
-    rmsnorm_kernel<float><<<n_rows, block, 0, stream>>>(x, (const float*)delta, gain, (float*)out,
-                                                       rows, H, eps);
+    rmsnorm_kernel<float><<<n_rows, block, 0, stream>>>(x, (const float*)delta, ms, gain,
+                                                       (float*)out, rows, H, eps);
   else
-    rmsnorm_kernel<bf16><<<n_rows, block, 0, stream>>>(x, (const bf16*)delta, gain, (bf16*)out,
+    rmsnorm_kernel<bf16><<<n_rows, block, 0, stream>>>(x, (const bf16*)delta, ms, gain, (bf16*)out,
                                                       rows, H, eps);
   NINFER_LAUNCH_CHECK();
   return 0;
@@ -205,16 +250,16 @@ extern "C" int ninfer_rope_kv_write(void* qkv, const float* bias, const int* pos
 }
 
 extern "C" int ninfer_moe_combine(float* residual, const void* y, const float* w,
-                                  const void* shared, const float* gate, int T, int H, int k,
-                                  int dtype, hipStream_t stream) {
+                                  const void* shared, const float* gate, int gate_stride, int T,
+                                  int H, int k, int dtype, hipStream_t stream) {
   NINFER_REQUIRE(T > 0 && H > 0 && k > 0, "moe_combine: T=%d H=%d k=%d must be positive", T, H, k);
   NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "moe_combine: unknown dtype %d", dtype);
   if (dtype == kF32)
     moe_combine_kernel<float><<<dim3(T, (H + 255) / 256), 256, 0, stream>>>(residual, (const float*)y, w,
-                                                    (const float*)shared, gate, H, k);
+                                                    (const float*)shared, gate, gate_stride, H, k);
   else
     moe_combine_kernel<bf16><<<dim3(T, (H + 255) / 256), 256, 0, stream>>>(residual, (const bf16*)y, w,
-                                                   (const bf16*)shared, gate, H, k);
+                                                   (const bf16*)shared, gate, gate_stride, H, k);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

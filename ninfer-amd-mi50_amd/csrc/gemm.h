@@ -16,6 +16,9 @@ struct GemmArgs {
   const int* offsets;    // [groups + 1] sorted-row ranges per group, or null (dense)
   const int* a_index;    // sorted row -> a_index[r] / a_div is the row of A, or null
   const int* c_index;    // sorted row -> row of C, or null
+  const int* tiles16;    // grouped: {expert, first row, end row, 0} per 16-row tile, or null
+  const int* tiles64;    // the same for 64-row tiles
+  const int* tile_counts;  // {number of 16-row tiles, number of 64-row tiles}
   int64_t w_group_stride;  // elements between the weights of two groups
   int M;                 // rows (dense) or number of sorted rows (grouped)
   int N;                 // output features (per SwiGLU half)
@@ -68,6 +71,20 @@ __device__ inline bool find_tile(const int* __restrict__ offsets, int groups, in
   }
   __syncthreads();
   return info[2] >= 0;
+}
+
+// The rows of tile `ti`: from the tile list routing wrote (one 16-byte load),
+// or by scanning the offsets when there is no list. `info` is 3 ints of LDS.
+__device__ inline bool grouped_tile(const GemmArgs& a, const int* __restrict__ tiles, int which,
+                                    int tile_rows, int ti, int* info) {
+  if (!tiles) return find_tile(a.offsets, a.groups, tile_rows, ti, info);
+  int count = a.tile_counts[which];
+  int4 t = ((const int4*)tiles)[ti];
+  if (ti >= count) return false;
+  info[0] = t.y;
+  info[1] = t.z;
+  info[2] = t.x;
+  return true;
 }
 
 int gemm_check(const GemmArgs& a);

@@ -33,7 +33,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a) {
   __shared__ int tile_info[3];
 
   int row0, row_end, group = 0;
-  if (a.offsets) {
+  if (a.offsets && a.tiles16) {
+    // every thread reads the tile's entry itself: no barrier before the first loads
+    int count = a.tile_counts[0];
+    int4 t = ((const int4*)a.tiles16)[blockIdx.y];
+    if ((int)blockIdx.y >= count) return;
+    group = t.x;
+    row0 = t.y;
+    row_end = t.z;
+  } else if (a.offsets) {
     if (!find_tile(a.offsets, a.groups, SM, blockIdx.y, tile_info)) return;
     group = tile_info[2];
     row0 = tile_info[0];

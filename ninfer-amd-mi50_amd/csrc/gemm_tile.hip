@@ -35,7 +35,8 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(GemmArgs a) {
 
   int row0, row_end, group = 0;
   if (a.offsets) {
-    if (!find_tile(a.offsets, a.groups, TM, blockIdx.x, tile_info)) return;
+    if (!grouped_tile(a, a.tiles64, 1, TM, blockIdx.x, tile_info)) return;
+    __syncthreads();
     group = tile_info[2];
     row0 = tile_info[0];
     row_end = tile_info[1];

@@ -10,12 +10,22 @@ constexpr int kMaxExpertsPerLane = 16;  // up to 1024 experts
 // One wave per row. p = softmax(logits) over all E; the k largest p in
 // descending order, ties to the lower expert index; weights p (renorm: p / sum
 // of the chosen). Reference formulas: src/ops/moe.hip:65-82.
+__device__ __forceinline__ void route_row(const float* __restrict__ row, int E, int k, int renorm,
+                                          int* __restrict__ ids, float* __restrict__ wts, int lane);
+
 __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict__ logits, int ld,
                                                          int E, int k, int renorm,
                                                          int* __restrict__ ids,
                                                          float* __restrict__ wts) {
-  const int t = blockIdx.x, lane = threadIdx.x;
-  const float* row = logits + (int64_t)t * ld;
+  const int t = blockIdx.x;
+  route_row(logits + (int64_t)t * ld, E, k, renorm, ids + (int64_t)t * k, wts + (int64_t)t * k,
+            threadIdx.x);
+}
+
+// One row's softmax + top-k by one wave (shared by the two routing kernels).
+__device__ __forceinline__ void route_row(const float* __restrict__ row, int E, int k, int renorm,
+                                          int* __restrict__ ids, float* __restrict__ wts,
+                                          int lane) {
   float p[kMaxExpertsPerLane];
   float m = -INFINITY;
 #pragma unroll
@@ -38,8 +48,7 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict
     int e = lane + i * 64;
     p[i] = e < E ? p[i] / sum : -1.f;  // -1 marks "not a candidate"
   }
-  float chosen_sum = 0.f;
-  float my_w = 0.f;
+  float chosen_sum = 0.f, my_w = 0.f;
   int my_id = 0;
   for (int j = 0; j < k; ++j) {
     float best = -1.f;
@@ -71,34 +80,74 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict
     }
   }
   if (lane < k) {
-    ids[(int64_t)t * k + lane] = my_id;
-    wts[(int64_t)t * k + lane] = renorm ? my_w / chosen_sum : my_w;
+    ids[lane] = my_id;
+    wts[lane] = renorm ? my_w / chosen_sum : my_w;
   }
 }
 
-// Rows grouped by expert: offsets[e] .. offsets[e+1] are the positions in
-// `order` of the flat (row, choice) indices routed to expert e. One block; the
-// order inside an expert is not fixed (atomic cursors), which no result depends
-// on: every routed row is computed on its own and written back by its index.
-__global__ void moe_align_kernel(const int* __restrict__ ids, int n, int E,
-                                 int* __restrict__ offsets, int* __restrict__ order) {
-  extern __shared__ int cnt[];  // [E] counts, then cursors
+// Rows grouped by expert, by one block: offsets[e] .. offsets[e+1] are the
+// positions in `order` of the flat (row, choice) indices routed to expert e.
+// The order inside an expert is not fixed (atomic cursors), which no result
+// depends on: every routed row is computed on its own and written back by its
+// index. Also writes the lists of 16-row and 64-row tiles the grouped products
+// walk: {expert, first row, end row, 0} per tile, and their counts.
+// `cnt` is E + 1 ints of LDS; ids may be in LDS or global memory.
+__device__ void align_block(const int* ids, int n, int E, int* __restrict__ offsets,
+                            int* __restrict__ order, int* __restrict__ tiles16,
+                            int* __restrict__ tiles64, int* __restrict__ tile_counts, int* cnt) {
   for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cnt[ids[i]], 1);
   __syncthreads();
   if (threadIdx.x == 0) {
-    int run = 0;
+    int run = 0, n16 = 0, n64 = 0;
     for (int e = 0; e < E; ++e) {
       int c = cnt[e];
       offsets[e] = run;
       cnt[e] = run;
+      if (tiles16) {
+        for (int r = run; r < run + c; r += 16) {
+          ((int4*)tiles16)[n16++] = make_int4(e, r, run + c, 0);
+        }
+        for (int r = run; r < run + c; r += 64) {
+          ((int4*)tiles64)[n64++] = make_int4(e, r, run + c, 0);
+        }
+      }
       run += c;
     }
     offsets[E] = run;
+    if (tile_counts) {
+      tile_counts[0] = n16;
+      tile_counts[1] = n64;
+    }
   }
   __syncthreads();
   for (int i = threadIdx.x; i < n; i += blockDim.x) order[atomicAdd(&cnt[ids[i]], 1)] = i;
+}
+
+__global__ void moe_align_kernel(const int* __restrict__ ids, int n, int E,
+                                 int* __restrict__ offsets, int* __restrict__ order,
+                                 int* __restrict__ tiles16, int* __restrict__ tiles64,
+                                 int* __restrict__ tile_counts) {
+  extern __shared__ int cnt[];
+  align_block(ids, n, E, offsets, order, tiles16, tiles64, tile_counts, cnt);
+}
+
+// Few rows (decode): softmax + top-k of every row and the grouping by expert
+// in one launch of one block.
+__global__ __launch_bounds__(1024) void moe_route_small_kernel(
+    const float* __restrict__ logits, int ld, int T, int E, int k, int renorm,
+    int* __restrict__ ids, float* __restrict__ wts, int* __restrict__ offsets,
+    int* __restrict__ order, int* __restrict__ tiles16, int* __restrict__ tiles64,
+    int* __restrict__ tile_counts) {
+  extern __shared__ int cnt[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  for (int t = wave; t < T; t += waves)
+    route_row(logits + (int64_t)t * ld, E, k, renorm, ids + (int64_t)t * k, wts + (int64_t)t * k,
+              lane);
+  __threadfence();
+  __syncthreads();  // the ids written above are read below by other threads of this block
+  align_block(ids, T * k, E, offsets, order, tiles16, tiles64, tile_counts, cnt);
 }
 
 }  // namespace ninfer
@@ -117,11 +166,36 @@ extern "C" int ninfer_router_topk(const float* logits, int ld, int T, int E, int
   return 0;
 }
 
+// tiles16 / tiles64 / tile_counts may be null (no tile lists). tiles16 holds
+// 4 ints for each of up to min(n, n / 16 + E) tiles, tiles64 for n / 64 + E.
 extern "C" int ninfer_moe_align(const int* ids, int n, int E, int* offsets, int* order,
+                                int* tiles16, int* tiles64, int* tile_counts,
                                 hipStream_t stream) {
   NINFER_REQUIRE(n > 0 && E > 0, "moe_align: n=%d E=%d must be positive", n, E);
   NINFER_REQUIRE(E <= 8192, "moe_align: %d experts exceed 8192", E);
-  moe_align_kernel<<<1, 1024, E * sizeof(int), stream>>>(ids, n, E, offsets, order);
+  NINFER_REQUIRE((!tiles16) == (!tiles64) && (!tiles16) == (!tile_counts),
+                 "moe_align: tile lists come together or not at all");
+  moe_align_kernel<<<1, 1024, (E + 1) * sizeof(int), stream>>>(ids, n, E, offsets, order, tiles16,
+                                                             tiles64, tile_counts);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+// Routing of few rows in one launch: top-k and grouping (T <= 256).
+extern "C" int ninfer_moe_route_small(const float* logits, int ld, int T, int E, int k,
+                                      int renorm, int* ids, float* wts, int* offsets, int* order,
+                                      int* tiles16, int* tiles64, int* tile_counts,
+                                      hipStream_t stream) {
+  NINFER_REQUIRE(T > 0 && T <= 256, "moe_route_small: T=%d not in [1, 256]", T);
+  NINFER_REQUIRE(E > 0 && E <= 64 * kMaxExpertsPerLane, "moe_route_small: %d experts exceed %d", E,
+                 64 * kMaxExpertsPerLane);
+  NINFER_REQUIRE(k >= 1 && k <= E && k <= 64, "moe_route_small: k=%d not in [1, min(%d, 64)]", k, E);
+  NINFER_REQUIRE(ld >= E, "moe_route_small: row stride %d < %d experts", ld, E);
+  NINFER_REQUIRE((!tiles16) == (!tiles64) && (!tiles16) == (!tile_counts),
+                 "moe_route_small: tile lists come together or not at all");
+  int threads = T >= 16 ? 1024 : 64 * T;
+  moe_route_small_kernel<<<1, threads, (E + 1) * sizeof(int), stream>>>(
+      logits, ld, T, E, k, renorm, ids, wts, offsets, order, tiles16, tiles64, tile_counts);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

@@ -26,7 +26,8 @@ class _GemmArgs(ctypes.Structure):
     _fields_ = [("A", ctypes.c_void_p), ("W", ctypes.c_void_p), ("C", ctypes.c_void_p),
                 ("bias", ctypes.c_void_p), ("offsets", ctypes.c_void_p),
                 ("a_index", ctypes.c_void_p), ("c_index", ctypes.c_void_p),
-                ("w_group_stride", ctypes.c_int64),
+                ("tiles16", ctypes.c_void_p), ("tiles64", ctypes.c_void_p),
+                ("tile_counts", ctypes.c_void_p), ("w_group_stride", ctypes.c_int64),
                 ("M", ctypes.c_int), ("N", ctypes.c_int), ("K", ctypes.c_int),
                 ("lda", ctypes.c_int), ("ldc", ctypes.c_int), ("groups", ctypes.c_int),
                 ("a_div", ctypes.c_int), ("in_dtype", ctypes.c_int), ("out_dtype", ctypes.c_int),
@@ -100,7 +101,9 @@ class HipOps:
             ctypes.c_void_p(out.data_ptr()), tokens.shape[0], table.shape[1], _DT[table.dtype],
             self._stream()))
 
-    def rmsnorm(self, x, gain, eps, out, delta=None, rows=None):
+    def rmsnorm(self, x, gain, eps, out, delta=None, rows=None, rows_sum=None):
+        """out = norm(x [+ delta] [+ rows_sum]); `rows_sum` is a weighted sum of
+        rows (an object with y, weights, shared, gate) added on the fly."""
         _dev(x, "x", torch.float32, 2)
         _dev(gain, "gain", torch.float32, 1)
         _dev(out, "out", dims=2)
@@ -114,11 +117,33 @@ class HipOps:
             _need(out.shape[0] == rows.shape[0], "rmsnorm: out has the wrong number of rows")
         else:
             _need(out.shape[0] == x.shape[0], "rmsnorm: out has the wrong number of rows")
+        my, mw, msh, mg, mgs, mk = None, None, None, None, 0, 0
+        if rows_sum is not None:
+            mk, mgs = self._check_rows_sum(rows_sum, x.shape[0], h, out.dtype)
+            my, mw = rows_sum.y.data_ptr(), rows_sum.weights.data_ptr()
+            msh, mg = _ptr(rows_sum.shared), _ptr(rows_sum.gate)
         self._ok(self.lib.ninfer_rmsnorm(
             ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(_ptr(delta)),
             ctypes.c_void_p(gain.data_ptr()), ctypes.c_void_p(out.data_ptr()),
             ctypes.c_void_p(_ptr(rows)), out.shape[0], h, ctypes.c_float(eps), _DT[out.dtype],
-            self._stream()))
+            ctypes.c_void_p(my), ctypes.c_void_p(mw), ctypes.c_void_p(msh), ctypes.c_void_p(mg),
+            mgs, mk, self._stream()))
+
+    @staticmethod
+    def _check_rows_sum(rs, t, h, dtype):
+        _dev(rs.y, "y", dtype, 2)
+        _dev(rs.weights, "weights", torch.float32, 2)
+        k = rs.weights.shape[1]
+        _need(rs.weights.shape[0] == t and rs.y.shape == (t * k, h), "row sum: shapes differ")
+        stride = 0
+        if rs.shared is not None:
+            _dev(rs.shared, "shared", dtype, 2)
+            _need(rs.shared.shape == (t, h), "row sum: shared has the wrong shape")
+        if rs.gate is not None:
+            _need(rs.gate.is_cuda and rs.gate.dtype == torch.float32 and rs.gate.dim() == 1
+                  and rs.gate.shape[0] == t, "row sum: gate must be 32-bit [rows] on the GPU")
+            stride = rs.gate.stride(0)
+        return k, stride
 
     def rope_kv_write(self, qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv, head_dim,
                       k_pool, v_pool, block_table, page_size, write_kv=True):
@@ -159,19 +184,27 @@ class HipOps:
         if shared is not None:
             _dev(shared, "shared", y.dtype, 2)
             _need(shared.shape == (t, h), "moe_combine: shared has the wrong shape")
+        stride = 1
         if gate is not None:
-            _dev(gate, "gate", torch.float32)
-            _need(gate.numel() == t, "moe_combine: gate has the wrong size")
+            _need(gate.is_cuda and gate.dtype == torch.float32 and gate.numel() == t,
+                  "moe_combine: gate must be 32-bit with one value per row, on the GPU")
+            gate = gate.reshape(t)
+            stride = gate.stride(0)
         self._ok(self.lib.ninfer_moe_combine(
             ctypes.c_void_p(residual.data_ptr()), ctypes.c_void_p(y.data_ptr()),
             ctypes.c_void_p(wts.data_ptr()), ctypes.c_void_p(_ptr(shared)),
-            ctypes.c_void_p(_ptr(gate)), t, h, k, _DT[y.dtype], self._stream()))
+            ctypes.c_void_p(_ptr(gate)), stride, t, h, k, _DT[y.dtype], self._stream()))
 
     # ---- products ---------------------------------------------------------------
     def _gemm(self, a, w, c, *, n, k, m, bias=None, offsets=None, a_index=None, c_index=None,
-              a_div=1, groups=1, epilogue=0, w_group_stride=0):
+              a_div=1, groups=1, epilogue=0, w_group_stride=0, tiles=None):
+        t16 = t64 = tc = None
+        if tiles is not None and tiles.tiles16 is not None:
+            t16, t64, tc = tiles.tiles16.data_ptr(), tiles.tiles64.data_ptr(), \
+                tiles.tile_counts.data_ptr()
         args = _GemmArgs(a.data_ptr(), w.data_ptr(), c.data_ptr(), _ptr(bias), _ptr(offsets),
-                         _ptr(a_index), _ptr(c_index), w_group_stride, m, n, k, a.shape[1],
+                         _ptr(a_index), _ptr(c_index), t16, t64, tc, w_group_stride, m, n, k,
+                         a.shape[1],
                          c.shape[1], groups, a_div, _DT[a.dtype], _DT[c.dtype], epilogue)
         self._ok(self.lib.ninfer_gemm(ctypes.byref(args), 1 if self.force_generic else 0,
                                       self._stream()))
@@ -223,7 +256,7 @@ class HipOps:
             return
         self._gemm(x, w_gate_up, out, m=x.shape[0], n=inner, k=x.shape[1], epilogue=1)
 
-    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out):
+    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None):
         """out[r] = swiglu of row order[r] // top_k of x by the expert that owns
         sorted position r."""
         _dev(x, "x", dims=2)
@@ -238,9 +271,9 @@ class HipOps:
         _need(offsets.shape[0] == e + 1, "grouped_swiglu: offsets size")
         _need(n == x.shape[0] * top_k and out.shape == (n, inner), "grouped_swiglu: row counts")
         self._gemm(x, w_gate_up, out, m=n, n=inner, k=h, offsets=offsets, a_index=order,
-                   a_div=top_k, groups=e, epilogue=1, w_group_stride=two_i * h)
+                   a_div=top_k, groups=e, epilogue=1, w_group_stride=two_i * h, tiles=tiles)
 
-    def grouped_down(self, h, w_down, offsets, order, out):
+    def grouped_down(self, h, w_down, offsets, order, out, tiles=None):
         """out[order[r]] = h[r] Wd_e^T for the expert e that owns sorted position r."""
         _dev(h, "h", dims=2)
         _dev(w_down, "w_down", h.dtype, 3)
@@ -252,7 +285,7 @@ class HipOps:
         _need(inner == h.shape[1] and h.shape[0] == n, "grouped_down: input shape")
         _need(out.shape == (n, hidden) and offsets.shape[0] == e + 1, "grouped_down: shapes")
         self._gemm(h, w_down, out, m=n, n=hidden, k=inner, offsets=offsets, c_index=order,
-                   groups=e, w_group_stride=hidden * inner)
+                   groups=e, w_group_stride=hidden * inner, tiles=tiles)
 
     # ---- routing ------------------------------------------------------------------
     def router_topk(self, logits, experts, top_k, renorm, ids, wts):
@@ -266,16 +299,53 @@ class HipOps:
             1 if renorm else 0, ctypes.c_void_p(ids.data_ptr()), ctypes.c_void_p(wts.data_ptr()),
             self._stream()))
 
-    def moe_align(self, ids, experts, offsets, order):
+    def _tile_ptrs(self, tiles, n, experts):
+        if tiles is None or tiles.tiles16 is None:
+            return None, None, None
+        _dev(tiles.tiles16, "tiles16", torch.int32, 2)
+        _dev(tiles.tiles64, "tiles64", torch.int32, 2)
+        _dev(tiles.tile_counts, "tile_counts", torch.int32, 1)
+        _need(tiles.tiles16.shape == (min(n, n // 16 + experts), 4)
+              and tiles.tiles64.shape == (n // 64 + experts, 4) and tiles.tile_counts.shape[0] == 2,
+              "routing: tile lists have the wrong sizes")
+        return tiles.tiles16.data_ptr(), tiles.tiles64.data_ptr(), tiles.tile_counts.data_ptr()
+
+    def moe_align(self, ids, experts, offsets, order, tiles=None):
         _dev(ids, "ids", torch.int32)
         _dev(offsets, "offsets", torch.int32, 1)
         _dev(order, "order", torch.int32, 1)
         _need(offsets.shape[0] == experts + 1 and order.shape[0] == ids.numel(),
               "moe_align: output sizes")
+        t16, t64, tc = self._tile_ptrs(tiles, ids.numel(), experts)
         self._ok(self.lib.ninfer_moe_align(
             ctypes.c_void_p(ids.data_ptr()), ids.numel(), experts,
             ctypes.c_void_p(offsets.data_ptr()), ctypes.c_void_p(order.data_ptr()),
-            self._stream()))
+            ctypes.c_void_p(t16), ctypes.c_void_p(t64), ctypes.c_void_p(tc), self._stream()))
+
+    def moe_route(self, logits, experts, top_k, renorm, r):
+        """Softmax + top-k per row and the grouping by expert, into the routing
+        record `r` (ids, weights, offsets, order, tile lists): one launch for up
+        to 256 rows, two for more."""
+        t = logits.shape[0]
+        if t > 256:
+            self.router_topk(logits, experts, top_k, renorm, r.ids, r.weights)
+            self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r)
+            return
+        _dev(logits, "logits", torch.float32, 2)
+        _dev(r.ids, "ids", torch.int32, 2)
+        _dev(r.weights, "weights", torch.float32, 2)
+        _dev(r.offsets, "offsets", torch.int32, 1)
+        _dev(r.order, "order", torch.int32, 1)
+        _need(r.ids.shape == (t, top_k) and r.weights.shape == (t, top_k)
+              and r.offsets.shape[0] == experts + 1 and r.order.shape[0] == t * top_k,
+              "moe_route: output sizes")
+        t16, t64, tc = self._tile_ptrs(r, t * top_k, experts)
+        self._ok(self.lib.ninfer_moe_route_small(
+            ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, experts, top_k,
+            1 if renorm else 0, ctypes.c_void_p(r.ids.data_ptr()),
+            ctypes.c_void_p(r.weights.data_ptr()), ctypes.c_void_p(r.offsets.data_ptr()),
+            ctypes.c_void_p(r.order.data_ptr()), ctypes.c_void_p(t16), ctypes.c_void_p(t64),
+            ctypes.c_void_p(tc), self._stream()))
 
     # ---- attention ------------------------------------------------------------------
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,

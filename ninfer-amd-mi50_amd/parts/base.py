@@ -78,6 +78,31 @@ class StepContext:
         return torch.empty(shape, dtype=dtype or self.act_dtype, device=self.device)
 
 
+@dataclass
+class PendingRows:
+    """A weighted sum of rows that a part leaves to be added to the residual by
+    whoever comes next (a norm's kernel adds it on the fly):
+    sum_j weights[t, j] * y[t * k + j, :] + sigmoid(gate[t]) * shared[t, :].
+    `shared` and `gate` may be None (no such term / factor 1). `gate` is a
+    32-bit view [T] that may be strided."""
+    y: torch.Tensor
+    weights: torch.Tensor
+    shared: Optional[torch.Tensor] = None
+    gate: Optional[torch.Tensor] = None
+
+    def add_to(self, ctx: "StepContext", residual: torch.Tensor) -> None:
+        ctx.ops.moe_combine(residual, self.y, self.weights, self.shared, self.gate)
+
+
+def settle(ctx: "StepContext", residual: torch.Tensor, pending) -> Optional[torch.Tensor]:
+    """For parts that take only plain rows: a PendingRows is added into the
+    residual now; a tensor (or None) is handed back unchanged."""
+    if isinstance(pending, PendingRows):
+        pending.add_to(ctx, residual)
+        return None
+    return pending
+
+
 class WeightBinder:
     """Reads tensors by name from a weight source and places them on the
     device: matrices in the compute dtype, gains and biases in 32-bit."""
@@ -127,7 +152,9 @@ class Part:
 
 
 class Norm(Part):
-    """y = norm(residual [+ pending]); the sum is kept in `residual` (32-bit)."""
+    """y = norm(residual [+ pending]); the sum is kept in `residual` (32-bit).
+    `pending` is rows [T, hidden], a PendingRows, or None (a norm that cannot
+    add a PendingRows on the fly calls `settle` first)."""
 
     def forward(self, ctx: StepContext, residual: torch.Tensor,
                 pending: Optional[torch.Tensor]) -> torch.Tensor:
@@ -170,8 +197,9 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """Row-wise transform. `forward` returns rows to add to the residual, or
-    None if it has already added its result to `residual` itself."""
+    """Row-wise transform. `forward` returns what is to be added to the
+    residual: rows [T, hidden], a PendingRows, or None if it has already added
+    its result to `residual` itself."""
 
     def forward(self, ctx: StepContext, x: torch.Tensor, residual: torch.Tensor
                 ) -> Optional[torch.Tensor]:

@@ -19,7 +19,7 @@ import torch
 
 from ..registry import register_part
 from ..weights.source import TensorSpec
-from .base import FeedForward, Part, StepContext, WeightBinder
+from .base import FeedForward, Part, PendingRows, StepContext, WeightBinder
 from .mlp import SwiGLU
 
 
@@ -40,14 +40,33 @@ class SoftmaxTopKRouter(Part):
     def bind(self, w: WeightBinder) -> None:
         self.weight = w.matrix(self.prefix + "weight")
 
-    def route(self, ctx: StepContext, x: torch.Tensor):
-        t = x.shape[0]
-        logits = ctx.empty((t, self.experts), torch.float32)
-        ctx.ops.linear(x, self.weight, logits)
-        ids = ctx.empty((t, self.top_k), torch.int32)
-        wts = ctx.empty((t, self.top_k), torch.float32)
-        ctx.ops.router_topk(logits, self.experts, self.top_k, self.renorm, ids, wts)
-        return ids, wts
+    def logits(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
+        out = ctx.empty((x.shape[0], self.experts), torch.float32)
+        ctx.ops.linear(x, self.weight, out)
+        return out
+
+    def route(self, ctx: StepContext, logits: torch.Tensor) -> "Routing":
+        """Choose experts from router logits [T, >= experts] (more columns are
+        ignored) and group the routed rows by expert, all on the device."""
+        t, k, e = logits.shape[0], self.top_k, self.experts
+        n = t * k
+        r = Routing(ids=ctx.empty((t, k), torch.int32), weights=ctx.empty((t, k), torch.float32),
+                    offsets=ctx.empty((e + 1,), torch.int32), order=ctx.empty((n,), torch.int32),
+                    tiles16=ctx.empty((min(n, n // 16 + e), 4), torch.int32),
+                    tiles64=ctx.empty((n // 64 + e, 4), torch.int32),
+                    tile_counts=ctx.empty((2,), torch.int32))
+        ctx.ops.moe_route(logits, e, k, self.renorm, r)
+        return r
+
+
+class Routing:
+    """What routing leaves on the device: chosen experts and weights per row,
+    the (row, choice) indices grouped by expert (`order`, `offsets`), and the
+    lists of 16-row and 64-row tiles the grouped products walk."""
+
+    def __init__(self, ids, weights, offsets, order, tiles16=None, tiles64=None, tile_counts=None):
+        self.ids, self.weights, self.offsets, self.order = ids, weights, offsets, order
+        self.tiles16, self.tiles64, self.tile_counts = tiles16, tiles64, tile_counts
 
 
 class RoutedExperts(Part):
@@ -83,16 +102,14 @@ class RoutedExperts(Part):
             w.matrix_into(p + "up_proj.weight", self.w_gate_up[e, i:])
             w.matrix_into(p + "down_proj.weight", self.w_down[e])
 
-    def run(self, ctx: StepContext, x: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    def run(self, ctx: StepContext, x: torch.Tensor, routing: "Routing") -> torch.Tensor:
         """Expert outputs [T*k, hidden], row t*k + j for the j-th choice of row t."""
-        t, k = ids.shape
-        offsets = ctx.empty((self.experts + 1,), torch.int32)
-        order = ctx.empty((t * k,), torch.int32)
-        ctx.ops.moe_align(ids, self.experts, offsets, order)
+        t, k = routing.ids.shape
         h = ctx.empty((t * k, self.inner))
-        ctx.ops.grouped_swiglu(x, self.w_gate_up, offsets, order, k, h)
+        ctx.ops.grouped_swiglu(x, self.w_gate_up, routing.offsets, routing.order, k, h,
+                               tiles=routing)
         y = ctx.empty((t * k, self.hidden))
-        ctx.ops.grouped_down(h, self.w_down, offsets, order, y)
+        ctx.ops.grouped_down(h, self.w_down, routing.offsets, routing.order, y, tiles=routing)
         return y
 
 
@@ -121,17 +138,30 @@ class SparseMoE(FeedForward):
         if self.shared is not None:
             self.shared_gate = w.matrix(self.prefix + "shared_expert_gate.weight")
 
+    def bind_all(self, w: WeightBinder) -> None:
+        super().bind_all(w)
+        if self.shared is not None:
+            # one product gives the router logits and the shared expert's gate logit
+            e = self.router.experts
+            self.router_and_gate = torch.cat([self.router.weight, self.shared_gate])
+            self.router.weight = self.router_and_gate[:e]
+            self.shared_gate = self.router_and_gate[e:]
+
     def forward(self, ctx: StepContext, x, residual):
-        ids, wts = self.router.route(ctx, x)
-        self.last_ids = ids
-        y = self.experts.run(ctx, x, ids)
         shared = gate = None
         if self.shared is not None:
+            logits = ctx.empty((x.shape[0], self.router.experts + 1), torch.float32)
+            ctx.ops.linear(x, self.router_and_gate, logits)
+            gate = logits[:, self.router.experts]
+        else:
+            logits = self.router.logits(ctx, x)
+        routing = self.router.route(ctx, logits)
+        self.last_ids = routing.ids
+        y = self.experts.run(ctx, x, routing)
+        if self.shared is not None:
             shared = self.shared.run(ctx, x)
-            gate = ctx.empty((x.shape[0], 1), torch.float32)
-            ctx.ops.linear(x, self.shared_gate, gate)
-        ctx.ops.moe_combine(residual, y, wts, shared, gate)
-        return None
+        # not added here: the next norm's kernel adds it to the residual on the fly
+        return PendingRows(y, routing.weights, shared, gate)
 
 
 register_part("feed_forward", "sparse_moe", SparseMoE)

@@ -12,7 +12,7 @@ import torch
 
 from ..registry import register_part
 from ..weights.source import TensorSpec
-from .base import Norm, StepContext, WeightBinder
+from .base import Norm, PendingRows, StepContext, WeightBinder
 
 
 class RMSNorm(Norm):
@@ -30,12 +30,18 @@ class RMSNorm(Norm):
 
     def forward(self, ctx: StepContext, residual, pending):
         out = ctx.empty((residual.shape[0], self.size))
-        ctx.ops.rmsnorm(residual, self.gain, self.eps, out, delta=pending)
+        if isinstance(pending, PendingRows):
+            ctx.ops.rmsnorm(residual, self.gain, self.eps, out, rows_sum=pending)
+        else:
+            ctx.ops.rmsnorm(residual, self.gain, self.eps, out, delta=pending)
         return out
 
     def forward_rows(self, ctx: StepContext, residual, rows, pending=None):
         out = ctx.empty((rows.shape[0], self.size))
-        ctx.ops.rmsnorm(residual, self.gain, self.eps, out, delta=pending, rows=rows)
+        if isinstance(pending, PendingRows):
+            ctx.ops.rmsnorm(residual, self.gain, self.eps, out, rows_sum=pending, rows=rows)
+        else:
+            ctx.ops.rmsnorm(residual, self.gain, self.eps, out, delta=pending, rows=rows)
         return out
 
 

@@ -24,15 +24,22 @@ class PlainOps:
     def embed(self, tokens, table, out):
         out.copy_(_f(table[tokens.long()]))
 
-    def rmsnorm(self, x, gain, eps, out, delta=None, rows=None):
+    def rmsnorm(self, x, gain, eps, out, delta=None, rows=None, rows_sum=None):
+        extra = None
+        if delta is not None:
+            extra = _f(delta)
+        if rows_sum is not None:
+            add = torch.zeros_like(x)
+            self.moe_combine(add, rows_sum.y, rows_sum.weights, rows_sum.shared, rows_sum.gate)
+            extra = add if extra is None else extra + add
         if rows is None:
-            if delta is not None:
-                x += _f(delta)
+            if extra is not None:
+                x += extra
             v = x
         else:
             v = x[rows.long()]
-            if delta is not None:
-                v = v + _f(delta[rows.long()])
+            if extra is not None:
+                v = v + extra[rows.long()]
         ms = (v * v).sum(-1, keepdim=True) / v.shape[-1]
         out.copy_((v * torch.rsqrt(ms + eps) * gain).to(out.dtype))
 
@@ -82,7 +89,7 @@ class PlainOps:
         u = _f(x) @ _f(w_gate_up[inner:]).T
         out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
 
-    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out):
+    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None):
         e, two_i, _ = w_gate_up.shape
         inner = two_i // 2
         off = offsets.tolist()
@@ -95,7 +102,7 @@ class PlainOps:
             uu = xs @ _f(w_gate_up[g, inner:]).T
             out[off[g]:off[g + 1]] = (gg / (1 + torch.exp(-gg)) * uu).to(out.dtype)
 
-    def grouped_down(self, h, w_down, offsets, order, out):
+    def grouped_down(self, h, w_down, offsets, order, out, tiles=None):
         e = w_down.shape[0]
         off = offsets.tolist()
         for g in range(e):
@@ -119,12 +126,24 @@ class PlainOps:
         if renorm:
             wts /= wts.sum(-1, keepdim=True)
 
-    def moe_align(self, ids, experts, offsets, order):
+    def moe_align(self, ids, experts, offsets, order, tiles=None):
         flat = ids.reshape(-1).long()
         counts = torch.bincount(flat, minlength=experts)
         offsets[0] = 0
         offsets[1:] = torch.cumsum(counts, 0).to(torch.int32)
         order.copy_(torch.sort(flat, stable=True).indices.to(torch.int32))
+        if tiles is not None and tiles.tiles16 is not None:
+            off = offsets.tolist()
+            for size, out in ((16, tiles.tiles16), (64, tiles.tiles64)):
+                lst = [[e, r, off[e + 1], 0] for e in range(experts)
+                       for r in range(off[e], off[e + 1], size)]
+                if lst:
+                    out[:len(lst)] = torch.tensor(lst, dtype=torch.int32, device=out.device)
+                tiles.tile_counts[0 if size == 16 else 1] = len(lst)
+
+    def moe_route(self, logits, experts, top_k, renorm, r):
+        self.router_topk(logits, experts, top_k, renorm, r.ids, r.weights)
+        self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r)
 
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,
                         page_size, window, scale, out):

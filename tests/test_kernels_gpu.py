@@ -170,6 +170,20 @@ def test_router_align_experts_combine(ops_mode, gen, dtype, t, e, k, h, inner):
     ops.grouped_down(h2, wd, off1, ord1, y1)
     plain.grouped_down(h2, wd, off1, ord1, y2)
     close(y1, y2, dtype, scale=h2.float().abs().max().item() * math.sqrt(inner) * 0.3)
+    # the same products walking the tile lists that routing writes
+    from ninfer_amd.parts.moe import Routing
+    n = t * k
+    i32 = lambda *sh: torch.zeros(*sh, device="cuda", dtype=torch.int32)
+    tl = Routing(ids1, w1, off1, i32(n), i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2))
+    ops.moe_align(ids1, e, i32(e + 1), tl.order, tiles=tl)
+    h3 = torch.zeros_like(h1)
+    ops.grouped_swiglu(x, wgu, off1, tl.order, k, h3, tiles=tl)
+    y3 = torch.zeros_like(y1)
+    ops.grouped_down(h3, wd, off1, tl.order, y3, tiles=tl)
+    y4 = torch.zeros_like(y1)
+    plain.grouped_down(h3, wd, off1, tl.order, y4)
+    close(y3, y4, dtype, scale=h2.float().abs().max().item() * math.sqrt(inner) * 0.3)
+    close(y3, y2, dtype, scale=h2.float().abs().max().item() * math.sqrt(inner) * 0.3)
     shared = rnd((t, h), dtype, gen)
     gate = torch.randn(t, 1, generator=gen, device="cuda")
     r1 = torch.randn(t, h, generator=gen, device="cuda")
@@ -181,6 +195,68 @@ def test_router_align_experts_combine(ops_mode, gen, dtype, t, e, k, h, inner):
     ops.moe_combine(r1, y2, w1)
     plain.moe_combine(r2, y2, w1)
     close(r1, r2, torch.float32, scale=y2.float().abs().max().item())
+
+
+@pytest.mark.parametrize("t,e,k", [(1, 60, 4), (8, 60, 4), (64, 64, 8), (200, 8, 3), (300, 60, 4),
+                                   (1000, 5, 2)])
+def test_routing_in_one_call_with_tile_lists(ops, gen, t, e, k):
+    """moe_route (one launch for few rows, two for many) against the twins; the
+    tile lists cover every routed row exactly once, expert by expert."""
+    from ninfer_amd.parts.moe import Routing
+    logits = torch.randn(t, e + 1, generator=gen, device="cuda") * 2   # one more column: ignored
+    n = t * k
+
+    def routing():
+        i32 = lambda *s: torch.zeros(*s, device="cuda", dtype=torch.int32)
+        return Routing(i32(t, k), torch.zeros(t, k, device="cuda"), i32(e + 1), i32(n),
+                       i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2))
+    r1, r2 = routing(), routing()
+    ops.moe_route(logits, e, k, True, r1)
+    PlainOps().moe_route(logits, e, k, True, r2)
+    assert torch.equal(r1.ids, r2.ids) and torch.equal(r1.offsets, r2.offsets)
+    close(r1.weights, r2.weights, torch.float32)
+    assert torch.equal(r1.tile_counts, r2.tile_counts)
+    n16, n64 = r1.tile_counts.tolist()
+    assert torch.equal(r1.tiles16[:n16], r2.tiles16[:n16])
+    assert torch.equal(r1.tiles64[:n64], r2.tiles64[:n64])
+    covered = []
+    for ex, r0, end, _ in r1.tiles16[:n16].tolist():
+        covered += list(range(r0, min(r0 + 16, end)))
+        assert int(r1.offsets[ex]) <= r0 < end == int(r1.offsets[ex + 1])
+    assert covered == list(range(n))
+    flat = r1.ids.reshape(-1)
+    off = r1.offsets.tolist()
+    for g in range(e):
+        assert all(int(flat[i]) == g for i in r1.order[off[g]:off[g + 1]].tolist())
+    assert sorted(r1.order.tolist()) == list(range(n))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_adds_a_sum_of_rows_on_the_fly(ops, gen, dtype):
+    from ninfer_amd.parts import PendingRows
+    t, h, k = 9, 200, 3
+    gain = 1 + 0.1 * torch.randn(h, generator=gen, device="cuda")
+    x = torch.randn(t, h, generator=gen, device="cuda")
+    logits = torch.randn(t, 7, generator=gen, device="cuda")
+    for shared, gate in ((None, None), (rnd((t, h), dtype, gen), None),
+                         (rnd((t, h), dtype, gen), logits[:, 6])):     # a strided gate column
+        pend = PendingRows(rnd((t * k, h), dtype, gen), torch.rand(t, k, generator=gen,
+                                                                   device="cuda"), shared, gate)
+        x1, x2 = x.clone(), x.clone()
+        o1 = torch.empty(t, h, device="cuda", dtype=dtype)
+        o2 = torch.empty_like(o1)
+        ops.rmsnorm(x1, gain, 1e-6, o1, rows_sum=pend)
+        PlainOps().rmsnorm(x2, gain, 1e-6, o2, rows_sum=pend)
+        close(o1, o2, dtype)
+        close(x1, x2, torch.float32)
+        sel = torch.tensor([t - 1, 2], device="cuda", dtype=torch.int32)
+        o1 = torch.empty(2, h, device="cuda", dtype=dtype)
+        o2 = torch.empty_like(o1)
+        x1 = x.clone()
+        ops.rmsnorm(x1, gain, 1e-6, o1, rows_sum=pend, rows=sel)
+        PlainOps().rmsnorm(x.clone(), gain, 1e-6, o2, rows_sum=pend, rows=sel)
+        close(o1, o2, dtype)
+        assert torch.equal(x1, x)
 
 
 def test_router_ties_go_to_the_lower_index(ops):

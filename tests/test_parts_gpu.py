@@ -99,9 +99,20 @@ def test_feed_forward_parts(ops, dtype):
         else:
             clear = torch.ones(t, dtype=torch.bool)
         ref = pm.routed_experts(x.float(), ids, wts, wr, "m.") + pm.shared_expert(x.float(), wr, "m.")
+        from ninfer_amd.parts import PendingRows, RMSNorm
         residual = torch.zeros(t, hidden, device="cuda")
-        assert moe.forward(ctx, x.cuda(), residual) is None      # it adds into the residual itself
+        pending = moe.forward(ctx, x.cuda(), residual)
+        assert isinstance(pending, PendingRows)       # left for the next norm's kernel to add
+        norm = RMSNorm("n.", hidden, 1e-6)
+        bind(norm, {"n.weight": torch.ones(hidden)}, dtype)
+        normed = norm.forward(ctx, residual, pending)   # adds on the fly, keeps the sum
         torch.testing.assert_close(residual.cpu()[clear], ref[clear], **BOUND[dtype])
+        torch.testing.assert_close(normed.float().cpu()[clear],
+                                   pm.rms_norm(ref, torch.ones(hidden), 1e-6)[clear],
+                                   **BOUND[dtype])
+        residual2 = torch.zeros(t, hidden, device="cuda")
+        pending.add_to(ctx, residual2)                  # the same sum by the stand-alone kernel
+        torch.testing.assert_close(residual2, residual, atol=1e-6, rtol=1e-6)
         assert clear.sum() > t // 2
 
 
