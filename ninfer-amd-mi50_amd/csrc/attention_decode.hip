@@ -23,15 +23,20 @@ namespace ninfer {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-constexpr int kChunk = 256;      // keys per block
 constexpr int kDecWaves = 4;
+
+// Keys per block: 256, or 128 when that many blocks would leave the GPU idle.
+static int decode_chunk(int T, int Hkv, int max_kv_len) {
+  long blocks = (long)T * Hkv * ((max_kv_len + 255) / 256);
+  return blocks < 1024 ? 128 : 256;
+}
 
 __device__ __forceinline__ void cvt8(const bf16x8& v, float* f) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
 }
 
-template <int LPK, int GQ>
+template <int LPK, int GQ, int kChunk>
 __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a, int head_groups) {
   constexpr int D = 8 * LPK;
   constexpr int KPI = 64 / LPK;             // keys per wave instruction
@@ -177,7 +182,8 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
 
 // out[t, h, :] = sum_c acc_c exp(m_c - M) / sum_c l_c exp(m_c - M), chunks in order.
 // Block of 128 threads; LDS holds one scale per chunk.
-__global__ __launch_bounds__(128) void attn_decode_merge_kernel(AttnArgs a, int n_chunks) {
+__global__ __launch_bounds__(128) void attn_decode_merge_kernel(AttnArgs a, int n_chunks,
+                                                                int kChunk) {
   extern __shared__ float scale_s[];   // [n_chunks]
   __shared__ float red[4];
   const int t = blockIdx.x, h = blockIdx.y, D = a.D, tid = threadIdx.x;
@@ -215,7 +221,7 @@ __global__ __launch_bounds__(128) void attn_decode_merge_kernel(AttnArgs a, int 
 }
 
 int64_t attention_decode_workspace_floats(int T, int Hq, int D, int max_kv_len) {
-  int n_chunks = (max_kv_len + kChunk - 1) / kChunk;
+  int n_chunks = (max_kv_len + 127) / 128;   // the smaller chunk size bounds the need
   return (int64_t)T * Hq * n_chunks * (D + 2);
 }
 
@@ -225,33 +231,44 @@ bool attention_decode_takes(const AttnArgs& a) {
   return a.dtype == kBF16 && d_ok && a.q_stride % 8 == 0 && a.workspace != nullptr;
 }
 
-template <int LPK>
+template <int LPK, int CHUNK>
 static void launch_decode(const AttnArgs& a, int n_chunks, hipStream_t stream) {
   int group = a.Hq / a.Hkv;
+  dim3 block(kDecWaves * 64);
   if (group == 1) {
-    attn_decode_kernel<LPK, 1><<<dim3(n_chunks, a.Hkv, a.T), kDecWaves * 64, 0, stream>>>(a, 1);
+    attn_decode_kernel<LPK, 1, CHUNK><<<dim3(n_chunks, a.Hkv, a.T), block, 0, stream>>>(a, 1);
   } else if (group == 2) {
-    attn_decode_kernel<LPK, 2><<<dim3(n_chunks, a.Hkv, a.T), kDecWaves * 64, 0, stream>>>(a, 1);
+    attn_decode_kernel<LPK, 2, CHUNK><<<dim3(n_chunks, a.Hkv, a.T), block, 0, stream>>>(a, 1);
   } else {
     int hg = (group + 3) / 4;
-    attn_decode_kernel<LPK, 4><<<dim3(n_chunks, a.Hkv * hg, a.T), kDecWaves * 64, 0, stream>>>(a, hg);
+    attn_decode_kernel<LPK, 4, CHUNK><<<dim3(n_chunks, a.Hkv * hg, a.T), block, 0, stream>>>(a, hg);
   }
 }
 
+template <int LPK>
+static void launch_decode_chunk(const AttnArgs& a, int chunk, int n_chunks, hipStream_t stream) {
+  if (chunk == 128)
+    launch_decode<LPK, 128>(a, n_chunks, stream);
+  else
+    launch_decode<LPK, 256>(a, n_chunks, stream);
+}
+
 int attention_decode(const AttnArgs& a, hipStream_t stream) {
-  int n_chunks = (a.max_kv_len + kChunk - 1) / kChunk;
+  const int chunk = decode_chunk(a.T, a.Hkv, a.max_kv_len);
+  const int n_chunks = (a.max_kv_len + chunk - 1) / chunk;
   NINFER_REQUIRE(a.workspace_floats >= attention_decode_workspace_floats(a.T, a.Hq, a.D, a.max_kv_len),
                  "paged_attention: workspace of %lld floats is too small", (long long)a.workspace_floats);
   switch (a.D) {
-    case 16: launch_decode<2>(a, n_chunks, stream); break;
-    case 32: launch_decode<4>(a, n_chunks, stream); break;
-    case 64: launch_decode<8>(a, n_chunks, stream); break;
-    case 128: launch_decode<16>(a, n_chunks, stream); break;
-    case 256: launch_decode<32>(a, n_chunks, stream); break;
+    case 16: launch_decode_chunk<2>(a, chunk, n_chunks, stream); break;
+    case 32: launch_decode_chunk<4>(a, chunk, n_chunks, stream); break;
+    case 64: launch_decode_chunk<8>(a, chunk, n_chunks, stream); break;
+    case 128: launch_decode_chunk<16>(a, chunk, n_chunks, stream); break;
+    case 256: launch_decode_chunk<32>(a, chunk, n_chunks, stream); break;
     default: return set_error(-1, "paged_attention: decode kernel does not take head size %d", a.D);
   }
   NINFER_LAUNCH_CHECK();
-  attn_decode_merge_kernel<<<dim3(a.T, a.Hq), 128, n_chunks * sizeof(float), stream>>>(a, n_chunks);
+  attn_decode_merge_kernel<<<dim3(a.T, a.Hq), 128, n_chunks * sizeof(float), stream>>>(a, n_chunks,
+                                                                                      chunk);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

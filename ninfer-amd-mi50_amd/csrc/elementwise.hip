@@ -30,23 +30,15 @@ struct MoeSum {
   int k;
 };
 
-template <typename T>
-__device__ __forceinline__ float moe_sum_at(const MoeSum& ms, int64_t t, int i, int H, float g) {
-  float acc = 0.f;
-  const T* y = (const T*)ms.y;
-  for (int j = 0; j < ms.k; ++j) acc += ms.w[t * ms.k + j] * to_f32(y[(t * ms.k + j) * H + i]);
-  if (ms.shared) acc += g * to_f32(((const T*)ms.shared)[t * H + i]);
-  return acc;
-}
-
 constexpr int kNormPerThread = 8;
 
 // y = (x [+ delta] [+ moe sum]) * rsqrt(mean(.^2) + eps) * gain  (reference
 // src/ops/kernels.hip:17-41 and :100-129). With rows == nullptr the sum is
 // written back to x; with rows the kernel reads row rows[i] and leaves x alone.
 // Every thread keeps its (at most 8) elements in registers between the two
-// passes. The reduction order depends only on H and the block size, never on
-// the number of rows.
+// passes; all loads of a thread are independent of each other, so they are in
+// flight together. The reduction order depends only on H and the block size,
+// never on the number of rows.
 template <typename T>
 __global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta, MoeSum ms,
                                const float* __restrict__ gain, T* __restrict__ out,
@@ -57,10 +49,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delt
   float* xr = x + r_in * H;
   const T* dr = delta ? delta + r_in * H : nullptr;
   T* orow = out + r_out * H;
-  float g = 1.f;
-  if (ms.y && ms.shared && ms.gate) g = 1.f / (1.f + expf(-ms.gate[r_in * ms.gate_stride]));
   float vals[kNormPerThread];
-  float acc = 0.f;
 #pragma unroll
   for (int c = 0; c < kNormPerThread; ++c) {
     int i = threadIdx.x + c * blockDim.x;
@@ -68,11 +57,42 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delt
     if (i < H) {
       v = xr[i];
       if (dr) v += to_f32(dr[i]);
-      if (ms.y) v += moe_sum_at<T>(ms, r_in, i, H, g);
     }
     vals[c] = v;
-    acc += v * v;
   }
+  if (ms.y) {
+    const T* y = (const T*)ms.y + r_in * ms.k * H;
+    const float* w = ms.w + r_in * ms.k;
+    for (int j0 = 0; j0 < ms.k; j0 += 4) {   // four routed rows at a time, loads independent
+      float wj[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wj[j] = j0 + j < ms.k ? w[j0 + j] : 0.f;
+#pragma unroll
+      for (int c = 0; c < kNormPerThread; ++c) {
+        int i = threadIdx.x + c * blockDim.x;
+        if (i < H) {
+          float yv[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            yv[j] = j0 + j < ms.k ? to_f32(y[(int64_t)(j0 + j) * H + i]) : 0.f;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) vals[c] += wj[j] * yv[j];
+        }
+      }
+    }
+    if (ms.shared) {
+      float g = ms.gate ? 1.f / (1.f + expf(-ms.gate[r_in * ms.gate_stride])) : 1.f;
+      const T* sh = (const T*)ms.shared + r_in * H;
+#pragma unroll
+      for (int c = 0; c < kNormPerThread; ++c) {
+        int i = threadIdx.x + c * blockDim.x;
+        if (i < H) vals[c] += g * to_f32(sh[i]);
+      }
+    }
+  }
+  float acc = 0.f;
+#pragma unroll
+  for (int c = 0; c < kNormPerThread; ++c) acc += vals[c] * vals[c];
   float total = block_sum(acc, red);
   float inv = rsqrtf(total / (float)H + eps);
   const bool write_back = !rows && (dr || ms.y);
@@ -210,8 +230,10 @@ extern "C" int ninfer_rmsnorm(float* x, const void* delta, const float* gain, vo
   NINFER_REQUIRE(H <= 1024 * kNormPerThread, "rmsnorm: width %d exceeds %d", H,
                  1024 * kNormPerThread);
   NINFER_REQUIRE(!moe_y || (moe_w && moe_k > 0), "rmsnorm: a row sum needs weights and k");
-  int block = ((H + kNormPerThread - 1) / kNormPerThread + 63) / 64 * 64;
-  if (block < 128) block = 128;
+  // few elements per thread: short chains of loads; at most 1024 threads
+  int block = (H / 2 + 63) / 64 * 64;
+  if (block < 64) block = 64;
+  if (block > 1024) block = 1024;
   MoeSum ms{moe_y, moe_w, moe_shared, moe_gate, moe_gate_stride, moe_k};
   if (dtype == kF32)
     rmsnorm_kernel<float><<<n_rows, block, 0, stream>>>(x, (const float*)delta, ms, gain,

@@ -99,26 +99,44 @@ __device__ void align_block(const int* ids, int n, int E, int* __restrict__ offs
   __syncthreads();
   for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cnt[ids[i]], 1);
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0, n16 = 0, n64 = 0;
-    for (int e = 0; e < E; ++e) {
-      int c = cnt[e];
-      offsets[e] = run;
-      cnt[e] = run;
-      if (tiles16) {
-        for (int r = run; r < run + c; r += 16) {
-          ((int4*)tiles16)[n16++] = make_int4(e, r, run + c, 0);
-        }
-        for (int r = run; r < run + c; r += 64) {
-          ((int4*)tiles64)[n64++] = make_int4(e, r, run + c, 0);
+  if (threadIdx.x < 64) {
+    // the first wave scans 64 experts at a time: rows, 16-row tiles, 64-row tiles
+    const int lane = threadIdx.x;
+    int run0 = 0, n16 = 0, n64 = 0;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+      const int e = e0 + lane;
+      const int c = e < E ? cnt[e] : 0;
+      const int t16 = (c + 15) / 16, t64 = (c + 63) / 64;
+      int ic = c, i16 = t16, i64 = t64;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        int a1 = __shfl_up(ic, off, 64), a2 = __shfl_up(i16, off, 64), a3 = __shfl_up(i64, off, 64);
+        if (lane >= off) {
+          ic += a1;
+          i16 += a2;
+          i64 += a3;
         }
       }
-      run += c;
+      const int run = run0 + ic - c;
+      if (e < E) {
+        offsets[e] = run;
+        cnt[e] = run;
+        if (tiles16) {
+          int p16 = n16 + i16 - t16, p64 = n64 + i64 - t64;
+          for (int r = run; r < run + c; r += 16) ((int4*)tiles16)[p16++] = make_int4(e, r, run + c, 0);
+          for (int r = run; r < run + c; r += 64) ((int4*)tiles64)[p64++] = make_int4(e, r, run + c, 0);
+        }
+      }
+      run0 += __shfl(ic, 63, 64);
+      n16 += __shfl(i16, 63, 64);
+      n64 += __shfl(i64, 63, 64);
     }
-    offsets[E] = run;
-    if (tile_counts) {
-      tile_counts[0] = n16;
-      tile_counts[1] = n64;
+    if (lane == 0) {
+      offsets[E] = run0;
+      if (tile_counts) {
+        tile_counts[0] = n16;
+        tile_counts[1] = n64;
+      }
     }
   }
   __syncthreads();

@@ -80,11 +80,16 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   float* w = work + (int64_t)r * V;
   const float temp = temperature[r];
 
-  // repetition penalty on a copy of the row
-  for (int i = tid; i < V; i += blockDim.x) w[i] = row[i];
-  __syncthreads();
+  // repetition penalty on a copy of the row (greedy rows without a penalty read the row itself)
   float rp = rep_penalty ? rep_penalty[r] : 1.f;
-  if (rp != 1.f && pen_offsets) {
+  const bool penalised = rp != 1.f && pen_offsets && pen_offsets[r + 1] > pen_offsets[r];
+  if (!(temp > 0.f) && !penalised) {
+    w = const_cast<float*>(row);
+  } else {
+    for (int i = tid; i < V; i += blockDim.x) w[i] = row[i];
+  }
+  __syncthreads();
+  if (penalised) {
     for (int e = pen_offsets[r] + tid; e < pen_offsets[r + 1]; e += blockDim.x) {
       int tok = pen_tokens[e];
       if (tok < 0 || tok >= V) continue;
@@ -95,15 +100,22 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   }
   __syncthreads();
 
-  // max and argmax (ties: lowest index)
+  // max and argmax (ties: lowest index); four loads in flight per thread
   float best = -INFINITY;
   int best_i = 0x7fffffff;
-  for (int i = tid; i < V; i += blockDim.x) {
-    float v = w[i];
-    if (v > best) {
-      best = v;
-      best_i = i;
+  for (int i0 = tid; i0 < V; i0 += 4 * blockDim.x) {
+    float v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      int i = i0 + u * blockDim.x;
+      v[u] = i < V ? w[i] : -INFINITY;
     }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (v[u] > best) {
+        best = v[u];
+        best_i = i0 + u * blockDim.x;
+      }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
