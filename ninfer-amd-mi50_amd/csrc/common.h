@@ -48,6 +48,14 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   return t;
 }
 
+// A workgroup barrier that waits for this wave's LDS traffic only. The plain
+// __syncthreads() also drains every global load in flight, which undoes
+// software prefetching: loads issued for a later tile would be waited for at
+// the next barrier. Use where the barrier only orders LDS reads and writes.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 int set_error(int code, const char* fmt, ...);
 
 #define NINFER_REQUIRE(cond, ...)                         \

@@ -17,8 +17,8 @@ struct GemmArgs {
   const int* a_index;    // sorted row -> a_index[r] / a_div is the row of A, or null
   const int* c_index;    // sorted row -> row of C, or null
   const int* tiles16;    // grouped: {expert, first row, end row, 0} per 16-row tile, or null
-  const int* tiles64;    // the same for 64-row tiles
-  const int* tile_counts;  // {number of 16-row tiles, number of 64-row tiles}
+  const int* tiles64;    // the same for tiles of big_rows rows
+  const int* tile_counts;  // {number of 16-row tiles, number of big tiles}
   int64_t w_group_stride;  // elements between the weights of two groups
   int M;                 // rows (dense) or number of sorted rows (grouped)
   int N;                 // output features (per SwiGLU half)
@@ -30,6 +30,7 @@ struct GemmArgs {
   int in_dtype;          // of A and W
   int out_dtype;         // of C
   int epilogue;
+  int big_rows;          // rows of a big grouped tile: 64 or 128 (0: 64)
 };
 
 // Which rows does tile `ti` of the grouped enumeration cover? Tiles of

@@ -94,7 +94,7 @@ __device__ __forceinline__ void route_row(const float* __restrict__ row, int E, 
 // `cnt` is E + 1 ints of LDS; ids may be in LDS or global memory.
 __device__ void align_block(const int* ids, int n, int E, int* __restrict__ offsets,
                             int* __restrict__ order, int* __restrict__ tiles16,
-                            int* __restrict__ tiles64, int* __restrict__ tile_counts, int* cnt) {
+                            int* __restrict__ tiles64, int* __restrict__ tile_counts, int big, int* cnt) {
   for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cnt[ids[i]], 1);
@@ -106,7 +106,7 @@ __device__ void align_block(const int* ids, int n, int E, int* __restrict__ offs
     for (int e0 = 0; e0 < E; e0 += 64) {
       const int e = e0 + lane;
       const int c = e < E ? cnt[e] : 0;
-      const int t16 = (c + 15) / 16, t64 = (c + 63) / 64;
+      const int t16 = (c + 15) / 16, t64 = (c + big - 1) / big;
       int ic = c, i16 = t16, i64 = t64;
 #pragma unroll
       for (int off = 1; off < 64; off <<= 1) {
@@ -124,7 +124,7 @@ __device__ void align_block(const int* ids, int n, int E, int* __restrict__ offs
         if (tiles16) {
           int p16 = n16 + i16 - t16, p64 = n64 + i64 - t64;
           for (int r = run; r < run + c; r += 16) ((int4*)tiles16)[p16++] = make_int4(e, r, run + c, 0);
-          for (int r = run; r < run + c; r += 64) ((int4*)tiles64)[p64++] = make_int4(e, r, run + c, 0);
+          for (int r = run; r < run + c; r += big) ((int4*)tiles64)[p64++] = make_int4(e, r, run + c, 0);
         }
       }
       run0 += __shfl(ic, 63, 64);
@@ -146,9 +146,9 @@ __device__ void align_block(const int* ids, int n, int E, int* __restrict__ offs
 __global__ void moe_align_kernel(const int* __restrict__ ids, int n, int E,
                                  int* __restrict__ offsets, int* __restrict__ order,
                                  int* __restrict__ tiles16, int* __restrict__ tiles64,
-                                 int* __restrict__ tile_counts) {
+                                 int* __restrict__ tile_counts, int big) {
   extern __shared__ int cnt[];
-  align_block(ids, n, E, offsets, order, tiles16, tiles64, tile_counts, cnt);
+  align_block(ids, n, E, offsets, order, tiles16, tiles64, tile_counts, big, cnt);
 }
 
 // Few rows (decode): softmax + top-k of every row and the grouping by expert
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(1024) void moe_route_small_kernel(
     const float* __restrict__ logits, int ld, int T, int E, int k, int renorm,
     int* __restrict__ ids, float* __restrict__ wts, int* __restrict__ offsets,
     int* __restrict__ order, int* __restrict__ tiles16, int* __restrict__ tiles64,
-    int* __restrict__ tile_counts) {
+    int* __restrict__ tile_counts, int big) {
   extern __shared__ int cnt[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
   for (int t = wave; t < T; t += waves)
@@ -165,7 +165,7 @@ __global__ __launch_bounds__(1024) void moe_route_small_kernel(
               lane);
   __threadfence();
   __syncthreads();  // the ids written above are read below by other threads of this block
-  align_block(ids, T * k, E, offsets, order, tiles16, tiles64, tile_counts, cnt);
+  align_block(ids, T * k, E, offsets, order, tiles16, tiles64, tile_counts, big, cnt);
 }
 
 }  // namespace ninfer
@@ -185,16 +185,18 @@ extern "C" int ninfer_router_topk(const float* logits, int ld, int T, int E, int
 }
 
 // tiles16 / tiles64 / tile_counts may be null (no tile lists). tiles16 holds
-// 4 ints for each of up to min(n, n / 16 + E) tiles, tiles64 for n / 64 + E.
+// 4 ints for each of up to min(n, n / 16 + E) tiles of 16 rows, tiles64 for up
+// to n / 64 + E tiles of big_rows (64 or 128) rows.
 extern "C" int ninfer_moe_align(const int* ids, int n, int E, int* offsets, int* order,
-                                int* tiles16, int* tiles64, int* tile_counts,
+                                int* tiles16, int* tiles64, int* tile_counts, int big_rows,
                                 hipStream_t stream) {
+  NINFER_REQUIRE(big_rows == 64 || big_rows == 128, "moe_align: big tiles of %d rows", big_rows);
   NINFER_REQUIRE(n > 0 && E > 0, "moe_align: n=%d E=%d must be positive", n, E);
   NINFER_REQUIRE(E <= 8192, "moe_align: %d experts exceed 8192", E);
   NINFER_REQUIRE((!tiles16) == (!tiles64) && (!tiles16) == (!tile_counts),
                  "moe_align: tile lists come together or not at all");
   moe_align_kernel<<<1, 1024, (E + 1) * sizeof(int), stream>>>(ids, n, E, offsets, order, tiles16,
-                                                             tiles64, tile_counts);
+                                                             tiles64, tile_counts, big_rows);
   NINFER_LAUNCH_CHECK();
   return 0;
 }
@@ -202,8 +204,10 @@ extern "C" int ninfer_moe_align(const int* ids, int n, int E, int* offsets, int*
 // Routing of few rows in one launch: top-k and grouping (T <= 256).
 extern "C" int ninfer_moe_route_small(const float* logits, int ld, int T, int E, int k,
                                       int renorm, int* ids, float* wts, int* offsets, int* order,
-                                      int* tiles16, int* tiles64, int* tile_counts,
+                                      int* tiles16, int* tiles64, int* tile_counts, int big_rows,
                                       hipStream_t stream) {
+  NINFER_REQUIRE(big_rows == 64 || big_rows == 128, "moe_route_small: big tiles of %d rows",
+                 big_rows);
   NINFER_REQUIRE(T > 0 && T <= 256, "moe_route_small: T=%d not in [1, 256]", T);
   NINFER_REQUIRE(E > 0 && E <= 64 * kMaxExpertsPerLane, "moe_route_small: %d experts exceed %d", E,
                  64 * kMaxExpertsPerLane);
@@ -213,7 +217,8 @@ extern "C" int ninfer_moe_route_small(const float* logits, int ld, int T, int E,
                  "moe_route_small: tile lists come together or not at all");
   int threads = T >= 16 ? 1024 : 64 * T;
   moe_route_small_kernel<<<1, threads, (E + 1) * sizeof(int), stream>>>(
-      logits, ld, T, E, k, renorm, ids, wts, offsets, order, tiles16, tiles64, tile_counts);
+      logits, ld, T, E, k, renorm, ids, wts, offsets, order, tiles16, tiles64, tile_counts,
+      big_rows);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

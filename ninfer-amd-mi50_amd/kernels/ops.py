@@ -31,7 +31,7 @@ class _GemmArgs(ctypes.Structure):
                 ("M", ctypes.c_int), ("N", ctypes.c_int), ("K", ctypes.c_int),
                 ("lda", ctypes.c_int), ("ldc", ctypes.c_int), ("groups", ctypes.c_int),
                 ("a_div", ctypes.c_int), ("in_dtype", ctypes.c_int), ("out_dtype", ctypes.c_int),
-                ("epilogue", ctypes.c_int)]
+                ("epilogue", ctypes.c_int), ("big_rows", ctypes.c_int)]
 
 
 class _AttnArgs(ctypes.Structure):
@@ -199,13 +199,15 @@ class HipOps:
     def _gemm(self, a, w, c, *, n, k, m, bias=None, offsets=None, a_index=None, c_index=None,
               a_div=1, groups=1, epilogue=0, w_group_stride=0, tiles=None):
         t16 = t64 = tc = None
+        big = 0
         if tiles is not None and tiles.tiles16 is not None:
             t16, t64, tc = tiles.tiles16.data_ptr(), tiles.tiles64.data_ptr(), \
                 tiles.tile_counts.data_ptr()
+            big = tiles.big_rows
         args = _GemmArgs(a.data_ptr(), w.data_ptr(), c.data_ptr(), _ptr(bias), _ptr(offsets),
                          _ptr(a_index), _ptr(c_index), t16, t64, tc, w_group_stride, m, n, k,
                          a.shape[1],
-                         c.shape[1], groups, a_div, _DT[a.dtype], _DT[c.dtype], epilogue)
+                         c.shape[1], groups, a_div, _DT[a.dtype], _DT[c.dtype], epilogue, big)
         self._ok(self.lib.ninfer_gemm(ctypes.byref(args), 1 if self.force_generic else 0,
                                       self._stream()))
 
@@ -320,7 +322,8 @@ class HipOps:
         self._ok(self.lib.ninfer_moe_align(
             ctypes.c_void_p(ids.data_ptr()), ids.numel(), experts,
             ctypes.c_void_p(offsets.data_ptr()), ctypes.c_void_p(order.data_ptr()),
-            ctypes.c_void_p(t16), ctypes.c_void_p(t64), ctypes.c_void_p(tc), self._stream()))
+            ctypes.c_void_p(t16), ctypes.c_void_p(t64), ctypes.c_void_p(tc),
+            getattr(tiles, "big_rows", 64) if tiles is not None else 64, self._stream()))
 
     def moe_route(self, logits, experts, top_k, renorm, r):
         """Softmax + top-k per row and the grouping by expert, into the routing
@@ -345,7 +348,7 @@ class HipOps:
             1 if renorm else 0, ctypes.c_void_p(r.ids.data_ptr()),
             ctypes.c_void_p(r.weights.data_ptr()), ctypes.c_void_p(r.offsets.data_ptr()),
             ctypes.c_void_p(r.order.data_ptr()), ctypes.c_void_p(t16), ctypes.c_void_p(t64),
-            ctypes.c_void_p(tc), self._stream()))
+            ctypes.c_void_p(tc), r.big_rows, self._stream()))
 
     # ---- attention ------------------------------------------------------------------
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,

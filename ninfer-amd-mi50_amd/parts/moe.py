@@ -54,7 +54,8 @@ class SoftmaxTopKRouter(Part):
                     offsets=ctx.empty((e + 1,), torch.int32), order=ctx.empty((n,), torch.int32),
                     tiles16=ctx.empty((min(n, n // 16 + e), 4), torch.int32),
                     tiles64=ctx.empty((n // 64 + e, 4), torch.int32),
-                    tile_counts=ctx.empty((2,), torch.int32))
+                    tile_counts=ctx.empty((2,), torch.int32),
+                    big_rows=128 if n >= 96 * e else 64)
         ctx.ops.moe_route(logits, e, k, self.renorm, r)
         return r
 
@@ -64,9 +65,11 @@ class Routing:
     the (row, choice) indices grouped by expert (`order`, `offsets`), and the
     lists of 16-row and 64-row tiles the grouped products walk."""
 
-    def __init__(self, ids, weights, offsets, order, tiles16=None, tiles64=None, tile_counts=None):
+    def __init__(self, ids, weights, offsets, order, tiles16=None, tiles64=None, tile_counts=None,
+                 big_rows=64):
         self.ids, self.weights, self.offsets, self.order = ids, weights, offsets, order
         self.tiles16, self.tiles64, self.tile_counts = tiles16, tiles64, tile_counts
+        self.big_rows = big_rows   # rows of a tile in `tiles64`: 64, or 128 when experts get many rows
 
 
 class RoutedExperts(Part):

@@ -134,7 +134,7 @@ class PlainOps:
         order.copy_(torch.sort(flat, stable=True).indices.to(torch.int32))
         if tiles is not None and tiles.tiles16 is not None:
             off = offsets.tolist()
-            for size, out in ((16, tiles.tiles16), (64, tiles.tiles64)):
+            for size, out in ((16, tiles.tiles16), (tiles.big_rows, tiles.tiles64)):
                 lst = [[e, r, off[e + 1], 0] for e in range(experts)
                        for r in range(off[e], off[e + 1], size)]
                 if lst:

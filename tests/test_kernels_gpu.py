@@ -86,7 +86,8 @@ def test_rmsnorm(ops, gen, dtype, rows, h):
 @pytest.mark.parametrize("m,n,k", [(1, 48, 40), (3, 130, 72), (17, 64, 200), (70, 200, 136),
                                    (129, 96, 64), (5, 130, 256), (16, 48, 2048), (33, 100, 128),
                                    (8, 2048, 1408), (1, 300, 5632), (2, 61, 96), (200, 60, 128),
-                                   (333, 700, 256), (64, 256, 32)])
+                                   (333, 700, 256), (64, 256, 32), (130, 1000, 256), (600, 129, 512),
+                                   (257, 300, 384)])
 def test_linear(ops_mode, gen, dtype, m, n, k):
     ops = ops_mode
     x, w = rnd((m, k), dtype, gen), rnd((n, k), dtype, gen)
@@ -129,7 +130,8 @@ def test_linear_row_result_does_not_depend_on_batch(ops, gen):
                                            (150, 60, 4, 128, 80), (3, 6, 6, 72, 40),
                                            (40, 6, 2, 128, 64), (300, 4, 2, 64, 96),
                                            (8, 60, 4, 256, 160), (700, 5, 3, 128, 192),
-                                           (512, 8, 2, 64, 96)])
+                                           (512, 8, 2, 64, 96), (600, 5, 2, 256, 256),
+                                           (300, 7, 3, 384, 128)])
 def test_router_align_experts_combine(ops_mode, gen, dtype, t, e, k, h, inner):
     """The whole sparse feed-forward chain, kernel by kernel, against the twins;
     with few rows most experts get none."""
@@ -174,7 +176,8 @@ def test_router_align_experts_combine(ops_mode, gen, dtype, t, e, k, h, inner):
     from ninfer_amd.parts.moe import Routing
     n = t * k
     i32 = lambda *sh: torch.zeros(*sh, device="cuda", dtype=torch.int32)
-    tl = Routing(ids1, w1, off1, i32(n), i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2))
+    tl = Routing(ids1, w1, off1, i32(n), i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2),
+                 big_rows=128 if n >= 96 * e else 64)
     ops.moe_align(ids1, e, i32(e + 1), tl.order, tiles=tl)
     h3 = torch.zeros_like(h1)
     ops.grouped_swiglu(x, wgu, off1, tl.order, k, h3, tiles=tl)
@@ -209,7 +212,8 @@ def test_routing_in_one_call_with_tile_lists(ops, gen, t, e, k):
     def routing():
         i32 = lambda *s: torch.zeros(*s, device="cuda", dtype=torch.int32)
         return Routing(i32(t, k), torch.zeros(t, k, device="cuda"), i32(e + 1), i32(n),
-                       i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2))
+                       i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2),
+                       big_rows=128 if t >= 300 else 64)
     r1, r2 = routing(), routing()
     ops.moe_route(logits, e, k, True, r1)
     PlainOps().moe_route(logits, e, k, True, r2)
