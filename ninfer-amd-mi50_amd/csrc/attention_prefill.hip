@@ -84,41 +84,67 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
   constexpr int V_BLOCKS = (PK / 4) * (D / 8);        // 4 x 8 blocks in a V tile
   static_assert(K_VECS % 256 == 0, "tile does not divide over the block");
 
-  for (int t0 = (lo_first / PK) * PK; t0 <= pos_last; t0 += PK) {
-    __syncthreads();  // the previous tile has been consumed
+  // A tile's keys and values travel global -> registers -> LDS; the next
+  // tile's loads are issued before the products of the current one.
+  constexpr int V_PER_THREAD = (V_BLOCKS + 255) / 256;
+  bf16x8 kreg[K_PER_THREAD], vreg[V_PER_THREAD][4];
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  auto load_regs = [&](int t0) {
 #pragma unroll
     for (int i = 0; i < K_PER_THREAD; ++i) {
       int vec = tid + i * 256;
       int key = vec / (D / 8), dv = vec % (D / 8);
       int kp = t0 + key;
-      bf16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
+      kreg[i] = zero8;
       if (kp <= pos_last) {
         int page = bt[kp / ps];
         if (page >= 0)
-          val = *(const bf16x8*)(kpool + (((int64_t)page * Hkv + g) * ps + kp % ps) * D + 8 * dv);
+          kreg[i] = *(const bf16x8*)(kpool + (((int64_t)page * Hkv + g) * ps + kp % ps) * D + 8 * dv);
       }
-      *(bf16x8*)(k_s + key * KPAD + 8 * dv) = val;
     }
-    for (int blk = tid; blk < V_BLOCKS; blk += 256) {
+#pragma unroll
+    for (int i = 0; i < V_PER_THREAD; ++i) {
+      int blk = tid + i * 256;
       int kg = blk % (PK / 4), dv = blk / (PK / 4);
-      bf16x8 rows[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         int kp = t0 + 4 * kg + r;
-        rows[r] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
-        if (kp <= pos_last) {
+        vreg[i][r] = zero8;
+        if (blk < V_BLOCKS && kp <= pos_last) {
           int page = bt[kp / ps];
           if (page >= 0)
-            rows[r] = *(const bf16x8*)(vpool + (((int64_t)page * Hkv + g) * ps + kp % ps) * D + 8 * dv);
+            vreg[i][r] = *(const bf16x8*)(vpool + (((int64_t)page * Hkv + g) * ps + kp % ps) * D + 8 * dv);
         }
       }
+    }
+  };
+  auto store_regs = [&]() {
 #pragma unroll
-      for (int d = 0; d < 8; ++d) {
-        bf16x4 col = {rows[0][d], rows[1][d], rows[2][d], rows[3][d]};
-        *(bf16x4*)(vt_s + (8 * dv + d) * VPAD + 4 * kg) = col;
+    for (int i = 0; i < K_PER_THREAD; ++i) {
+      int vec = tid + i * 256;
+      *(bf16x8*)(k_s + (vec / (D / 8)) * KPAD + 8 * (vec % (D / 8))) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < V_PER_THREAD; ++i) {
+      int blk = tid + i * 256;
+      if (blk < V_BLOCKS) {
+        int kg = blk % (PK / 4), dv = blk / (PK / 4);
+#pragma unroll
+        for (int d = 0; d < 8; ++d) {
+          bf16x4 col = {vreg[i][0][d], vreg[i][1][d], vreg[i][2][d], vreg[i][3][d]};
+          *(bf16x4*)(vt_s + (8 * dv + d) * VPAD + 4 * kg) = col;
+        }
       }
     }
-    __syncthreads();
+  };
+
+  const int t_first = (lo_first / PK) * PK;
+  load_regs(t_first);
+  for (int t0 = t_first; t0 <= pos_last; t0 += PK) {
+    lds_barrier();   // the previous tile has been consumed
+    store_regs();
+    lds_barrier();
+    if (t0 + PK <= pos_last) load_regs(t0 + PK);
 
     // S^T = K Q^T : 4 key blocks of 16
     f32x4 s[4];

@@ -106,10 +106,12 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delt
   }
 }
 
-// One block per (row, head) of the fused q|k|v row. Adds the bias, rotates q
+// One block per row of the fused q|k|v activations. Adds the bias, rotates q
 // heads in place and k heads on their way into the page; v heads are copied.
 // Pairs are (i, i + rot/2) within the first `rot` dims of a head (reference
 // src/ops/kernels.hip:86-91, full rotation there); dims >= rot pass through.
+// A work item is one rotating pair or one pass-through element, read and
+// written by one thread, so q can be rewritten in place without a barrier.
 // Page lookup: logical page pos / page_size of the row's request.
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restrict__ bias,
@@ -119,43 +121,48 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
                                      int D, T* __restrict__ kpool, T* __restrict__ vpool,
                                      const int* __restrict__ block_table, int bt_stride,
                                      int page_size, int write_kv) {
-  int t = blockIdx.x;
-  int head = blockIdx.y;
-  int d = threadIdx.x;
-  int W = (Hq + 2 * Hkv) * D;
-  int col = head * D + d;
+  const int t = blockIdx.x;
+  const int half = rot >> 1;
+  const int per_head = half + (D - rot);          // items of a rotated head
+  const int n_heads = write_kv ? Hq + 2 * Hkv : Hq;
+  const int W = (Hq + 2 * Hkv) * D;
   T* row = qkv + (int64_t)t * W;
-  bool is_q = head < Hq;
-  bool is_k = !is_q && head < Hq + Hkv;
-  if (!is_q && !write_kv) return;  // uniform per block
-  int pos = positions[t];
-  float v = 0.f, partner = 0.f;
-  int half = rot >> 1;
-  if (d < D) {
-    v = to_f32(row[col]) + (bias ? bias[col] : 0.f);
-    if ((is_q || is_k) && d < rot) {
-      int pd = d < half ? d + half : d - half;
-      partner = to_f32(row[head * D + pd]) + (bias ? bias[head * D + pd] : 0.f);
+  const int pos = positions[t];
+  const int page = write_kv ? block_table[(int64_t)row_seq[t] * bt_stride + pos / page_size] : 0;
+  const int slot = pos % page_size;
+  for (int it = blockIdx.y * blockDim.x + threadIdx.x; it < n_heads * per_head;
+       it += gridDim.y * blockDim.x) {
+    const int head = it / per_head, i = it % per_head;
+    const bool is_q = head < Hq, is_k = !is_q && head < Hq + Hkv;
+    const int base = head * D;
+    int d0, d1 = -1;                               // element(s) of this item
+    float v0, v1 = 0.f;
+    if (i < half) {
+      d0 = i;
+      d1 = i + half;
+      v0 = to_f32(row[base + d0]) + (bias ? bias[base + d0] : 0.f);
+      v1 = to_f32(row[base + d1]) + (bias ? bias[base + d1] : 0.f);
+      if (is_q || is_k) {
+        float phi = (float)pos * inv_freq[i];
+        float c = cosf(phi), s = sinf(phi);
+        float r0 = v0 * c - v1 * s, r1 = v0 * s + v1 * c;
+        v0 = r0;
+        v1 = r1;
+      }
+    } else {
+      d0 = rot + (i - half);
+      v0 = to_f32(row[base + d0]) + (bias ? bias[base + d0] : 0.f);
+    }
+    if (is_q) {
+      row[base + d0] = from_f32<T>(v0);
+      if (d1 >= 0) row[base + d1] = from_f32<T>(v1);
+    } else {
+      const int kvh = is_k ? head - Hq : head - Hq - Hkv;
+      T* dst = (is_k ? kpool : vpool) + (((int64_t)page * Hkv + kvh) * page_size + slot) * D;
+      dst[d0] = from_f32<T>(v0);
+      if (d1 >= 0) dst[d1] = from_f32<T>(v1);
     }
   }
-  __syncthreads();  // all reads of the row are done before q is rewritten
-  if (d >= D) return;
-  float res = v;
-  if ((is_q || is_k) && d < rot) {
-    int i = d < half ? d : d - half;
-    float phi = (float)pos * inv_freq[i];
-    float c = cosf(phi), s = sinf(phi);
-    res = d < half ? v * c - partner * s : partner * s + v * c;
-  }
-  if (is_q) {
-    row[col] = from_f32<T>(res);
-    return;
-  }
-  int seq = row_seq[t];
-  int page = block_table[(int64_t)seq * bt_stride + pos / page_size];
-  int kvh = is_k ? head - Hq : head - Hq - Hkv;
-  int64_t off = (((int64_t)page * Hkv + kvh) * page_size + (pos % page_size)) * D + d;
-  (is_k ? kpool : vpool)[off] = from_f32<T>(res);
 }
 
 // residual[t,:] += sum_j w[t,j] * y[t*k + j,:] + sigmoid(gate[t]) * shared[t,:]
@@ -257,8 +264,11 @@ extern "C" int ninfer_rope_kv_write(void* qkv, const float* bias, const int* pos
   NINFER_REQUIRE(rot_dim == 0 || inv_freq, "rope_kv_write: rotary size %d without a table", rot_dim);
   NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "rope_kv_write: unknown dtype %d", dtype);
   NINFER_REQUIRE(page_size > 0 && bt_stride > 0, "rope_kv_write: bad page size or table width");
-  dim3 grid(T, Hq + 2 * Hkv);
-  int block = (D + 63) / 64 * 64;
+  // few rows: spread a row's items over several blocks; many rows: one block per row
+  int items = (Hq + 2 * Hkv) * (rot_dim / 2 + D - rot_dim);
+  int per_row = T >= 256 ? 1 : (items + 255) / 256;
+  dim3 grid(T, per_row);
+  int block = 256;
   if (dtype == kF32)
     rope_kv_write_kernel<float><<<grid, block, 0, stream>>>(
         (float*)qkv, bias, positions, row_seq, inv_freq, rot_dim, Hq, Hkv, D, (float*)kpool,
