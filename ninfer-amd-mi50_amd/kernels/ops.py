@@ -328,9 +328,10 @@ class HipOps:
     def moe_route(self, logits, experts, top_k, renorm, r):
         """Softmax + top-k per row and the grouping by expert, into the routing
         record `r` (ids, weights, offsets, order, tile lists): one launch for up
-        to 256 rows, two for more."""
+        to 16 rows (one block does both), two for more (top-k by one wave per
+        row in parallel, then the grouping)."""
         t = logits.shape[0]
-        if t > 256:
+        if t > 16:
             self.router_topk(logits, experts, top_k, renorm, r.ids, r.weights)
             self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r)
             return
