@@ -255,7 +255,7 @@ bool gemm_tile_takes(const GemmArgs& a) {
          ((uintptr_t)a.W % 16 == 0) && a.w_group_stride % 8 == 0;
 }
 
-static int g_tile_variant = 0;   // tests and tuning: 0 = default
+static int g_tile_variant = 0;   // tests: 0 = choose by shape
 
 template <int TM, int TN, int TK, int WGM, int P>
 static int launch_tile(const GemmArgs& a, hipStream_t stream) {
@@ -287,16 +287,11 @@ static int launch_tile(const GemmArgs& a, hipStream_t stream) {
 }
 
 int gemm_tile(const GemmArgs& a, hipStream_t stream) {
-  switch (g_tile_variant) {
-    case 1: return launch_tile<64, 256, 32, 4, 2>(a, stream);
-    case 3: return launch_tile<64, 256, 64, 4, 2>(a, stream);
-    case 4: return launch_tile<64, 128, 64, 2, 2>(a, stream);
-    case 7: return launch_tile<128, 128, 64, 2, 2>(a, stream);
-    case 9: return launch_tile<128, 256, 64, 4, 2>(a, stream);
-    default: break;
-  }
-  // 128-row tiles when there are rows to fill them: twice the work per weight read
-  const bool big = a.offsets ? a.big_rows == 128 : a.M >= 256;
+  // 128-row tiles when there are rows to fill them: twice the work per weight read.
+  // g_tile_variant (tests): 1 forces 64-row tiles, 2 forces 128-row tiles on dense products.
+  bool big = a.offsets ? a.big_rows == 128 : a.M >= 256;
+  if (!a.offsets && g_tile_variant == 1) big = false;
+  if (!a.offsets && g_tile_variant == 2) big = true;
   if (big) return launch_tile<128, 128, 64, 2, 2>(a, stream);
   return launch_tile<64, 128, 64, 2, 2>(a, stream);
 }

@@ -117,3 +117,31 @@ def test_graph_replay_equals_eager(case, dtype):
     assert runners[1]._graphs and any(e["graph"] is not None for e in runners[1]._graphs.values())
     for a, b in zip(*outs):
         assert torch.equal(a, b)
+
+
+def test_graph_replay_with_many_requests(model_dirs):
+    """40 requests decode together: dense products of more than 32 rows go to the
+    vendor library, also inside the captured graph. Every replay must equal the
+    eager step (a library call that records nodes a replay mishandles would
+    show here), with eager work between the replays."""
+    from ninfer_amd import Chunk, EngineOptions, load_model
+    d = model_dirs["A"]["bfloat16"]
+    vocab = TINY["A"][0]["vocab_size"]
+    n = 40
+    outs = [[], []]
+    for which, use_graph in enumerate((False, True)):
+        runner = load_model(d, EngineOptions(dtype="bfloat16", max_context=64, num_sequences=n + 1,
+                                             page_size=8, use_graph=use_graph))
+        slots = [runner.open() for _ in range(n)]
+        for i, s in enumerate(slots):
+            runner.step([Chunk(s, util.random_tokens(3 + i % 5, vocab, i), [])])
+        for step in range(8):
+            toks = util.random_tokens(n, vocab, 1000 + step)
+            logits = runner.step([Chunk(s, [t], [0]) for s, t in zip(slots, toks)])
+            outs[which].append(logits.float().cpu().clone())
+            if step % 3 == 1:    # eager work of another shape between replays
+                extra = runner.open()
+                runner.step([Chunk(extra, util.random_tokens(9, vocab, step), [8])])
+                runner.close(extra)
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)

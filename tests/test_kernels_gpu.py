@@ -114,6 +114,32 @@ def test_swiglu_linear(ops_mode, gen, dtype, m, inner, k):
     close(o1, o2, dtype, scale=k * 0.3)
 
 
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("m,n,k", [(333, 700, 256), (70, 130, 384), (129, 1000, 512)])
+def test_tile_product_both_tile_heights(ops, gen, variant, m, n, k):
+    """The many-row kernel with 64-row and with 128-row tiles (tile counts that
+    are no multiple of the 8 XCDs, rows that end inside a tile)."""
+    ops.lib.ninfer_set_tile_variant(variant)
+    try:
+        x, w = rnd((m, k), torch.bfloat16, gen), rnd((n, k), torch.bfloat16, gen)
+        bias = torch.randn(n, generator=gen, device="cuda")
+        o1 = torch.empty(m, n, device="cuda")
+        o2 = torch.empty_like(o1)
+        ops.linear(x, w, o1, bias=bias)
+        PlainOps().linear(x, w, o2, bias=bias)
+        close(o1, o2, torch.float32, scale=200 * math.sqrt(k))
+        wgu = rnd((2 * n, k), torch.bfloat16, gen, 0.2)
+        h1 = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+        h2 = torch.empty_like(h1)
+        ops.library_min_rows, saved = 1 << 30, ops.library_min_rows
+        ops.swiglu_linear(x, wgu, h1)
+        ops.library_min_rows = saved
+        PlainOps().swiglu_linear(x, wgu, h2)
+        close(h1, h2, torch.bfloat16, scale=k * 0.2)
+    finally:
+        ops.lib.ninfer_set_tile_variant(0)
+
+
 def test_linear_row_result_does_not_depend_on_batch(ops, gen):
     """32-bit: a row's product is bit-identical alone and inside a batch."""
     x, w = rnd((70, 136), torch.float32, gen), rnd((200, 136), torch.float32, gen)
