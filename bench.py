@@ -33,6 +33,12 @@ CONFIG_C = {
 }
 
 
+CONFIG_D = dict(CONFIG_C, num_hidden_layers=28, hidden_size=3584, num_attention_heads=28,
+                num_key_value_heads=4, intermediate_size=18944, moe_intermediate_size=2560,
+                shared_expert_intermediate_size=20480, num_experts=64, num_experts_per_tok=8)
+MODELS = {"a2.7b": ("Qwen1.5-MoE-A2.7B", CONFIG_C), "57b-a14b": ("Qwen2-57B-A14B", CONFIG_D)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -45,6 +51,8 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--graph", action="store_true", help="decode through a captured HIP graph")
+    ap.add_argument("--model", default="a2.7b", choices=sorted(MODELS),
+                    help="layer sizes: a2.7b (the default and the headline) or 57b-a14b")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -57,7 +65,8 @@ def main() -> int:
     from ninfer_amd.sampling import SampleRow, Sampler, SamplingParams
     from collections import Counter
 
-    raw = dict(CONFIG_C)
+    model_name, model_cfg = MODELS[args.model]
+    raw = dict(model_cfg)
     layers_full = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
@@ -134,12 +143,12 @@ def main() -> int:
 
     dt, nbytes, n_exp = decode_run(args.batch, args.steps, args.warmup)
     result = {
-        "metric": "decode tok/s at batch 8 (Qwen1.5-MoE-A2.7B shapes, context 8192)",
+        "metric": f"decode tok/s at batch {args.batch} ({model_name} shapes, context {ctx})",
         "value": round(args.batch / dt, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
-        "config": {"model": "Qwen1.5-MoE-A2.7B shapes, random weights", "global_batch": args.batch,
+        "config": {"model": f"{model_name} shapes, random weights", "global_batch": args.batch,
                    "seq_len": ctx, "parallelism": "single GPU", "layers": L,
                    "layers_full": layers_full, "hidden": H, "heads": Hq, "kv_heads": Hkv,
                    "head_dim": D, "moe_intermediate": Im, "shared_intermediate": Is,
