@@ -32,33 +32,70 @@ struct MoeSum {
 
 constexpr int kNormPerThread = 8;
 
+// VEC consecutive elements as floats (VEC = 4: one 16-byte or 8-byte load).
+template <int VEC>
+__device__ __forceinline__ void load_vec(const float* p, float* f) {
+  if constexpr (VEC == 4) {
+    float4 v = *(const float4*)p;
+    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+  } else {
+    f[0] = p[0];
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void load_vec(const bf16* p, float* f) {
+  if constexpr (VEC == 4) {
+    uint2 v = *(const uint2*)p;   // four bf16: the upper halves of four floats
+    f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+  } else {
+    f[0] = to_f32(p[0]);
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void store_vec(float* p, const float* f) {
+  if constexpr (VEC == 4) *(float4*)p = make_float4(f[0], f[1], f[2], f[3]);
+  else p[0] = f[0];
+}
+template <int VEC>
+__device__ __forceinline__ void store_vec(bf16* p, const float* f) {
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) p[e] = __float2bfloat16(f[e]);
+}
+
 // y = (x [+ delta] [+ moe sum]) * rsqrt(mean(.^2) + eps) * gain  (reference
 // src/ops/kernels.hip:17-41 and :100-129). With rows == nullptr the sum is
 // written back to x; with rows the kernel reads row rows[i] and leaves x alone.
 // Every thread keeps its (at most 8) elements in registers between the two
-// passes; all loads of a thread are independent of each other, so they are in
-// flight together. The reduction order depends only on H and the block size,
-// never on the number of rows.
-template <typename T>
+// passes, in groups of VEC consecutive elements; all loads of a thread are
+// independent of each other, so they are in flight together. The reduction
+// order depends only on H, VEC and the block size, never on the number of rows.
+template <typename T, int VEC>
 __global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta, MoeSum ms,
                                const float* __restrict__ gain, T* __restrict__ out,
                                const int* __restrict__ rows, int H, float eps) {
+  constexpr int G = kNormPerThread / VEC;   // groups per thread
   __shared__ float red[16];
   int64_t r_out = blockIdx.x;
   int64_t r_in = rows ? rows[r_out] : r_out;
   float* xr = x + r_in * H;
   const T* dr = delta ? delta + r_in * H : nullptr;
   T* orow = out + r_out * H;
-  float vals[kNormPerThread];
+  float vals[G][VEC];
 #pragma unroll
-  for (int c = 0; c < kNormPerThread; ++c) {
-    int i = threadIdx.x + c * blockDim.x;
-    float v = 0.f;
+  for (int c = 0; c < G; ++c) {
+    int i = VEC * (threadIdx.x + c * blockDim.x);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) vals[c][e] = 0.f;
     if (i < H) {
-      v = xr[i];
-      if (dr) v += to_f32(dr[i]);
+      load_vec<VEC>(xr + i, vals[c]);
+      if (dr) {
+        float d[VEC];
+        load_vec<VEC>(dr + i, d);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) vals[c][e] += d[e];
+      }
     }
-    vals[c] = v;
   }
   if (ms.y) {
     const T* y = (const T*)ms.y + r_in * ms.k * H;
@@ -68,15 +105,23 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delt
 #pragma unroll
       for (int j = 0; j < 4; ++j) wj[j] = j0 + j < ms.k ? w[j0 + j] : 0.f;
 #pragma unroll
-      for (int c = 0; c < kNormPerThread; ++c) {
-        int i = threadIdx.x + c * blockDim.x;
+      for (int c = 0; c < G; ++c) {
+        int i = VEC * (threadIdx.x + c * blockDim.x);
         if (i < H) {
-          float yv[4];
+          float yv[4][VEC];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (j0 + j < ms.k) {
+              load_vec<VEC>(y + (int64_t)(j0 + j) * H + i, yv[j]);
+            } else {
+#pragma unroll
+              for (int e = 0; e < VEC; ++e) yv[j][e] = 0.f;
+            }
+          }
 #pragma unroll
           for (int j = 0; j < 4; ++j)
-            yv[j] = j0 + j < ms.k ? to_f32(y[(int64_t)(j0 + j) * H + i]) : 0.f;
 #pragma unroll
-          for (int j = 0; j < 4; ++j) vals[c] += wj[j] * yv[j];
+            for (int e = 0; e < VEC; ++e) vals[c][e] += wj[j] * yv[j][e];
         }
       }
     }
@@ -84,24 +129,35 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delt
       float g = ms.gate ? 1.f / (1.f + expf(-ms.gate[r_in * ms.gate_stride])) : 1.f;
       const T* sh = (const T*)ms.shared + r_in * H;
 #pragma unroll
-      for (int c = 0; c < kNormPerThread; ++c) {
-        int i = threadIdx.x + c * blockDim.x;
-        if (i < H) vals[c] += g * to_f32(sh[i]);
+      for (int c = 0; c < G; ++c) {
+        int i = VEC * (threadIdx.x + c * blockDim.x);
+        if (i < H) {
+          float sv[VEC];
+          load_vec<VEC>(sh + i, sv);
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) vals[c][e] += g * sv[e];
+        }
       }
     }
   }
   float acc = 0.f;
 #pragma unroll
-  for (int c = 0; c < kNormPerThread; ++c) acc += vals[c] * vals[c];
+  for (int c = 0; c < G; ++c)
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc += vals[c][e] * vals[c][e];
   float total = block_sum(acc, red);
   float inv = rsqrtf(total / (float)H + eps);
   const bool write_back = !rows && (dr || ms.y);
 #pragma unroll
-  for (int c = 0; c < kNormPerThread; ++c) {
-    int i = threadIdx.x + c * blockDim.x;
+  for (int c = 0; c < G; ++c) {
+    int i = VEC * (threadIdx.x + c * blockDim.x);
     if (i < H) {
-      if (write_back) xr[i] = vals[c];
-      orow[i] = from_f32<T>(vals[c] * inv * gain[i]);
+      if (write_back) store_vec<VEC>(xr + i, vals[c]);
+      float gv[VEC], o[VEC];
+      load_vec<VEC>(gain + i, gv);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) o[e] = vals[c][e] * inv * gv[e];
+      store_vec<VEC>(orow + i, o);
     }
   }
 }
@@ -237,17 +293,31 @@ extern "C" int ninfer_rmsnorm(float* x, const void* delta, const float* gain, vo
   NINFER_REQUIRE(H <= 1024 * kNormPerThread, "rmsnorm: width %d exceeds %d", H,
                  1024 * kNormPerThread);
   NINFER_REQUIRE(!moe_y || (moe_w && moe_k > 0), "rmsnorm: a row sum needs weights and k");
-  // few elements per thread: short chains of loads; at most 1024 threads
-  int block = (H / 2 + 63) / 64 * 64;
+  MoeSum ms{moe_y, moe_w, moe_shared, moe_gate, moe_gate_stride, moe_k};
+  // groups of 4 consecutive elements when every row pointer stays 16-byte aligned
+  auto aligned = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+  const bool vec = H % 4 == 0 && aligned(x) && aligned(delta) && aligned(out) && aligned(gain) &&
+                   aligned(moe_y) && aligned(moe_shared);
+  // few elements per thread (short chains of loads), at most 1024 threads
+  int per_thread = vec ? 4 : 2;
+  int block = ((H + per_thread - 1) / per_thread + 63) / 64 * 64;
   if (block < 64) block = 64;
   if (block > 1024) block = 1024;
-  MoeSum ms{moe_y, moe_w, moe_shared, moe_gate, moe_gate_stride, moe_k};
-  if (dtype == kF32)
-    rmsnorm_kernel<float><<<n_rows, block, 0, stream>>>(x, (const float*)delta, ms, gain,
-                                                       (float*)out, rows, H, eps);
-  else
-    rmsnorm_kernel<bf16><<<n_rows, block, 0, stream>>>(x, (const bf16*)delta, ms, gain, (bf16*)out,
-                                                      rows, H, eps);
+  if (dtype == kF32) {
+    if (vec)
+      rmsnorm_kernel<float, 4><<<n_rows, block, 0, stream>>>(x, (const float*)delta, ms, gain,
+                                                            (float*)out, rows, H, eps);
+    else
+      rmsnorm_kernel<float, 1><<<n_rows, block, 0, stream>>>(x, (const float*)delta, ms, gain,
+                                                            (float*)out, rows, H, eps);
+  } else {
+    if (vec)
+      rmsnorm_kernel<bf16, 4><<<n_rows, block, 0, stream>>>(x, (const bf16*)delta, ms, gain,
+                                                           (bf16*)out, rows, H, eps);
+    else
+      rmsnorm_kernel<bf16, 1><<<n_rows, block, 0, stream>>>(x, (const bf16*)delta, ms, gain,
+                                                           (bf16*)out, rows, H, eps);
+  }
   NINFER_LAUNCH_CHECK();
   return 0;
 }
