@@ -87,19 +87,19 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
   // A tile's keys and values travel global -> registers -> LDS; the next
   // tile's loads are issued before the products of the current one.
   constexpr int V_PER_THREAD = (V_BLOCKS + 255) / 256;
-  bf16x8 kreg[K_PER_THREAD], vreg[V_PER_THREAD][4];
+  bf16x8 kreg[2][K_PER_THREAD], vreg[2][V_PER_THREAD][4];
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  auto load_regs = [&](int t0) {
+  auto load_regs = [&](int st, int t0) {
 #pragma unroll
     for (int i = 0; i < K_PER_THREAD; ++i) {
       int vec = tid + i * 256;
       int key = vec / (D / 8), dv = vec % (D / 8);
       int kp = t0 + key;
-      kreg[i] = zero8;
+      kreg[st][i] = zero8;
       if (kp <= pos_last) {
         int page = bt[kp / ps];
         if (page >= 0)
-          kreg[i] = *(const bf16x8*)(kpool + (((int64_t)page * Hkv + g) * ps + kp % ps) * D + 8 * dv);
+          kreg[st][i] = *(const bf16x8*)(kpool + (((int64_t)page * Hkv + g) * ps + kp % ps) * D + 8 * dv);
       }
     }
 #pragma unroll
@@ -109,20 +109,20 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         int kp = t0 + 4 * kg + r;
-        vreg[i][r] = zero8;
+        vreg[st][i][r] = zero8;
         if (blk < V_BLOCKS && kp <= pos_last) {
           int page = bt[kp / ps];
           if (page >= 0)
-            vreg[i][r] = *(const bf16x8*)(vpool + (((int64_t)page * Hkv + g) * ps + kp % ps) * D + 8 * dv);
+            vreg[st][i][r] = *(const bf16x8*)(vpool + (((int64_t)page * Hkv + g) * ps + kp % ps) * D + 8 * dv);
         }
       }
     }
   };
-  auto store_regs = [&]() {
+  auto store_regs = [&](int st) {
 #pragma unroll
     for (int i = 0; i < K_PER_THREAD; ++i) {
       int vec = tid + i * 256;
-      *(bf16x8*)(k_s + (vec / (D / 8)) * KPAD + 8 * (vec % (D / 8))) = kreg[i];
+      *(bf16x8*)(k_s + (vec / (D / 8)) * KPAD + 8 * (vec % (D / 8))) = kreg[st][i];
     }
 #pragma unroll
     for (int i = 0; i < V_PER_THREAD; ++i) {
@@ -131,20 +131,20 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
         int kg = blk % (PK / 4), dv = blk / (PK / 4);
 #pragma unroll
         for (int d = 0; d < 8; ++d) {
-          bf16x4 col = {vreg[i][0][d], vreg[i][1][d], vreg[i][2][d], vreg[i][3][d]};
+          bf16x4 col = {vreg[st][i][0][d], vreg[st][i][1][d], vreg[st][i][2][d], vreg[st][i][3][d]};
           *(bf16x4*)(vt_s + (8 * dv + d) * VPAD + 4 * kg) = col;
         }
       }
     }
   };
 
-  const int t_first = (lo_first / PK) * PK;
-  load_regs(t_first);
-  for (int t0 = t_first; t0 <= pos_last; t0 += PK) {
+  // Tiles alternate between two register stages: the loads of tile t + 2 are
+  // issued as soon as tile t has moved to LDS, and are consumed two tiles later.
+  auto tile = [&](int st, int t0) {
     lds_barrier();   // the previous tile has been consumed
-    store_regs();
+    store_regs(st);
     lds_barrier();
-    if (t0 + PK <= pos_last) load_regs(t0 + PK);
+    if (t0 + 2 * PK <= pos_last) load_regs(st, t0 + 2 * PK);
 
     // S^T = K Q^T : 4 key blocks of 16
     f32x4 s[4];
@@ -197,6 +197,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
         o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[ks], o[db], 0, 0, 0);
       }
     }
+  };
+  const int t_first = (lo_first / PK) * PK;
+  load_regs(0, t_first);
+  if (t_first + PK <= pos_last) load_regs(1, t_first + PK);
+  for (int t0 = t_first; t0 <= pos_last; t0 += 2 * PK) {
+    tile(0, t0);
+    if (t0 + PK <= pos_last) tile(1, t0 + PK);
   }
 
   // the four lanes of a query hold partial sums of l

@@ -30,7 +30,7 @@ struct GemmArgs {
   int in_dtype;          // of A and W
   int out_dtype;         // of C
   int epilogue;
-  int big_rows;          // rows of a big grouped tile: 64 or 128 (0: 64)
+  int big_rows;          // rows of a big grouped tile: 64, 128 or 256 (0: 64)
 };
 
 // Which rows does tile `ti` of the grouped enumeration cover? Tiles of

@@ -1,0 +1,240 @@
+// C = A W^T for very many rows per weight matrix (bf16): 256 x 256 tiles, loaded
+// from global memory straight into LDS (global_load_lds_dwordx4), so that no
+// registers stage the tiles, in k tiles of 64 (whole 128-byte lines of every
+// row) and two buffers. Dense or grouped by expert, bias or SwiGLU epilogue, as
+// the staged kernel beside it; the reference sends these products to rocBLAS
+// (src/ops/linear.hip:21-35, src/models/model.hip:406-425).
+//
+// A block has 4 waves, one per SIMD, as a 2 x 2 grid; each wave owns 128 W rows
+// x 128 tokens = 4 x 4 tiles of v_mfma_f32_32x32x16_bf16 (256 accumulator
+// registers), which halves the LDS reads per product against 2 x 2 tiles.
+//
+// LDS rows are 128 bytes (64 bf16) and unpadded, because a wave's load writes
+// 1 KB contiguously (lane l at 16 l); the eight 16-byte chunks of row r are
+// stored in the order c ^ ((r / 2) % 8), chosen on the global side, so that the
+// 16 rows which one pass of a fragment read touches fall into 16 different
+// 16-byte columns of the banks.
+//
+// One barrier per k tile, before its last quarter: when a wave passes the
+// barrier of tile t, tile t + 1 has landed for every wave and every wave holds
+// the last fragments of tile t in registers, so the loads of tile t + 2 may
+// overwrite tile t. The fragments of every quarter are read while the products
+// of the quarter before run, across the barrier too.
+#include "gemm_tile.h"
+#include <type_traits>
+
+namespace ninfer {
+
+namespace direct {
+constexpr int TM = 256, TN = 256, TK = 64;
+constexpr int WGM = 2, WGN = 2;
+constexpr int COL = TM / WGN;             // staged token rows per wave column
+constexpr int FI = 4, FJ = 4;
+constexpr int NBUF = 2;
+constexpr int KK = TK / 16;                // quarters of a k tile: one MFMA depth each
+constexpr int ROW_BYTES = TK * 2;          // 128
+constexpr int X_BYTES = TM * ROW_BYTES;    // 32 KB
+constexpr int BUF_BYTES = (TM + TN) * ROW_BYTES;
+constexpr int LDS_BYTES = NBUF * BUF_BYTES;   // 128 KB
+}  // namespace direct
+
+#define NINFER_WAIT_LOADS(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
+
+template <bool SWIGLU, typename TC>
+__global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
+  using namespace direct;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  __shared__ int tile_info[3];
+
+  int bx, by;
+  block_to_tile(bx, by);
+  int row0, row_end, group;
+  if (!tile_rows<TM>(a, bx, tile_info, row0, row_end, group)) return;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave % WGM, wn = wave / WGM;
+  const int K = a.K, N = a.N;
+  const bf16* W = (const bf16*)a.W + (int64_t)group * a.w_group_stride;
+  constexpr int OUT_PER_BLOCK = SWIGLU ? TN / 2 : TN;
+  constexpr int OUT_PER_WAVE = OUT_PER_BLOCK / WGM;
+  const int out0 = by * OUT_PER_BLOCK;
+  const int rows_here = min(TM, row_end - row0);
+  // staged row l holds the tile's row (l % COL) * WGN + l / COL: column l / COL gets every WGN-th row
+  auto row_of = [&](int l) -> int { return (l % COL) * WGN + l / COL; };
+
+  // Loads: instruction i of wave w fills the 1 KB piece i * 4 + w of the X (and
+  // of the W) part of a buffer: 8 rows, lane l at row l / 8, stored chunk l % 8,
+  // which holds the row's chunk (l % 8) ^ ((row / 2) % 8); the piece's first row
+  // is a multiple of 8 and odd pieces belong to odd waves.
+  constexpr int NL = TM * ROW_BYTES / 1024 / 4;   // load instructions per wave, k tile and operand
+  const int chunk = (lane & 7) ^ ((((wave & 1) << 2) + (lane >> 4)) & 7);
+  const bf16* xsrc[NL];
+  const bf16* wsrc[NL];
+  int x_row[NL];
+#pragma unroll
+  for (int i = 0; i < NL; ++i) {
+    const int l = (i * 4 + wave) * 8 + (lane >> 3);
+    const int r = row_of(l);
+    // rows beyond the tile's last read its first row (one line, from L1): their results are
+    // never stored
+    x_row[i] = r < rows_here ? row0 + r : row0;
+    wsrc[i] = W + (int64_t)staged_w_row<TN, WGM, SWIGLU>(l, out0, N) * K + 8 * chunk;
+  }
+  if (a.a_index) {   // the index loads in flight together
+    int idx[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) idx[i] = a.a_index[x_row[i]];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) x_row[i] = idx[i] / a.a_div;
+  }
+#pragma unroll
+  for (int i = 0; i < NL; ++i) xsrc[i] = (const bf16*)a.A + (int64_t)x_row[i] * a.lda + 8 * chunk;
+  typedef const __attribute__((address_space(1))) void* gptr;
+  typedef __attribute__((address_space(3))) void* lptr;
+  auto issue = [&](int t) {   // k tile t into buffer t % NBUF
+    unsigned char* buf = smem + (t % NBUF) * BUF_BYTES + wave * 1024;
+#pragma unroll
+    for (int i = 0; i < NL; ++i)
+      __builtin_amdgcn_global_load_lds((gptr)(xsrc[i] + t * TK), (lptr)(buf + i * 4096), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < NL; ++i)
+      __builtin_amdgcn_global_load_lds((gptr)(wsrc[i] + t * TK), (lptr)(buf + X_BYTES + i * 4096), 16, 0, 0);
+  };
+
+  f32x16 acc[FI][FJ];
+#pragma unroll
+  for (int i = 0; i < FI; ++i)
+#pragma unroll
+    for (int jj = 0; jj < FJ; ++jj)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][jj][v] = 0.f;
+
+  // rows dealt to this wave's column, and its 32-row blocks that hold any
+  const int col_rows = rows_here > wn ? (rows_here - wn + WGN - 1) / WGN : 0;
+  const int n_jj = (col_rows + 31) / 32;
+  const int tok0 = wn * COL;
+
+  // fragment addresses: lane reads row lr of a 32-row block, k chunk 2 kk + lk, stored at
+  // chunk (2 kk + lk) ^ ((lr / 2) % 8) (the block's first row is a multiple of 16)
+  const int lr = lane & 31, lk = lane >> 5;
+  const int sw = (lr >> 1) & 7;
+  const int x_lane = (tok0 + lr) * ROW_BYTES;
+  const int w_lane = X_BYTES + (wm * (TN / WGM) + lr) * ROW_BYTES;
+  int c_quarter[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) c_quarter[kk] = 16 * ((2 * kk + lk) ^ sw);
+  const int nk = K / TK;
+
+  auto run = [&](auto nj_tag) {
+    constexpr int NJ = decltype(nj_tag)::value;
+    constexpr int NX = NJ > 0 ? NJ : 1;
+    bf16x8 wf[2][FI], xf[2][NX];
+    auto read_quarter = [&](int set, int t, int kk) {
+      if constexpr (NJ == 0) return;
+      const unsigned char* buf = smem + (t % NBUF) * BUF_BYTES + c_quarter[kk];
+#pragma unroll
+      for (int i = 0; i < FI; ++i) wf[set][i] = *(const bf16x8*)(buf + w_lane + i * 32 * ROW_BYTES);
+#pragma unroll
+      for (int jj = 0; jj < NJ; ++jj) xf[set][jj] = *(const bf16x8*)(buf + x_lane + jj * 32 * ROW_BYTES);
+    };
+    auto multiply = [&](int set) {
+#pragma unroll
+      for (int jj = 0; jj < NJ; ++jj)
+#pragma unroll
+        for (int i = 0; i < FI; ++i)
+          acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[set][i], xf[set][jj], acc[i][jj], 0, 0, 0);
+    };
+    // The order of a quarter: every fragment read of the next quarter goes between two
+    // products of this one, so that it has returned when its products begin.
+    auto interleave = [&]() {
+#pragma unroll
+      for (int i = 0; i < FI + NJ; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, FI * NJ > FI + NJ ? FI * NJ - FI - NJ : 0, 0);
+    };
+    // tiles 0 and 1 on their way, tile 0 landed
+    issue(0);
+    if (nk > 1) issue(1);
+    if (nk > 1) NINFER_WAIT_LOADS(16); else NINFER_WAIT_LOADS(0);
+    __builtin_amdgcn_s_barrier();
+    read_quarter(0, 0, 0);
+    int t = 0;
+    // steady state, free of conditions: tiles t + 1 and t + 2 exist
+    for (; t + 2 < nk; ++t) {
+#pragma unroll
+      for (int kk = 0; kk + 1 < KK; ++kk) {
+        read_quarter((kk + 1) & 1, t, kk + 1);
+        multiply(kk & 1);
+        interleave();
+      }
+      // this wave's loads of tile t + 1 have landed and its last fragments of tile t are in
+      // registers; after the barrier that holds for every wave
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      issue(t + 2);
+      read_quarter(KK & 1, t + 1, 0);
+      multiply((KK - 1) & 1);
+      interleave();
+    }
+    // the last two tiles
+    for (; t < nk; ++t) {
+#pragma unroll
+      for (int kk = 0; kk + 1 < KK; ++kk) {
+        read_quarter((kk + 1) & 1, t, kk + 1);
+        multiply(kk & 1);
+      }
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      if (t + 1 < nk) read_quarter(KK & 1, t + 1, 0);
+      multiply((KK - 1) & 1);
+    }
+  };
+  // one straight-line instance per count of live token blocks
+  switch (n_jj) {
+    case 0: run(std::integral_constant<int, 0>{}); break;
+    case 1: run(std::integral_constant<int, 1>{}); break;
+    case 2: run(std::integral_constant<int, 2>{}); break;
+    case 3: run(std::integral_constant<int, 3>{}); break;
+    default: run(std::integral_constant<int, 4>{}); break;
+  }
+  __syncthreads();   // every wave has read its last fragments: the buffers become the epilogue's stage
+  write_tile<FI, FJ, SWIGLU, TC>(a, acc, smem + wave * (FJ * 32 * FI * 64), tok0, row0, rows_here,
+                                 out0 + OUT_PER_WAVE * wm, row_of);
+}
+
+#undef NINFER_WAIT_LOADS
+
+bool gemm_tile_direct_takes(const GemmArgs& a) {
+  return a.in_dtype == kBF16 && a.K % direct::TK == 0 && a.lda % 8 == 0 &&
+         ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0) && a.w_group_stride % 8 == 0;
+}
+
+int gemm_tile_direct(const GemmArgs& a, hipStream_t stream) {
+  using namespace direct;
+  if (a.offsets && a.tiles64 && a.big_rows != TM)
+    return set_error(-1, "gemm: the grouped tile lists are made for %d rows, not %d", a.big_rows, TM);
+  const bool swiglu = a.epilogue == kEpilogueSwiGLU;
+  const int m_tiles = (a.M + TM - 1) / TM + (a.offsets ? a.groups : 0);
+  const int per_block = swiglu ? TN / 2 : TN;
+  const dim3 grid(m_tiles, (a.N + per_block - 1) / per_block);
+#define NINFER_DIRECT_LAUNCH(SW, TYPE)                                                          \
+  do {                                                                                          \
+    auto kern = gemm_tile_direct_kernel<SW, TYPE>;                                              \
+    hipError_t e = hipFuncSetAttribute((const void*)kern,                                       \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);  \
+    if (e != hipSuccess) return set_error(-2, "gemm: cannot get %d bytes of LDS", LDS_BYTES);   \
+    kern<<<grid, 256, LDS_BYTES, stream>>>(a);                                                  \
+  } while (0)
+  if (a.out_dtype == kF32) {
+    if (swiglu) NINFER_DIRECT_LAUNCH(true, float); else NINFER_DIRECT_LAUNCH(false, float);
+  } else {
+    if (swiglu) NINFER_DIRECT_LAUNCH(true, bf16); else NINFER_DIRECT_LAUNCH(false, bf16);
+  }
+#undef NINFER_DIRECT_LAUNCH
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace ninfer

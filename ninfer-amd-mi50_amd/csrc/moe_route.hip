@@ -186,11 +186,11 @@ extern "C" int ninfer_router_topk(const float* logits, int ld, int T, int E, int
 
 // tiles16 / tiles64 / tile_counts may be null (no tile lists). tiles16 holds
 // 4 ints for each of up to min(n, n / 16 + E) tiles of 16 rows, tiles64 for up
-// to n / 64 + E tiles of big_rows (64 or 128) rows.
+// to n / 64 + E tiles of big_rows (64, 128 or 256) rows.
 extern "C" int ninfer_moe_align(const int* ids, int n, int E, int* offsets, int* order,
                                 int* tiles16, int* tiles64, int* tile_counts, int big_rows,
                                 hipStream_t stream) {
-  NINFER_REQUIRE(big_rows == 64 || big_rows == 128, "moe_align: big tiles of %d rows", big_rows);
+  NINFER_REQUIRE(big_rows == 64 || big_rows == 128 || big_rows == 256, "moe_align: big tiles of %d rows", big_rows);
   NINFER_REQUIRE(n > 0 && E > 0, "moe_align: n=%d E=%d must be positive", n, E);
   NINFER_REQUIRE(E <= 8192, "moe_align: %d experts exceed 8192", E);
   NINFER_REQUIRE((!tiles16) == (!tiles64) && (!tiles16) == (!tile_counts),
@@ -206,7 +206,7 @@ extern "C" int ninfer_moe_route_small(const float* logits, int ld, int T, int E,
                                       int renorm, int* ids, float* wts, int* offsets, int* order,
                                       int* tiles16, int* tiles64, int* tile_counts, int big_rows,
                                       hipStream_t stream) {
-  NINFER_REQUIRE(big_rows == 64 || big_rows == 128, "moe_route_small: big tiles of %d rows",
+  NINFER_REQUIRE(big_rows == 64 || big_rows == 128 || big_rows == 256, "moe_route_small: big tiles of %d rows",
                  big_rows);
   NINFER_REQUIRE(T > 0 && T <= 256, "moe_route_small: T=%d not in [1, 256]", T);
   NINFER_REQUIRE(E > 0 && E <= 64 * kMaxExpertsPerLane, "moe_route_small: %d experts exceed %d", E,

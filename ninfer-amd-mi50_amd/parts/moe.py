@@ -55,9 +55,20 @@ class SoftmaxTopKRouter(Part):
                     tiles16=ctx.empty((min(n, n // 16 + e), 4), torch.int32),
                     tiles64=ctx.empty((n // 64 + e, 4), torch.int32),
                     tile_counts=ctx.empty((2,), torch.int32),
-                    big_rows=128 if n >= 96 * e else 64)
+                    big_rows=big_tile_rows(n, e))
         ctx.ops.moe_route(logits, e, k, self.renorm, r)
         return r
+
+
+def big_tile_rows(routed_rows: int, experts: int) -> int:
+    """Rows of the big tiles of the grouped products: the taller, the fewer times an
+    expert's weights are read, but a tile that is mostly empty still costs its
+    loads. Thresholds on the mean rows per expert, from measurement."""
+    if routed_rows >= 128 * experts:
+        return 256
+    if routed_rows >= 48 * experts:
+        return 128
+    return 64
 
 
 class Routing:
@@ -69,7 +80,7 @@ class Routing:
                  big_rows=64):
         self.ids, self.weights, self.offsets, self.order = ids, weights, offsets, order
         self.tiles16, self.tiles64, self.tile_counts = tiles16, tiles64, tile_counts
-        self.big_rows = big_rows   # rows of a tile in `tiles64`: 64, or 128 when experts get many rows
+        self.big_rows = big_rows   # rows of a tile in `tiles64`: 64, 128 or 256 (big_tile_rows)
 
 
 class RoutedExperts(Part):

@@ -114,11 +114,14 @@ def test_swiglu_linear(ops_mode, gen, dtype, m, inner, k):
     close(o1, o2, dtype, scale=k * 0.3)
 
 
-@pytest.mark.parametrize("variant", [1, 2])
-@pytest.mark.parametrize("m,n,k", [(333, 700, 256), (70, 130, 384), (129, 1000, 512)])
-def test_tile_product_both_tile_heights(ops, gen, variant, m, n, k):
-    """The many-row kernel with 64-row and with 128-row tiles (tile counts that
-    are no multiple of the 8 XCDs, rows that end inside a tile)."""
+@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("m,n,k", [(333, 700, 256), (70, 130, 384), (129, 1000, 512), (600, 520, 320),
+                                   (257, 264, 64), (40, 36, 128)])
+def test_tile_product_every_tile_height(ops, gen, variant, m, n, k):
+    """The many-row kernels with 64-row, 128-row and 256-row tiles (tile counts
+    that are no multiple of the 8 XCDs, rows that end inside a tile, one to five
+    k tiles of the 256-row kernel's pipeline, widths that are and are not a
+    multiple of 8: both epilogues)."""
     ops.lib.ninfer_set_tile_variant(variant)
     try:
         x, w = rnd((m, k), torch.bfloat16, gen), rnd((n, k), torch.bfloat16, gen)
@@ -202,17 +205,18 @@ def test_router_align_experts_combine(ops_mode, gen, dtype, t, e, k, h, inner):
     from ninfer_amd.parts.moe import Routing
     n = t * k
     i32 = lambda *sh: torch.zeros(*sh, device="cuda", dtype=torch.int32)
-    tl = Routing(ids1, w1, off1, i32(n), i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2),
-                 big_rows=128 if n >= 96 * e else 64)
-    ops.moe_align(ids1, e, i32(e + 1), tl.order, tiles=tl)
-    h3 = torch.zeros_like(h1)
-    ops.grouped_swiglu(x, wgu, off1, tl.order, k, h3, tiles=tl)
-    y3 = torch.zeros_like(y1)
-    ops.grouped_down(h3, wd, off1, tl.order, y3, tiles=tl)
-    y4 = torch.zeros_like(y1)
-    plain.grouped_down(h3, wd, off1, tl.order, y4)
-    close(y3, y4, dtype, scale=h2.float().abs().max().item() * math.sqrt(inner) * 0.3)
-    close(y3, y2, dtype, scale=h2.float().abs().max().item() * math.sqrt(inner) * 0.3)
+    for big in (64, 128, 256):   # every height of the big tiles, whatever the rows per expert
+        tl = Routing(ids1, w1, off1, i32(n), i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2),
+                     big_rows=big)
+        ops.moe_align(ids1, e, i32(e + 1), tl.order, tiles=tl)
+        h3 = torch.zeros_like(h1)
+        ops.grouped_swiglu(x, wgu, off1, tl.order, k, h3, tiles=tl)
+        y3 = torch.zeros_like(y1)
+        ops.grouped_down(h3, wd, off1, tl.order, y3, tiles=tl)
+        y4 = torch.zeros_like(y1)
+        plain.grouped_down(h3, wd, off1, tl.order, y4)
+        close(y3, y4, dtype, scale=h2.float().abs().max().item() * math.sqrt(inner) * 0.3)
+        close(y3, y2, dtype, scale=h2.float().abs().max().item() * math.sqrt(inner) * 0.3)
     shared = rnd((t, h), dtype, gen)
     gate = torch.randn(t, 1, generator=gen, device="cuda")
     r1 = torch.randn(t, h, generator=gen, device="cuda")
@@ -239,7 +243,7 @@ def test_routing_in_one_call_with_tile_lists(ops, gen, t, e, k):
         i32 = lambda *s: torch.zeros(*s, device="cuda", dtype=torch.int32)
         return Routing(i32(t, k), torch.zeros(t, k, device="cuda"), i32(e + 1), i32(n),
                        i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2),
-                       big_rows=128 if t >= 300 else 64)
+                       big_rows=256 if t >= 1000 else 128 if t >= 300 else 64)
     r1, r2 = routing(), routing()
     ops.moe_route(logits, e, k, True, r1)
     PlainOps().moe_route(logits, e, k, True, r2)
