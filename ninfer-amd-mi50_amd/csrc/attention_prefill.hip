@@ -1,15 +1,20 @@
 // Paged attention for prompt portions (bf16) on the matrix cores.
 //
-// One block of 4 waves owns 64 consecutive rows of one request and one query
-// head; each wave owns 16 of the rows. Keys and values are walked in tiles of
+// One block owns NQ * 32 consecutive rows of one request and one query head
+// (128 or 64 rows: every key and value it loads serves that many). It has
+// 2 NQ waves: rows are dealt to NQ groups of 32, and two waves share a group,
+// one for the first and one for the second 32 keys of every tile, each with a
+// running max, sum and output of its own that are merged at the end. So every
+// SIMD holds two waves, and the softmax arithmetic of one overlaps the matrix
+// products of the other. Keys and values are walked in tiles of
 // 64 aligned to absolute positions, through LDS: K as stored ([key][d]), V
 // transposed ([d][key]) so that both products read their contraction index
-// contiguously. With v_mfma_f32_16x16x32_bf16 the wave computes
+// contiguously. With v_mfma_f32_32x32x16_bf16 the wave computes
 //   S^T[key][q] = K Q^T      (A = K rows from LDS, B = Q held in registers)
-// whose accumulator layout gives lane l the scores of query l % 16 for keys
-// 4 (l / 16) + v of every 16-key block: the softmax of a query runs in the four
-// lanes that share l % 16 (two cross-lane steps), and the probabilities, packed
-// to bf16 in place, are already the B operand of
+// whose accumulator layout gives lane l the scores of query l % 32 for keys
+// 8 (v / 4) + 4 (l / 32) + v % 4 of every 32-key block: the softmax of a query
+// runs in the two lanes that share l % 32 (one cross-lane step), and the
+// probabilities, packed to bf16 in place, are already the B operand of
 //   O^T[d][q] += V^T P^T     (A = V^T rows from LDS)
 // if the contraction index is numbered the way the lanes hold it; so
 // probabilities never leave registers, and the running max and sum of a query
@@ -28,19 +33,27 @@ namespace ninfer {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int PQ = 64;   // query rows per block
 constexpr int PK = 64;   // keys per tile
 
-template <int D>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
-  constexpr int KS = D / 32;        // k-steps of Q K^T
-  constexpr int DB = D / 16;        // 16-row blocks of O^T
+template <int D, int NQ>
+__global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
+  constexpr int KH = 2;             // waves per group of 32 rows: each meets one half of a tile's keys
+  constexpr int NT = NQ * KH * 64;
+  constexpr int NKB = 2 / KH;       // 32-key blocks of a tile that one wave meets
+  constexpr int PQ = NQ * 32;       // query rows per block
+  constexpr int KS = D / 16;        // k-steps of Q K^T
+  constexpr int DB = D / 32;        // 32-row blocks of O^T
   constexpr int KPAD = D + 8;       // bf16 per K row in LDS
-  constexpr int VPAD = PK + 8;      // bf16 per V^T row in LDS
-  __shared__ __attribute__((aligned(16))) bf16 k_s[PK * KPAD];
-  __shared__ __attribute__((aligned(16))) bf16 vt_s[D * VPAD];
+  constexpr int VPAD = PK + 4;      // bf16 per V^T row in LDS: 8-byte reads of 32 rows spread over the banks
+  constexpr int K_TILE = PK * KPAD, V_TILE = D * VPAD;   // bf16 of a tile in LDS
+  constexpr int MERGE = 2 + DB * 16 + 1;                   // floats a lane hands over at the end (odd stride)
+  constexpr int TILES_BYTES = 2 * (K_TILE + V_TILE) * 2, MERGE_BYTES = NQ * 64 * MERGE * 4;
+  // two tiles of each (one read, one written); at the end the same memory merges the two key halves
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[TILES_BYTES > MERGE_BYTES ? TILES_BYTES : MERGE_BYTES];
+  bf16* const k_lds = (bf16*)lds_raw;                  // [2][K_TILE]
+  bf16* const vt_lds = k_lds + 2 * K_TILE;             // [2][V_TILE]
   __shared__ int tile_info[3];
 
   if (!find_tile(a.seq_row_start, a.S, PQ, blockIdx.x, tile_info)) return;
@@ -48,7 +61,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
   const int h = blockIdx.y;
   const int g = h / (a.Hq / a.Hkv);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int c = lane & 15, j = lane >> 4;
+  const int c = lane & 31, j = lane >> 5;
 
   const int pos_first = a.positions[row0];               // rows of a request are consecutive
   const int n_rows = min(PQ, row_end - row0);
@@ -57,76 +70,102 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
   const int* bt = a.block_table + (int64_t)seq * a.bt_stride;
   const bf16* kpool = (const bf16*)a.kpool;
   const bf16* vpool = (const bf16*)a.vpool;
-  const int ps = a.page_size, Hkv = a.Hkv;
+  // the page size divides the tile of 64 keys: a power of two
+  const int ps_shift = __builtin_ctz(a.page_size), ps_mask = a.page_size - 1, Hkv = a.Hkv;
 
-  // this lane's query (B operand): row q = wave * 16 + c, dims 32 ks + 8 j .. +7
-  const int q_local = wave * 16 + c;
+  // this lane's query (B operand): row q = qg * 32 + c, dims 16 ks + 8 j .. +7; the wave
+  // meets the 32 NKB keys from 32 NKB kh of every tile
+  const int qg = wave % NQ, kh = wave / NQ;
+  const int q_local = qg * 32 + c;
   const bool q_valid = q_local < n_rows;
+  const bool wave_live = qg * 32 < n_rows;    // a wave without rows only helps to load
   const int q_pos = pos_first + q_local;
   const int q_lo = a.window > 0 ? max(0, q_pos - a.window + 1) : 0;
+  // keys this wave's rows can see: tiles outside are loaded for the others but not multiplied
+  const int wave_pos_last = pos_first + min(qg * 32 + 31, n_rows - 1);
+  const int wave_lo = a.window > 0 ? max(0, pos_first + qg * 32 - a.window + 1) : 0;
   bf16x8 qf[KS];
   {
     const bf16* qr = (const bf16*)a.q + (int64_t)(row0 + (q_valid ? q_local : 0)) * a.q_stride +
                      h * D + 8 * j;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const bf16x8*)(qr + 32 * ks);
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const bf16x8*)(qr + 16 * ks);
   }
 
-  f32x4 o[DB];
+  f32x16 o[DB];
 #pragma unroll
-  for (int db = 0; db < DB; ++db) o[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
+  // scores are kept in units of log 2, so that a probability is one v_exp_f32
+  const float scale2 = a.scale * 1.44269504088896f;
   float m = -1e30f, l = 0.f;
 
   // global -> LDS mapping. K: thread loads 16 bytes (8 dims) of a key row.
   // V: thread loads a 4-key x 8-dim block and stores it transposed.
   constexpr int K_VECS = PK * D / 8;                  // 16-byte vectors in a K tile
-  constexpr int K_PER_THREAD = K_VECS / 256;
+  constexpr int K_PER_THREAD = (K_VECS + NT - 1) / NT;
   constexpr int V_BLOCKS = (PK / 4) * (D / 8);        // 4 x 8 blocks in a V tile
-  static_assert(K_VECS % 256 == 0, "tile does not divide over the block");
+  constexpr int V_PER_THREAD = (V_BLOCKS + NT - 1) / NT;
+  static_assert(K_VECS % NT == 0, "tile does not divide over the block");
 
-  // A tile's keys and values travel global -> registers -> LDS; the next
-  // tile's loads are issued before the products of the current one.
-  constexpr int V_PER_THREAD = (V_BLOCKS + 255) / 256;
+  // A tile's keys and values travel global -> registers -> LDS. Tile i is
+  // multiplied from LDS buffer i % 2 while tile i + 1 moves from its registers to
+  // the other buffer, the loads of tile i + 3 are issued into those registers,
+  // and the page numbers of tile i + 5 are fetched: no load waits for another
+  // inside the loop.
   bf16x8 kreg[2][K_PER_THREAD], vreg[2][V_PER_THREAD][4];
+  int kpage[2][K_PER_THREAD], vpage[2][V_PER_THREAD];
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  auto load_regs = [&](int st, int t0) {
+  // Every load below is unconditional (a select replaces what is not there by zeros): a
+  // load under a condition would have to be waited for where the condition ends.
+  auto load_pages = [&](int st, int t0) {
 #pragma unroll
     for (int i = 0; i < K_PER_THREAD; ++i) {
-      int vec = tid + i * 256;
-      int key = vec / (D / 8), dv = vec % (D / 8);
-      int kp = t0 + key;
-      kreg[st][i] = zero8;
-      if (kp <= pos_last) {
-        int page = bt[kp / ps];
-        if (page >= 0)
-          kreg[st][i] = *(const bf16x8*)(kpool + (((int64_t)page * Hkv + g) * ps + kp % ps) * D + 8 * dv);
-      }
+      int kp = t0 + (tid + i * NT) / (D / 8);
+      kpage[st][i] = bt[min(kp, pos_last) >> ps_shift];   // always a table entry of the request
     }
 #pragma unroll
     for (int i = 0; i < V_PER_THREAD; ++i) {
-      int blk = tid + i * 256;
+      int blk = (tid + i * NT) % V_BLOCKS;     // threads beyond the tile repeat a block and store nothing
+      int kp = t0 + 4 * (blk % (PK / 4));      // four keys of one page (the page size is a multiple of 4)
+      vpage[st][i] = bt[min(kp, pos_last) >> ps_shift];
+    }
+  };
+  auto load_regs = [&](int st, int t0) {
+#pragma unroll
+    for (int i = 0; i < K_PER_THREAD; ++i) {
+      int vec = tid + i * NT;
+      int kp = t0 + vec / (D / 8), dv = vec % (D / 8);
+      // a key that is not there is read from the pool's first page and replaced by zeros
+      const int page = kpage[st][i];
+      const bf16x8 got = *(const bf16x8*)(kpool + ((((int64_t)max(page, 0) * Hkv + g) << ps_shift) + (kp & ps_mask)) * D + 8 * dv);
+      kreg[st][i] = (page >= 0 && kp <= pos_last) ? got : zero8;
+    }
+#pragma unroll
+    for (int i = 0; i < V_PER_THREAD; ++i) {
+      int blk = (tid + i * NT) % V_BLOCKS;
       int kg = blk % (PK / 4), dv = blk / (PK / 4);
+      const int page = vpage[st][i];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         int kp = t0 + 4 * kg + r;
-        vreg[st][i][r] = zero8;
-        if (blk < V_BLOCKS && kp <= pos_last) {
-          int page = bt[kp / ps];
-          if (page >= 0)
-            vreg[st][i][r] = *(const bf16x8*)(vpool + (((int64_t)page * Hkv + g) * ps + kp % ps) * D + 8 * dv);
-        }
+        const bf16x8 got = *(const bf16x8*)(vpool + ((((int64_t)max(page, 0) * Hkv + g) << ps_shift) + (kp & ps_mask)) * D + 8 * dv);
+        vreg[st][i][r] = (page >= 0 && kp <= pos_last) ? got : zero8;
       }
     }
   };
-  auto store_regs = [&](int st) {
+  auto store_regs = [&](int st, int buf) {
+    bf16* k_s = k_lds + buf * K_TILE;
+    bf16* vt_s = vt_lds + buf * V_TILE;
 #pragma unroll
     for (int i = 0; i < K_PER_THREAD; ++i) {
-      int vec = tid + i * 256;
+      int vec = tid + i * NT;
       *(bf16x8*)(k_s + (vec / (D / 8)) * KPAD + 8 * (vec % (D / 8))) = kreg[st][i];
     }
 #pragma unroll
     for (int i = 0; i < V_PER_THREAD; ++i) {
-      int blk = tid + i * 256;
+      int blk = tid + i * NT;
       if (blk < V_BLOCKS) {
         int kg = blk % (PK / 4), dv = blk / (PK / 4);
 #pragma unroll
@@ -138,86 +177,135 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     }
   };
 
-  // Tiles alternate between two register stages: the loads of tile t + 2 are
-  // issued as soon as tile t has moved to LDS, and are consumed two tiles later.
-  auto tile = [&](int st, int t0) {
-    lds_barrier();   // the previous tile has been consumed
-    store_regs(st);
-    lds_barrier();
-    if (t0 + 2 * PK <= pos_last) load_regs(st, t0 + 2 * PK);
-
-    // S^T = K Q^T : 4 key blocks of 16
-    f32x4 s[4];
+  // the products of this wave's part of the tile at keys t0.. in LDS buffer buf
+  auto multiply = [&](int buf, int t0) {
+    const int k0 = t0 + 32 * NKB * kh;
+    // not for tiles beyond the last key, or out of sight of every row of the wave
+    if (!wave_live || k0 > wave_pos_last || k0 + 32 * NKB <= wave_lo) return;
+    const bf16* k_s = k_lds + buf * K_TILE;
+    const bf16* vt_s = vt_lds + buf * V_TILE;
+    // S^T = K Q^T : NKB key blocks of 32 x 32 queries
+    f32x16 s[NKB];
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-      s[kb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int kb = 0; kb < NKB; ++kb) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        bf16x8 kf = *(const bf16x8*)(k_s + (kb * 16 + c) * KPAD + 32 * ks + 8 * j);
-        s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], s[kb], 0, 0, 0);
+        bf16x8 kf = *(const bf16x8*)(k_s + ((NKB * kh + kb) * 32 + c) * KPAD + 16 * ks + 8 * j);
+        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s[kb], 0, 0, 0);
       }
     }
-    // lane holds, for query c, keys t0 + 16 kb + 4 j + v
+    // lane holds, for query c, keys k0 + 32 kb + 8 (v / 4) + 4 j + v % 4
     float mx = -1e30f;
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
+    for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        int kp = t0 + 16 * kb + 4 * j + v;
-        float val = (kp <= q_pos && kp >= q_lo) ? s[kb][v] * a.scale : -1e30f;
+      for (int v = 0; v < 16; ++v) {
+        int kp = k0 + 32 * kb + 8 * (v >> 2) + 4 * j + (v & 3);
+        float val = (kp <= q_pos && kp >= q_lo) ? s[kb][v] * scale2 : -1e30f;
         s[kb][v] = val;
         mx = fmaxf(mx, val);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m, mx);
-    const float alpha = __expf(m - m_new);
+    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
     float psum = 0.f;
-    bf16x8 pf[2];
+    // pf[kb][h]: the 16-key step h of key block kb; slot i of lane j is key 16 h + 8 (i / 4) + 4 j + i % 4
+    bf16x8 pf[NKB][2];
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
+    for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        float p = __expf(s[kb][v] - m_new);
+      for (int v = 0; v < 16; ++v) {
+        float p = __builtin_amdgcn_exp2f(s[kb][v] - m_new);
         psum += p;
-        pf[kb >> 1][(kb & 1) * 4 + v] = (__bf16)p;
+        pf[kb][v >> 3][v & 7] = (__bf16)p;
       }
     l = l * alpha + psum;
+    // the output needs rescaling only when some row's maximum has moved
+    const bool moved = __any(m_new > m);
     m = m_new;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      o[db] *= alpha;
-      // contraction slot (j, i): key 32 ks + 4 j + i for i < 4, 32 ks + 16 + 4 j + i - 4 else
+      if (moved) o[db] *= alpha;
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        const bf16* vr = vt_s + (db * 16 + c) * VPAD + 32 * ks + 4 * j;
-        bf16x4 lo4 = *(const bf16x4*)vr;
-        bf16x4 hi4 = *(const bf16x4*)(vr + 16);
-        bf16x8 vf = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[ks], o[db], 0, 0, 0);
-      }
+      for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+        for (int hs = 0; hs < 2; ++hs) {
+          const bf16* vr = vt_s + (db * 32 + c) * VPAD + 32 * (NKB * kh + kb) + 16 * hs + 4 * j;
+          bf16x4 lo4 = *(const bf16x4*)vr;
+          bf16x4 hi4 = *(const bf16x4*)(vr + 8);
+          bf16x8 vf = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kb][hs], o[db], 0, 0, 0);
+        }
     }
   };
+
   const int t_first = (lo_first / PK) * PK;
+  load_pages(0, t_first);
+  load_pages(1, t_first + PK);
   load_regs(0, t_first);
-  if (t_first + PK <= pos_last) load_regs(1, t_first + PK);
+  load_regs(1, t_first + PK);
+  load_pages(0, t_first + 2 * PK);
+  load_pages(1, t_first + 3 * PK);
+  store_regs(0, 0);
+  load_regs(0, t_first + 2 * PK);
+  load_pages(0, t_first + 4 * PK);
+  lds_barrier();
+  // Two tiles per turn, so that the register stage and the buffer of each are constants.
+  // Nothing in the loop stands under a condition: tiles beyond the last key are loaded as
+  // zeros and skipped by the products, so the wait before a store counts exactly the loads
+  // issued after the ones it needs.
   for (int t0 = t_first; t0 <= pos_last; t0 += 2 * PK) {
-    tile(0, t0);
-    if (t0 + PK <= pos_last) tile(1, t0 + PK);
+    store_regs(1, 1);
+    load_regs(1, t0 + 3 * PK);
+    load_pages(1, t0 + 5 * PK);
+    multiply(0, t0);
+    lds_barrier();   // tile t0 + PK is whole, tile t0 has been read by every wave
+    store_regs(0, 0);
+    load_regs(0, t0 + 4 * PK);
+    load_pages(0, t0 + 6 * PK);
+    multiply(1, t0 + PK);
+    lds_barrier();
   }
 
-  // the four lanes of a query hold partial sums of l
-  l += __shfl_xor(l, 16, 64);
+  // Merge the two key halves of every row group: the waves of the second half hand their
+  // max, sum and output over through LDS (the last barrier of the loop has freed it).
+  float* mine = (float*)lds_raw + (qg * 64 + lane) * MERGE;
+  if (kh == 1) {
+    mine[0] = m;
+    mine[1] = l;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) mine[2 + 16 * db + v] = o[db][v];
+  }
+  __syncthreads();
+  if (kh == 1) return;
+  {
+    const float m1 = mine[0], l1 = mine[1];
+    const float m_all = fmaxf(m, m1);
+    const float a0 = __builtin_amdgcn_exp2f(m - m_all), a1 = __builtin_amdgcn_exp2f(m1 - m_all);
+    l = l * a0 + l1 * a1;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[db][v] = o[db][v] * a0 + mine[2 + 16 * db + v] * a1;
+  }
+  // the two lanes of a query hold partial sums of l
   l += __shfl_xor(l, 32, 64);
   if (q_valid) {
+    // lane holds, of its query's output, dims 32 db + 8 (v / 4) + 4 j + v % 4
     const float inv = 1.f / l;
     bf16* orow = (bf16*)a.out + ((int64_t)(row0 + q_local) * a.Hq + h) * D;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      bf16x4 val = {(__bf16)(o[db][0] * inv), (__bf16)(o[db][1] * inv), (__bf16)(o[db][2] * inv),
-                    (__bf16)(o[db][3] * inv)};
-      *(bf16x4*)(orow + db * 16 + 4 * j) = val;
-    }
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        bf16x4 val = {(__bf16)(o[db][4 * qd] * inv), (__bf16)(o[db][4 * qd + 1] * inv),
+                      (__bf16)(o[db][4 * qd + 2] * inv), (__bf16)(o[db][4 * qd + 3] * inv)};
+        *(bf16x4*)(orow + db * 32 + 8 * qd + 4 * j) = val;
+      }
   }
 }
 
@@ -226,14 +314,22 @@ bool attention_prefill_takes(const AttnArgs& a) {
          PK % a.page_size == 0 && a.seq_row_start != nullptr;
 }
 
-int attention_prefill(const AttnArgs& a, hipStream_t stream) {
+template <int NQ>
+static int launch_prefill(const AttnArgs& a, hipStream_t stream) {
+  constexpr int PQ = NQ * 32;
   dim3 grid((a.T + PQ - 1) / PQ + a.S, a.Hq);
   if (a.D == 128)
-    attn_prefill_kernel<128><<<grid, 256, 0, stream>>>(a);
+    attn_prefill_kernel<128, NQ><<<grid, NQ * 128, 0, stream>>>(a);
   else
-    attn_prefill_kernel<64><<<grid, 256, 0, stream>>>(a);
+    attn_prefill_kernel<64, NQ><<<grid, NQ * 128, 0, stream>>>(a);
   NINFER_LAUNCH_CHECK();
   return 0;
+}
+
+int attention_prefill(const AttnArgs& a, hipStream_t stream) {
+  // 128 rows per block when requests bring that many: every key loaded serves more rows
+  if (a.max_qlen > 64) return launch_prefill<4>(a, stream);
+  return launch_prefill<2>(a, stream);
 }
 
 }  // namespace ninfer
