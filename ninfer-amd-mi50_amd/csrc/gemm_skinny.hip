@@ -13,6 +13,11 @@
 // rows), weights stream through registers with four 16-byte loads in flight
 // per lane and chunk.
 //
+// A dense product whose 16-feature tiles would be few is cut into tiles of
+// fewer features (some of each matrix instruction's rows stay empty, which
+// costs nothing where the weights' way into the CUs is the bound), so that the
+// blocks are a whole multiple of the CUs and all CUs pull equally.
+//
 // Grouped form as in the plain kernel: tiles of 16 sorted rows per expert are
 // enumerated from the device-side offsets; a block whose tile does not exist
 // exits. The reference runs these products as one GEMV per row (decode,
@@ -27,8 +32,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int SM = 16;  // rows of A per tile
 
-template <int WAVES, bool SWIGLU, typename TC>
-__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a) {
+template <int WAVES, bool FULL, bool SWIGLU, typename TC>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a, int rows_arg) {
   __shared__ float red[WAVES][SWIGLU ? 2 : 1][256];
   __shared__ int tile_info[3];
 
@@ -54,7 +59,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a) {
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, j = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int rows = FULL ? 16 : rows_arg;   // features per block, at most 16
+  const int n0 = blockIdx.x * rows;
+  const bool w_valid = FULL || r < rows;   // lanes of the empty rows load nothing
   const int K = a.K;
 
   const bf16* W = (const bf16*)a.W + (int64_t)group * a.w_group_stride;
@@ -79,8 +86,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a) {
       bf16x8 w[4], u[4], x[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        w[i] = *(const bf16x8*)(wrow + (s0 + i) * 32);
-        if (SWIGLU) u[i] = *(const bf16x8*)(urow + (s0 + i) * 32);
+        w[i] = w_valid ? *(const bf16x8*)(wrow + (s0 + i) * 32) : zero;
+        if (SWIGLU) u[i] = w_valid ? *(const bf16x8*)(urow + (s0 + i) * 32) : zero;
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) x[i] = m_valid ? *(const bf16x8*)(xrow + (s0 + i) * 32) : zero;
@@ -91,11 +98,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a) {
       }
     } else {
       for (int s = s0; s < steps; ++s) {
-        bf16x8 w = *(const bf16x8*)(wrow + s * 32);
+        bf16x8 w = w_valid ? *(const bf16x8*)(wrow + s * 32) : zero;
         bf16x8 x = m_valid ? *(const bf16x8*)(xrow + s * 32) : zero;
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, x, acc, 0, 0, 0);
         if (SWIGLU) {
-          bf16x8 u = *(const bf16x8*)(urow + s * 32);
+          bf16x8 u = w_valid ? *(const bf16x8*)(urow + s * 32) : zero;
           accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u, x, accu, 0, 0, 0);
         }
       }
@@ -113,7 +120,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a) {
   if (threadIdx.x < 256) {
     const int m = threadIdx.x >> 4, f = threadIdx.x & 15;
     const int row = row0 + m, col = n0 + f;
-    if (row < row_end && col < a.N) {
+    if (row < row_end && col < a.N && f < rows) {
       float v = 0.f, up = 0.f;
 #pragma unroll
       for (int w = 0; w < WAVES; ++w) {
@@ -132,22 +139,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a) {
 }
 
 template <int WAVES>
-static void launch_skinny(const GemmArgs& a, hipStream_t stream) {
+static void launch_skinny(const GemmArgs& a, int rows, hipStream_t stream) {
   int m_tiles = a.offsets ? min((a.M + SM - 1) / SM + a.groups, a.M) : (a.M + SM - 1) / SM;
-  dim3 grid((a.N + 15) / 16, m_tiles);
+  dim3 grid((a.N + rows - 1) / rows, m_tiles);
   dim3 block(WAVES * 64);
   bool swiglu = a.epilogue == kEpilogueSwiGLU;
-  if (a.out_dtype == kF32) {
-    if (swiglu)
-      gemm_skinny_kernel<WAVES, true, float><<<grid, block, 0, stream>>>(a);
-    else
-      gemm_skinny_kernel<WAVES, false, float><<<grid, block, 0, stream>>>(a);
-  } else {
-    if (swiglu)
-      gemm_skinny_kernel<WAVES, true, bf16><<<grid, block, 0, stream>>>(a);
-    else
-      gemm_skinny_kernel<WAVES, false, bf16><<<grid, block, 0, stream>>>(a);
-  }
+#define NINFER_SKINNY(FULL)                                                                   \
+  do {                                                                                        \
+    if (a.out_dtype == kF32) {                                                                \
+      if (swiglu)                                                                             \
+        gemm_skinny_kernel<WAVES, FULL, true, float><<<grid, block, 0, stream>>>(a, rows);    \
+      else                                                                                    \
+        gemm_skinny_kernel<WAVES, FULL, false, float><<<grid, block, 0, stream>>>(a, rows);   \
+    } else {                                                                                  \
+      if (swiglu)                                                                             \
+        gemm_skinny_kernel<WAVES, FULL, true, bf16><<<grid, block, 0, stream>>>(a, rows);     \
+      else                                                                                    \
+        gemm_skinny_kernel<WAVES, FULL, false, bf16><<<grid, block, 0, stream>>>(a, rows);    \
+    }                                                                                         \
+  } while (0)
+  if (rows == 16) NINFER_SKINNY(true); else NINFER_SKINNY(false);
+#undef NINFER_SKINNY
 }
 
 // Shapes the kernel takes: bf16 inputs, K a multiple of 32, rows 16-byte aligned.
@@ -161,12 +173,20 @@ int gemm_skinny(const GemmArgs& a, hipStream_t stream) {
   int m_tiles = a.offsets ? a.groups : (a.M + SM - 1) / SM;
   long blocks = (long)((a.N + 15) / 16) * m_tiles;
   int chunks = a.K / 128;
+  // features per block: 16, or for a dense product with few tiles the count that makes the
+  // blocks a whole multiple of the CUs
+  int rows = 16;
+  const int cus = 256;
+  if (!a.offsets && m_tiles == 1 && blocks < 8 * cus) {
+    const int per_cu = (a.N + 16 * cus - 1) / (16 * cus);          // blocks each CU gets
+    rows = (a.N + per_cu * cus - 1) / (per_cu * cus);
+  }
   if (blocks < 512 && chunks >= 16)
-    launch_skinny<16>(a, stream);
+    launch_skinny<16>(a, rows, stream);
   else if (blocks < 2048 && chunks >= 8)
-    launch_skinny<8>(a, stream);
+    launch_skinny<8>(a, rows, stream);
   else
-    launch_skinny<4>(a, stream);
+    launch_skinny<4>(a, rows, stream);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

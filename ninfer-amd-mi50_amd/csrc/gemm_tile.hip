@@ -243,6 +243,8 @@ int gemm_tile(const GemmArgs& a, hipStream_t stream) {
     auto blocks = [&](int tm, int tn) { return ((a.M + tm - 1) / tm) * ((n_units + tn - 1) / tn); };
     const int cus = 256;
     rows = blocks(256, 256) >= cus ? 256 : blocks(128, 128) >= cus ? 128 : 64;
+    if (a.M <= 64) rows = 64;           // and no taller than the rows there are
+    else if (a.M <= 128 && rows > 128) rows = 128;
   }
   if (rows == 256) return gemm_tile_direct(a, stream);
   if (rows == 128) return launch_tile<128, 128, 64, 4, 2, 2>(a, stream);
