@@ -91,6 +91,8 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   for (int i = 0; i < NL; ++i) xsrc[i] = (const bf16*)a.A + (int64_t)x_row[i] * a.lda + 8 * chunk;
   typedef const __attribute__((address_space(1))) void* gptr;
   typedef __attribute__((address_space(3))) void* lptr;
+  // Every lane of every load takes part: with some lanes switched off, a load into LDS did
+  // not leave the other lanes' bytes where this layout expects them (products came out wrong).
   auto issue = [&](int t) {   // k tile t into buffer t % NBUF
     unsigned char* buf = smem + (t % NBUF) * BUF_BYTES + wave * 1024;
 #pragma unroll
