@@ -62,7 +62,8 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
   const int* bt = a.block_table + (int64_t)a.row_seq[t] * a.bt_stride;
   const bf16* kpool = (const bf16*)a.kpool;
   const bf16* vpool = (const bf16*)a.vpool;
-  const int ps = a.page_size, Hkv = a.Hkv;
+  // the page size is a power of two (attention_decode_takes)
+  const int ps_shift = __builtin_ctz(a.page_size), ps_mask = a.page_size - 1, Hkv = a.Hkv;
 
   float q[GQ][8];
 #pragma unroll
@@ -86,20 +87,27 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
     for (int d = 0; d < 8; ++d) acc[i][d] = 0.f;
   }
 
+  // Every load is unconditional: a key outside lo..pos is read at the nearest key inside
+  // (a page the request holds) and its values are not used. First the page numbers of all
+  // the wave's keys, then keys and values, none waiting for another.
   const int wbase = c0 + wave * KEYS_PER_WAVE;
+  int64_t koff[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int j = min(max(wbase + it * KPI + kslot, lo), pos);
+    const int page = bt[j >> ps_shift];
+    koff[it] = ((((int64_t)page * Hkv + g) << ps_shift) + (j & ps_mask)) * D + 8 * sub;
+  }
+#pragma unroll
   for (int it0 = 0; it0 < ITERS; it0 += UNROLL) {
     bf16x8 kf[UNROLL], vf[UNROLL];
     bool ok[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      int j = wbase + (it0 + u) * KPI + kslot;
+      const int j = wbase + (it0 + u) * KPI + kslot;
       ok[u] = j >= lo && j <= pos;
-      if (ok[u]) {
-        int page = bt[j / ps];
-        int64_t off = (((int64_t)page * Hkv + g) * ps + (j % ps)) * D + 8 * sub;
-        kf[u] = *(const bf16x8*)(kpool + off);
-        vf[u] = *(const bf16x8*)(vpool + off);
-      }
+      kf[u] = *(const bf16x8*)(kpool + koff[it0 + u]);
+      vf[u] = *(const bf16x8*)(vpool + koff[it0 + u]);
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
@@ -228,7 +236,8 @@ int64_t attention_decode_workspace_floats(int T, int Hq, int D, int max_kv_len) 
 bool attention_decode_takes(const AttnArgs& a) {
   int d = a.D;
   bool d_ok = d == 16 || d == 32 || d == 64 || d == 128 || d == 256;
-  return a.dtype == kBF16 && d_ok && a.q_stride % 8 == 0 && a.workspace != nullptr;
+  bool ps_ok = (a.page_size & (a.page_size - 1)) == 0;
+  return a.dtype == kBF16 && d_ok && ps_ok && a.q_stride % 8 == 0 && a.workspace != nullptr;
 }
 
 template <int LPK, int CHUNK>
