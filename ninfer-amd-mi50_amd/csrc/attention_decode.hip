@@ -13,7 +13,7 @@
 // heads that share the kv head, so keys and values are read once for all of
 // them. Lane groups, then waves, are merged by the usual log-sum-exp rule and
 // the chunk's (m, l, acc) goes to the workspace.
-// Pass 2, grid (rows, query heads): merges the chunks of a row in chunk order.
+// Pass 2, grid (rows, query heads): merges the chunks of a row in a fixed order.
 //
 // Scores, softmax and sums are 32-bit. A row sees keys lo..pos with
 // lo = max(0, pos - window + 1); chunks are aligned to absolute positions.
@@ -188,43 +188,63 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
   }
 }
 
-// out[t, h, :] = sum_c acc_c exp(m_c - M) / sum_c l_c exp(m_c - M), chunks in order.
-// Block of 128 threads; LDS holds one scale per chunk.
-__global__ __launch_bounds__(128) void attn_decode_merge_kernel(AttnArgs a, int n_chunks,
-                                                                int kChunk) {
-  extern __shared__ float scale_s[];   // [n_chunks]
-  __shared__ float red[4];
+// out[t, h, :] = sum_c acc_c exp(m_c - M) / sum_c l_c exp(m_c - M).
+// Block of 512 threads: the chunks' m and l come in with one round of loads and stay in
+// LDS; then thread (d, part) sums the chunks c = part mod parts of dim d, all loads in
+// flight at once, and the parts are added in part order (fixed, so the result does not
+// depend on timing).
+constexpr int kMergeThreads = 512;
+
+__global__ __launch_bounds__(kMergeThreads) void attn_decode_merge_kernel(AttnArgs a, int n_chunks,
+                                                                         int kChunk) {
+  extern __shared__ float merge_s[];   // [n_chunks] scale, [n_chunks] l, [kMergeThreads] partial sums
+  float* scale_s = merge_s;
+  float* l_s = merge_s + n_chunks;
+  float* part_s = merge_s + 2 * n_chunks;
+  __shared__ float red[2 * kMergeThreads / 64];
   const int t = blockIdx.x, h = blockIdx.y, D = a.D, tid = threadIdx.x;
   const int pos = a.positions[t];
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int c_lo = lo / kChunk, c_hi = pos / kChunk;
   const float* ws = a.workspace + ((int64_t)t * a.Hq + h) * n_chunks * (D + 2);
   float mx = -1e30f;
-  for (int c = c_lo + tid; c <= c_hi; c += 128) {
-    float m = ws[c * (D + 2) + D];
+  for (int c = c_lo + tid; c <= c_hi; c += kMergeThreads) {
+    const float m = ws[c * (D + 2) + D], l = ws[c * (D + 2) + D + 1];
     scale_s[c] = m;
+    l_s[c] = l;
     mx = fmaxf(mx, m);
   }
   mx = wave_max(mx);
   if ((tid & 63) == 0) red[tid >> 6] = mx;
   __syncthreads();
-  const float M = fmaxf(red[0], red[1]);
+  float M = red[0];
+#pragma unroll
+  for (int w = 1; w < kMergeThreads / 64; ++w) M = fmaxf(M, red[w]);
   float lsum = 0.f;
-  for (int c = c_lo + tid; c <= c_hi; c += 128) {
-    float sc = __expf(scale_s[c] - M);
+  for (int c = c_lo + tid; c <= c_hi; c += kMergeThreads) {
+    const float sc = __expf(scale_s[c] - M);
     scale_s[c] = sc;
-    lsum += ws[c * (D + 2) + D + 1] * sc;
+    lsum += l_s[c] * sc;
   }
   lsum = wave_sum(lsum);
-  if ((tid & 63) == 0) red[2 + (tid >> 6)] = lsum;
+  if ((tid & 63) == 0) red[kMergeThreads / 64 + (tid >> 6)] = lsum;
   __syncthreads();
-  const float inv = 1.f / (red[2] + red[3]);
-  bf16* out = (bf16*)a.out + ((int64_t)t * a.Hq + h) * D;
-  for (int d = tid; d < D; d += 128) {
-    float acc = 0.f;
-#pragma unroll 4
-    for (int c = c_lo; c <= c_hi; ++c) acc = fmaf(ws[c * (D + 2) + d], scale_s[c], acc);
-    out[d] = __float2bfloat16(acc * inv);
+  float total = 0.f;
+#pragma unroll
+  for (int w = 0; w < kMergeThreads / 64; ++w) total += red[kMergeThreads / 64 + w];
+  const int parts = kMergeThreads / D;          // D <= 256: at least 2
+  const int d = tid % D, part = tid / D;
+  float acc = 0.f;
+  if (part < parts) {
+#pragma unroll 8
+    for (int c = c_lo + part; c <= c_hi; c += parts) acc = fmaf(ws[c * (D + 2) + d], scale_s[c], acc);
+  }
+  part_s[tid] = acc;
+  __syncthreads();
+  if (tid < D) {
+    float sum = 0.f;
+    for (int p = 0; p < parts; ++p) sum += part_s[p * D + tid];
+    ((bf16*)a.out)[((int64_t)t * a.Hq + h) * D + tid] = __float2bfloat16(sum / total);
   }
 }
 
@@ -276,8 +296,10 @@ int attention_decode(const AttnArgs& a, hipStream_t stream) {
     default: return set_error(-1, "paged_attention: decode kernel does not take head size %d", a.D);
   }
   NINFER_LAUNCH_CHECK();
-  attn_decode_merge_kernel<<<dim3(a.T, a.Hq), 128, n_chunks * sizeof(float), stream>>>(a, n_chunks,
-                                                                                      chunk);
+  const size_t merge_lds = (2 * (size_t)n_chunks + kMergeThreads) * sizeof(float);
+  NINFER_REQUIRE(merge_lds <= 48 * 1024, "paged_attention: a context of %d keys has too many chunks to merge",
+                 a.max_kv_len);
+  attn_decode_merge_kernel<<<dim3(a.T, a.Hq), kMergeThreads, merge_lds, stream>>>(a, n_chunks, chunk);
   NINFER_LAUNCH_CHECK();
   return 0;
 }
