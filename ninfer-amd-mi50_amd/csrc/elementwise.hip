@@ -221,6 +221,102 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
   }
 }
 
+// Eight consecutive elements at once (16 or 32 bytes).
+__device__ __forceinline__ void load8(const float* p, float* f) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16* p, float* f) {
+  typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+  const bf16x8 v = *(const bf16x8*)p;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = (float)v[e];
+}
+__device__ __forceinline__ void store8(float* p, const float* f) {
+  *(float4*)p = make_float4(f[0], f[1], f[2], f[3]);
+  *(float4*)(p + 4) = make_float4(f[4], f[5], f[6], f[7]);
+}
+__device__ __forceinline__ void store8(bf16* p, const float* f) {
+  typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+  bf16x8 v;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = (__bf16)f[e];
+  *(bf16x8*)p = v;
+}
+
+// The same as rope_kv_write_kernel for many rows, eight elements per access:
+// a work item is eight rotating pairs (dims i .. i + 7 and their partners at
+// + rot / 2) or eight pass-through elements. One block per row; the row's
+// cosines and sines are computed once, into LDS, for all its heads. Needs
+// rot / 2, D - rot and D to be multiples of 8 and 16-byte aligned rows.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_write_rows_kernel(
+    T* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ positions,
+    const int* __restrict__ row_seq, const float* __restrict__ inv_freq, int rot, int Hq, int Hkv,
+    int D, T* __restrict__ kpool, T* __restrict__ vpool, const int* __restrict__ block_table,
+    int bt_stride, int page_size, int write_kv) {
+  extern __shared__ float trig[];   // [rot / 2] cosines, [rot / 2] sines
+  const int t = blockIdx.x;
+  const int half = rot >> 1;
+  const int W = (Hq + 2 * Hkv) * D;
+  T* row = qkv + (int64_t)t * W;
+  const int pos = positions[t];
+  const int page = write_kv ? block_table[(int64_t)row_seq[t] * bt_stride + pos / page_size] : 0;
+  const int slot = pos % page_size;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float phi = (float)pos * inv_freq[i];
+    trig[i] = cosf(phi);
+    trig[half + i] = sinf(phi);
+  }
+  __syncthreads();
+  const int rot_items = half / 8, pass_items = (D - rot) / 8;   // of a rotated head
+  const int per_qk = rot_items + pass_items, per_v = D / 8;
+  const int n_qk = (write_kv ? Hq + Hkv : Hq) * per_qk;
+  const int n_items = n_qk + (write_kv ? Hkv * per_v : 0);
+  for (int it = threadIdx.x; it < n_items; it += blockDim.x) {
+    int head, d0;
+    bool rotate = false;
+    if (it < n_qk) {
+      head = it / per_qk;
+      const int i = it % per_qk;
+      rotate = i < rot_items;
+      d0 = rotate ? 8 * i : rot + 8 * (i - rot_items);
+    } else {
+      head = Hq + Hkv + (it - n_qk) / per_v;
+      d0 = 8 * ((it - n_qk) % per_v);
+    }
+    const int base = head * D;
+    T* dst = row + base;      // q: in place
+    if (head >= Hq) {
+      const bool is_k = head < Hq + Hkv;
+      const int kvh = is_k ? head - Hq : head - Hq - Hkv;
+      dst = (is_k ? kpool : vpool) + (((int64_t)page * Hkv + kvh) * page_size + slot) * D;
+    }
+    float v0[8], v1[8];
+    load8(row + base + d0, v0);
+    if (bias) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v0[e] += bias[base + d0 + e];
+    }
+    if (rotate) {
+      load8(row + base + d0 + half, v1);
+      if (bias) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v1[e] += bias[base + d0 + half + e];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float c = trig[d0 + e], s = trig[half + d0 + e];
+        const float r0 = v0[e] * c - v1[e] * s, r1 = v0[e] * s + v1[e] * c;
+        v0[e] = r0;
+        v1[e] = r1;
+      }
+      store8(dst + d0 + half, v1);
+    }
+    store8(dst + d0, v0);
+  }
+}
+
 // residual[t,:] += sum_j w[t,j] * y[t*k + j,:] + sigmoid(gate[t]) * shared[t,:]
 // in that order, in 32-bit (the reference scales and scatter-adds rounded
 // rows: src/ops/kernels.hip:216-223, src/ops/moe.hip:22-31).
@@ -334,6 +430,23 @@ extern "C" int ninfer_rope_kv_write(void* qkv, const float* bias, const int* pos
   NINFER_REQUIRE(rot_dim == 0 || inv_freq, "rope_kv_write: rotary size %d without a table", rot_dim);
   NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "rope_kv_write: unknown dtype %d", dtype);
   NINFER_REQUIRE(page_size > 0 && bt_stride > 0, "rope_kv_write: bad page size or table width");
+  // many rows of a shape that takes 8-element accesses: one block per row, vectorised
+  const bool vec_ok = (rot_dim / 2) % 8 == 0 && (D - rot_dim) % 8 == 0 && D % 8 == 0 &&
+                      ((uintptr_t)qkv % 32 == 0) && ((uintptr_t)kpool % 32 == 0) &&
+                      ((uintptr_t)vpool % 32 == 0);
+  if (T >= 256 && vec_ok) {
+    const size_t lds = rot_dim * sizeof(float);
+    if (dtype == kF32)
+      rope_kv_write_rows_kernel<float><<<T, 256, lds, stream>>>(
+          (float*)qkv, bias, positions, row_seq, inv_freq, rot_dim, Hq, Hkv, D, (float*)kpool,
+          (float*)vpool, block_table, bt_stride, page_size, write_kv);
+    else
+      rope_kv_write_rows_kernel<bf16><<<T, 256, lds, stream>>>(
+          (bf16*)qkv, bias, positions, row_seq, inv_freq, rot_dim, Hq, Hkv, D, (bf16*)kpool,
+          (bf16*)vpool, block_table, bt_stride, page_size, write_kv);
+    NINFER_LAUNCH_CHECK();
+    return 0;
+  }
   // few rows: spread a row's items over several blocks; many rows: one block per row
   int items = (Hq + 2 * Hkv) * (rot_dim / 2 + D - rot_dim);
   int per_row = T >= 256 ? 1 : (items + 255) / 256;

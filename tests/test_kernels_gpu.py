@@ -407,11 +407,15 @@ def test_paged_attention_finds_a_far_key(ops_mode, gen, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_q,n_kv,d,rot", [(4, 2, 16, 16), (3, 1, 32, 32), (16, 16, 128, 128),
-                                            (5, 5, 48, 24), (2, 1, 64, 0)])
-def test_rope_kv_write(ops, gen, dtype, n_q, n_kv, d, rot):
+                                            (5, 5, 48, 24), (2, 1, 64, 0), (3, 1, 64, 32),
+                                            (28, 4, 128, 128)])
+@pytest.mark.parametrize("seqs", [[(0, 9), (1000, 1), (30, 3)], [(5, 270), (0, 40), (300, 1)]],
+                         ids=["few-rows", "many-rows"])
+def test_rope_kv_write(ops, gen, dtype, n_q, n_kv, d, rot, seqs):
+    """Few rows and many rows take different kernels (the second reads and writes
+    eight elements at a time where the head layout allows it)."""
     from ninfer_amd.parts.rotary import Rotary
     ps = 8
-    seqs = [(0, 9), (1000, 1), (30, 3)]
     ctx, qkv, k_pool, v_pool, bt = _attention_case(gen, dtype, seqs, n_q, n_kv, d, ps, 200)
     table = Rotary(rot, 1e4).inv_freq().cuda() if rot else None
     bias = torch.randn(qkv.shape[1], generator=gen, device="cuda")
