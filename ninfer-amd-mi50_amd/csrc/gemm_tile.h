@@ -9,12 +9,22 @@ namespace ninfer {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-// Which tile does this block work on? Blocks go to the 8 XCDs in turn (block id
-// mod 8), and each XCD has its own L2: block ids that are congruent mod 8 get
-// neighbouring work, and work is ordered so that neighbours share their W tile
-// (the row tiles of one expert, four at a time) and then their rows of A.
-// bx: row tile (0 .. gridDim.x - 1), by: tile of output features.
-__device__ inline void block_to_tile(int& bx, int& by) {
+// Which tile does this block work on? bx: row tile (0 .. gridDim.x - 1), by: tile
+// of output features.
+// Dense: blocks go to the 8 XCDs in turn (block id mod 8), and each XCD has its
+// own L2: block ids that are congruent mod 8 get neighbouring work, and work is
+// ordered so that neighbours share their W tile (four row tiles at a time) and
+// then their rows of A.
+// Grouped: the launch order itself (row tiles fastest). Every (expert, feature
+// tile) panel of W is read by few blocks and has to stream from HBM, and blocks
+// that start together then read the same feature tile of different experts;
+// measured, this order is up to a fifth faster than the one above.
+__device__ inline void block_to_tile(bool grouped, int& bx, int& by) {
+  if (grouped) {
+    bx = blockIdx.x;
+    by = blockIdx.y;
+    return;
+  }
   const int total = gridDim.x * gridDim.y;
   const int id = blockIdx.x + gridDim.x * blockIdx.y;
   // ids congruent to x mod 8 number total / 8 (one more for x < total % 8): a bijection

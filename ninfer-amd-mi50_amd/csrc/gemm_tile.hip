@@ -47,7 +47,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void gemm_tile_kernel(GemmArgs a) {
   __shared__ int tile_info[3];
 
   int bx, by;
-  block_to_tile(bx, by);
+  block_to_tile(a.offsets != nullptr, bx, by);
   int row0, row_end, group;
   if (!tile_rows<TM>(a, bx, tile_info, row0, row_end, group)) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;

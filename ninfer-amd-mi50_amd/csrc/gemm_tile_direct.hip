@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   __shared__ int tile_info[3];
 
   int bx, by;
-  block_to_tile(bx, by);
+  block_to_tile(a.offsets != nullptr, bx, by);
   int row0, row_end, group;
   if (!tile_rows<TM>(a, bx, tile_info, row0, row_end, group)) return;
 
