@@ -56,9 +56,21 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
   bf16* const vt_lds = k_lds + 2 * K_TILE;             // [2][V_TILE]
   __shared__ int tile_info[3];
 
-  if (!find_tile(a.seq_row_start, a.S, PQ, blockIdx.x, tile_info)) return;
+  // Blocks go to the 8 XCDs in turn (block id mod 8) and each XCD has its own L2: ids
+  // that are congruent mod 8 get neighbouring work, heads outermost, so that an XCD
+  // meets the keys and values of few heads; within a head the later row tiles, which
+  // see the most keys, come first.
+  int tile, h;
+  {
+    const int total = gridDim.x * gridDim.y;
+    const int id = blockIdx.x + gridDim.x * blockIdx.y;
+    const int x = id % 8, q = total / 8, rem8 = total % 8;
+    const int w = x * q + min(x, rem8) + id / 8;   // a bijection: x < rem8 own one id more
+    h = w / gridDim.x;
+    tile = gridDim.x - 1 - w % gridDim.x;
+  }
+  if (!find_tile(a.seq_row_start, a.S, PQ, tile, tile_info)) return;
   const int row0 = tile_info[0], row_end = tile_info[1], seq = tile_info[2];
-  const int h = blockIdx.y;
   const int g = h / (a.Hq / a.Hkv);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int c = lane & 31, j = lane >> 5;
