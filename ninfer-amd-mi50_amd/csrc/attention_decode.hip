@@ -5,7 +5,8 @@
 // (src/ops/attention.hip:14-94); at long context and small batch that leaves
 // most of the GPU idle.
 //
-// Pass 1, grid (chunks, kv heads x head groups, rows), 4 waves per block. A
+// Pass 1, grid (kv heads x head groups, chunks, rows), 4 waves per block: blocks that start
+// together read the heads of the same pages, which lie side by side in the pool. A
 // key row of D = 8 LPK elements is read by LPK adjacent lanes, 16 bytes each,
 // so one wave instruction fetches 64 / LPK whole keys, contiguous in the page.
 // The dot product is reduced over those LPK lanes; each lane group keeps its
@@ -46,16 +47,17 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
   __shared__ float merge[kDecWaves][GQ][D + 2];
 
   const int t = blockIdx.z;
-  const int g = blockIdx.y / head_groups;            // kv head
-  const int hg = blockIdx.y % head_groups;           // which GQ-group of its query heads
+  const int g = blockIdx.x / head_groups;            // kv head
+  const int hg = blockIdx.x % head_groups;           // which GQ-group of its query heads
   const int group = a.Hq / a.Hkv;
   const int h0 = g * group + hg * GQ;                // first query head of this block
   const int n_heads = min(GQ, group - hg * GQ);
   const int pos = a.positions[t];
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
-  const int c0 = blockIdx.x * kChunk;
+  const int chunk_id = blockIdx.y;
+  const int c0 = chunk_id * kChunk;
   if (c0 > pos || c0 + kChunk <= lo) return;          // chunk outside the row's keys
-  const int n_chunks = gridDim.x;
+  const int n_chunks = gridDim.y;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = lane % LPK, kslot = lane / LPK;
@@ -179,7 +181,7 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
       ll += merge[w][i][D + 1] * sc;
       aa += merge[w][i][d] * sc;
     }
-    float* ws = a.workspace + (((int64_t)t * a.Hq + h0 + i) * n_chunks + blockIdx.x) * (D + 2);
+    float* ws = a.workspace + (((int64_t)t * a.Hq + h0 + i) * n_chunks + chunk_id) * (D + 2);
     ws[d] = aa;
     if (d == 0) {
       ws[D] = mm;
@@ -265,12 +267,12 @@ static void launch_decode(const AttnArgs& a, int n_chunks, hipStream_t stream) {
   int group = a.Hq / a.Hkv;
   dim3 block(kDecWaves * 64);
   if (group == 1) {
-    attn_decode_kernel<LPK, 1, CHUNK><<<dim3(n_chunks, a.Hkv, a.T), block, 0, stream>>>(a, 1);
+    attn_decode_kernel<LPK, 1, CHUNK><<<dim3(a.Hkv, n_chunks, a.T), block, 0, stream>>>(a, 1);
   } else if (group == 2) {
-    attn_decode_kernel<LPK, 2, CHUNK><<<dim3(n_chunks, a.Hkv, a.T), block, 0, stream>>>(a, 1);
+    attn_decode_kernel<LPK, 2, CHUNK><<<dim3(a.Hkv, n_chunks, a.T), block, 0, stream>>>(a, 1);
   } else {
     int hg = (group + 3) / 4;
-    attn_decode_kernel<LPK, 4, CHUNK><<<dim3(n_chunks, a.Hkv * hg, a.T), block, 0, stream>>>(a, hg);
+    attn_decode_kernel<LPK, 4, CHUNK><<<dim3(a.Hkv * hg, n_chunks, a.T), block, 0, stream>>>(a, hg);
   }
 }
 
