@@ -26,23 +26,30 @@
 namespace ninfer {
 
 namespace direct {
-constexpr int TM = 256, TN = 256, TK = 64;
+constexpr int TM = 256, TN = 256;
 constexpr int WGM = 2, WGN = 2;
 constexpr int COL = TM / WGN;             // staged token rows per wave column
 constexpr int FI = 4, FJ = 4;
-constexpr int NBUF = 2;
-constexpr int KK = TK / 16;                // quarters of a k tile: one MFMA depth each
-constexpr int ROW_BYTES = TK * 2;          // 128
-constexpr int X_BYTES = TM * ROW_BYTES;    // 32 KB
-constexpr int BUF_BYTES = (TM + TN) * ROW_BYTES;
-constexpr int LDS_BYTES = NBUF * BUF_BYTES;   // 128 KB
 }  // namespace direct
 
-#define NINFER_WAIT_LOADS(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
+// Wait until at most N of this wave's loads are under way (and, with LDS, until its LDS
+// reads have returned).
+template <int N> __device__ __forceinline__ void wait_loads() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+template <int N> __device__ __forceinline__ void wait_loads_and_lds() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(N) : "memory");
+}
 
-template <bool SWIGLU, typename TC>
+template <int TK, int NBUF, bool SWIGLU, typename TC>
 __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   using namespace direct;
+  constexpr int KK = TK / 16;                // parts of a k tile: one MFMA depth each
+  constexpr int ROW_BYTES = TK * 2;
+  constexpr int CPR = ROW_BYTES / 16;        // 16-byte chunks of a staged row
+  constexpr int RPP = 64 / CPR;              // rows of a 1 KB piece
+  constexpr int X_BYTES = TM * ROW_BYTES;
+  constexpr int BUF_BYTES = (TM + TN) * ROW_BYTES;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   __shared__ int tile_info[3];
 
@@ -63,17 +70,21 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   auto row_of = [&](int l) -> int { return (l % COL) * WGN + l / COL; };
 
   // Loads: instruction i of wave w fills the 1 KB piece i * 4 + w of the X (and
-  // of the W) part of a buffer: 8 rows, lane l at row l / 8, stored chunk l % 8,
-  // which holds the row's chunk (l % 8) ^ ((row / 2) % 8); the piece's first row
-  // is a multiple of 8 and odd pieces belong to odd waves.
+  // of the W) part of a buffer: RPP rows, lane l at row l / CPR, stored chunk
+  // l % CPR, which holds the row's chunk (l % CPR) ^ swizzle(row), where
+  // swizzle(row) = (row / (16 / CPR)) % CPR.
   constexpr int NL = TM * ROW_BYTES / 1024 / 4;   // load instructions per wave, k tile and operand
-  const int chunk = (lane & 7) ^ ((((wave & 1) << 2) + (lane >> 4)) & 7);
+  constexpr int NLT = 2 * NL;                     // loads per wave and k tile
+  // the row's part of the swizzle that the piece's number leaves: pieces i * 4 + w differ
+  // in multiples of 4 RPP rows between the loads of a wave, which the swizzle does not see
+  const int chunk = (lane % CPR) ^ (((wave * RPP + lane / CPR) / (16 / CPR)) % CPR);
+  static_assert((4 * RPP / (16 / CPR)) % CPR == 0, "the loads of a wave must share their swizzle");
   const bf16* xsrc[NL];
   const bf16* wsrc[NL];
   int x_row[NL];
 #pragma unroll
   for (int i = 0; i < NL; ++i) {
-    const int l = (i * 4 + wave) * 8 + (lane >> 3);
+    const int l = (i * 4 + wave) * RPP + lane / CPR;
     const int r = row_of(l);
     // rows beyond the tile's last read its first row (one line, from L1): their results are
     // never stored
@@ -117,23 +128,23 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   const int tok0 = wn * COL;
 
   // fragment addresses: lane reads row lr of a 32-row block, k chunk 2 kk + lk, stored at
-  // chunk (2 kk + lk) ^ ((lr / 2) % 8) (the block's first row is a multiple of 16)
+  // chunk (2 kk + lk) ^ swizzle(lr) (the block's first row is a multiple of 16)
   const int lr = lane & 31, lk = lane >> 5;
-  const int sw = (lr >> 1) & 7;
+  const int sw = (lr / (16 / CPR)) % CPR;
   const int x_lane = (tok0 + lr) * ROW_BYTES;
   const int w_lane = X_BYTES + (wm * (TN / WGM) + lr) * ROW_BYTES;
-  int c_quarter[KK];
+  int c_part[KK];
 #pragma unroll
-  for (int kk = 0; kk < KK; ++kk) c_quarter[kk] = 16 * ((2 * kk + lk) ^ sw);
+  for (int kk = 0; kk < KK; ++kk) c_part[kk] = 16 * ((2 * kk + lk) ^ sw);
   const int nk = K / TK;
 
   auto run = [&](auto nj_tag) {
     constexpr int NJ = decltype(nj_tag)::value;
     constexpr int NX = NJ > 0 ? NJ : 1;
     bf16x8 wf[2][FI], xf[2][NX];
-    auto read_quarter = [&](int set, int t, int kk) {
+    auto read_part = [&](int set, int t, int kk) {
       if constexpr (NJ == 0) return;
-      const unsigned char* buf = smem + (t % NBUF) * BUF_BYTES + c_quarter[kk];
+      const unsigned char* buf = smem + (t % NBUF) * BUF_BYTES + c_part[kk];
 #pragma unroll
       for (int i = 0; i < FI; ++i) wf[set][i] = *(const bf16x8*)(buf + w_lane + i * 32 * ROW_BYTES);
 #pragma unroll
@@ -156,40 +167,57 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
       }
       __builtin_amdgcn_sched_group_barrier(0x008, FI * NJ > FI + NJ ? FI * NJ - FI - NJ : 0, 0);
     };
-    // tiles 0 and 1 on their way, tile 0 landed
-    issue(0);
-    if (nk > 1) issue(1);
-    if (nk > 1) NINFER_WAIT_LOADS(16); else NINFER_WAIT_LOADS(0);
+    // Waiting for tile t + 1 leaves the tiles after it under way: `later` of them.
+    auto wait_tile = [&](int later) {
+      switch (later) {
+        case 0: wait_loads_and_lds<0>(); break;
+        case 1: wait_loads_and_lds<NLT>(); break;
+        case 2: wait_loads_and_lds<2 * NLT>(); break;
+        default: wait_loads_and_lds<(NBUF > 2 ? NBUF - 2 : 0) * NLT>(); break;
+      }
+    };
+    // every buffer's first tile on its way, tile 0 landed
+#pragma unroll
+    for (int b = 0; b < NBUF; ++b)
+      if (b < nk) issue(b);
+    {
+      const int later = min(NBUF, nk) - 1;
+      if (later >= 4) wait_loads<4 * NLT>();
+      else if (later == 3) wait_loads<3 * NLT>();
+      else if (later == 2) wait_loads<2 * NLT>();
+      else if (later == 1) wait_loads<NLT>();
+      else wait_loads<0>();
+    }
     __builtin_amdgcn_s_barrier();
-    read_quarter(0, 0, 0);
+    read_part(0, 0, 0);
     int t = 0;
-    // steady state, free of conditions: tiles t + 1 and t + 2 exist
-    for (; t + 2 < nk; ++t) {
+    // steady state, free of conditions: tile t + NBUF exists
+    for (; t + NBUF < nk; ++t) {
 #pragma unroll
       for (int kk = 0; kk + 1 < KK; ++kk) {
-        read_quarter((kk + 1) & 1, t, kk + 1);
+        read_part((kk + 1) & 1, t, kk + 1);
         multiply(kk & 1);
         interleave();
       }
       // this wave's loads of tile t + 1 have landed and its last fragments of tile t are in
-      // registers; after the barrier that holds for every wave
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      // registers; after the barrier that holds for every wave, and tile t's buffer is free
+      wait_loads_and_lds<(NBUF - 2) * NLT>();
       __builtin_amdgcn_s_barrier();
-      issue(t + 2);
-      read_quarter(KK & 1, t + 1, 0);
+      issue(t + NBUF);
+      read_part(KK & 1, t + 1, 0);
       multiply((KK - 1) & 1);
       interleave();
     }
-    // the last two tiles
+    // the last NBUF tiles
     for (; t < nk; ++t) {
 #pragma unroll
       for (int kk = 0; kk + 1 < KK; ++kk) {
-        read_quarter((kk + 1) & 1, t, kk + 1);
+        read_part((kk + 1) & 1, t, kk + 1);
         multiply(kk & 1);
       }
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      wait_tile(max(nk - t - 2, 0));
       __builtin_amdgcn_s_barrier();
-      if (t + 1 < nk) read_quarter(KK & 1, t + 1, 0);
+      if (t + 1 < nk) read_part(KK & 1, t + 1, 0);
       multiply((KK - 1) & 1);
     }
   };
@@ -201,29 +229,28 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
     case 3: run(std::integral_constant<int, 3>{}); break;
     default: run(std::integral_constant<int, 4>{}); break;
   }
+  static_assert(4 * FJ * 32 * FI * 64 <= NBUF * BUF_BYTES, "the epilogue's stage exceeds the buffers");
   __syncthreads();   // every wave has read its last fragments: the buffers become the epilogue's stage
   write_tile<FI, FJ, SWIGLU, TC>(a, acc, smem + wave * (FJ * 32 * FI * 64), tok0, row0, rows_here,
                                  out0 + OUT_PER_WAVE * wm, row_of);
 }
 
-#undef NINFER_WAIT_LOADS
-
 bool gemm_tile_direct_takes(const GemmArgs& a) {
-  return a.in_dtype == kBF16 && a.K % direct::TK == 0 && a.lda % 8 == 0 &&
+  return a.in_dtype == kBF16 && a.K % 64 == 0 && a.lda % 8 == 0 &&
          ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0) && a.w_group_stride % 8 == 0;
 }
 
-int gemm_tile_direct(const GemmArgs& a, hipStream_t stream) {
+template <int TK, int NBUF>
+static int launch_direct(const GemmArgs& a, hipStream_t stream) {
   using namespace direct;
-  if (a.offsets && a.tiles64 && a.big_rows != TM)
-    return set_error(-1, "gemm: the grouped tile lists are made for %d rows, not %d", a.big_rows, TM);
+  constexpr int LDS_BYTES = NBUF * (TM + TN) * TK * 2;
   const bool swiglu = a.epilogue == kEpilogueSwiGLU;
   const int m_tiles = (a.M + TM - 1) / TM + (a.offsets ? a.groups : 0);
   const int per_block = swiglu ? TN / 2 : TN;
   const dim3 grid(m_tiles, (a.N + per_block - 1) / per_block);
 #define NINFER_DIRECT_LAUNCH(SW, TYPE)                                                          \
   do {                                                                                          \
-    auto kern = gemm_tile_direct_kernel<SW, TYPE>;                                              \
+    auto kern = gemm_tile_direct_kernel<TK, NBUF, SW, TYPE>;                                    \
     hipError_t e = hipFuncSetAttribute((const void*)kern,                                       \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);  \
     if (e != hipSuccess) return set_error(-2, "gemm: cannot get %d bytes of LDS", LDS_BYTES);   \
@@ -237,6 +264,15 @@ int gemm_tile_direct(const GemmArgs& a, hipStream_t stream) {
 #undef NINFER_DIRECT_LAUNCH
   NINFER_LAUNCH_CHECK();
   return 0;
+}
+
+int gemm_tile_direct(const GemmArgs& a, hipStream_t stream) {
+  if (a.offsets && a.tiles64 && a.big_rows != direct::TM)
+    return set_error(-1, "gemm: the grouped tile lists are made for %d rows, not %d", a.big_rows,
+                     direct::TM);
+  // k tiles of 64 in two buffers: measured faster than tiles of 32 in four (whole 128-byte
+  // lines per row beat the deeper queue of loads)
+  return launch_direct<64, 2>(a, stream);
 }
 
 }  // namespace ninfer
