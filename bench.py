@@ -12,6 +12,13 @@ and its device sampler. One JSON line is printed: decoded tokens a second as
 `value`; the 2,048-token prefill under "prefill"; the decode step's memory
 roofline under "roofline"; decode at batch 1 and 64 under "points".
 Peaks: HBM 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s (fp32 157.3 TFLOP/s).
+
+    python bench.py --scenario long [--model 57b-a14b] [--requests 8] [--prompt 32768] [--new 256]
+
+is another measurement with a JSON line of its own: the scheduler serves
+`--requests` concurrent requests with random prompts of `--prompt` tokens,
+prefilled in portions of 2,048 tokens interleaved with the decoding of the
+others, `--new` tokens each, sampled at temperature 0.7 from fixed seeds.
 """
 import argparse
 import json
@@ -53,6 +60,10 @@ def main() -> int:
     ap.add_argument("--graph", action="store_true", help="decode through a captured HIP graph")
     ap.add_argument("--model", default="a2.7b", choices=sorted(MODELS),
                     help="layer sizes: a2.7b (the default and the headline) or 57b-a14b")
+    ap.add_argument("--scenario", default="decode", choices=["decode", "long"])
+    ap.add_argument("--requests", type=int, default=8, help="--scenario long: concurrent requests")
+    ap.add_argument("--prompt", type=int, default=32768, help="--scenario long: prompt tokens")
+    ap.add_argument("--new", type=int, default=256, help="--scenario long: new tokens a request")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -77,6 +88,8 @@ def main() -> int:
         raw["num_experts"], raw["num_experts_per_tok"], raw["vocab_size"]
     esize = 2 if args.dtype == "bfloat16" else 4
     page = 16
+    if args.scenario == "long":
+        return long_scenario(args, raw, model_name, layers_full)
     max_b = args.batch if args.no_points else max(args.batch, 64)
     ctx = args.context
     opt = EngineOptions(dtype=args.dtype, max_context=ctx, prefill_chunk=max(2048, max_b),
@@ -173,6 +186,65 @@ def main() -> int:
         result["points"] = points
     print(json.dumps(result), flush=True)
     return 0
+
+
+def long_scenario(args, raw, model_name, layers_full) -> int:
+    """Long prompts through the scheduler: portions of prompts beside decode tokens."""
+    import torch
+    from ninfer_amd import EngineOptions, Request, Scheduler, random_model
+    from ninfer_amd.sampling import Sampler, SamplingParams
+
+    n, plen, new = args.requests, args.prompt, args.new
+    page, chunk = 16, 2048
+    ctx = -(-(plen + new) // page) * page
+    opt = EngineOptions(dtype=args.dtype, max_context=ctx, prefill_chunk=chunk, num_sequences=n,
+                        page_size=page, use_graph=args.graph)
+    t0 = time.time()
+    runner = random_model(raw, 1234, opt)
+    torch.cuda.synchronize()
+    print(f"[bench] model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    sampler = Sampler(runner.ops, runner.device)
+    gen = torch.Generator().manual_seed(11)
+    V = raw["vocab_size"]
+
+    def serve(n_req, prompt_len, new_tokens):
+        sched = Scheduler(runner, sampler, max_batch_tokens=chunk, max_seqs=n_req)
+        reqs = [Request(id=f"r{i}", prompt=torch.randint(0, V, (prompt_len,), generator=gen).tolist(),
+                        params=SamplingParams(temperature=0.7, seed=100 + i, max_new_tokens=new_tokens))
+                for i in range(n_req)]
+        for r in reqs:
+            sched.add(r)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        last = t
+        while sched.has_work():
+            sched.step()
+            if time.perf_counter() - last > 20:
+                last = time.perf_counter()
+                fed = sum(r.cached for r in reqs if r.status == "running")
+                print(f"[bench] step {sched.steps}: {fed} tokens cached by running requests, "
+                      f"{len(sched.finished)} finished", file=sys.stderr, flush=True)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t, sched, reqs
+
+    serve(min(n, 2), 3 * chunk // 2, 4)                     # warm-up: every kind of step once
+    dt, sched, reqs = serve(n, plen, new)
+    generated = sum(len(r.output) for r in reqs)
+    failed = [r.id for r in reqs if r.status != "finished"]
+    print(json.dumps({
+        "metric": f"long-context serving ({model_name} shapes): {n} x {plen}-token prompts in "
+                  f"{chunk}-token portions interleaved with decode, {new} new tokens each",
+        "value": round((n * plen + generated) / dt, 1), "unit": "tok/s (prompt + generated)",
+        "seconds": round(dt, 3), "steps": sched.steps,
+        "prompt_tokens": n * plen, "generated_tokens": generated,
+        "preemptions": sum(r.preemptions for r in reqs), "failed": failed,
+        "n_gpus": 1, "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic", "config": {"model": f"{model_name} shapes, random weights",
+                                        "layers": raw["num_hidden_layers"], "layers_full": layers_full,
+                                        "requests": n, "prompt": plen, "new_tokens": new,
+                                        "portion": chunk, "page_size": page, "temperature": 0.7,
+                                        "graph": bool(args.graph)}}), flush=True)
+    return 1 if failed else 0
 
 
 if __name__ == "__main__":

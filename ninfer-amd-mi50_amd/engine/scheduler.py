@@ -58,6 +58,15 @@ class Request:
     def done(self) -> bool:
         return self.status in ("finished", "failed")
 
+    def next_tokens(self, n: int) -> List[int]:
+        """The n tokens after the cached ones (without joining prompt and output)."""
+        a, b, p = self.cached, self.cached + n, len(self.prompt)
+        if b <= p:
+            return self.prompt[a:b]
+        if a >= p:
+            return self.output[a - p:b - p]
+        return self.prompt[a:] + self.output[:b - p]
+
 
 @dataclass
 class PlannedStep:
@@ -205,8 +214,7 @@ class Scheduler:
             return done
         chunks = []
         for req, n, want in planned.chunks:
-            toks = req.tokens[req.cached:req.cached + n]
-            chunks.append(Chunk(req.slot, toks, [n - 1] if want else []))
+            chunks.append(Chunk(req.slot, req.next_tokens(n), [n - 1] if want else []))
         logits = self.runner.step(chunks)
         self.steps += 1
         rows = []

@@ -163,3 +163,12 @@ def test_random_arrivals_never_leak(setup):
             runner.cache.check()
     assert done == 14 and all(r.status == "finished" for r in sched.finished)
     assert all(g.allocator.in_use == 0 for g in runner.cache.groups)
+
+
+def test_next_tokens_spans_prompt_and_output():
+    from ninfer_amd import Request
+    r = Request(id="a", prompt=[1, 2, 3, 4], output=[9, 8, 7])
+    for cached in range(7):
+        for n in range(1, 8 - cached):
+            r.cached = cached
+            assert r.next_tokens(n) == r.tokens[cached:cached + n]
