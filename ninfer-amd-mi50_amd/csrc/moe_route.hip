@@ -10,8 +10,9 @@ constexpr int kMaxExpertsPerLane = 16;  // up to 1024 experts
 // One wave per row. p = softmax(logits) over all E; the k largest p in
 // descending order, ties to the lower expert index; weights p (renorm: p / sum
 // of the chosen). Reference formulas: src/ops/moe.hip:65-82.
-__device__ __forceinline__ void route_row(const float* __restrict__ row, int E, int k, int renorm,
-                                          int* __restrict__ ids, float* __restrict__ wts, int lane);
+// Returns the expert that lane j < k chose as its j-th (the same value it writes to ids[j]).
+__device__ __forceinline__ int route_row(const float* __restrict__ row, int E, int k, int renorm,
+                                         int* __restrict__ ids, float* __restrict__ wts, int lane);
 
 __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict__ logits, int ld,
                                                          int E, int k, int renorm,
@@ -23,9 +24,9 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict
 }
 
 // One row's softmax + top-k by one wave (shared by the two routing kernels).
-__device__ __forceinline__ void route_row(const float* __restrict__ row, int E, int k, int renorm,
-                                          int* __restrict__ ids, float* __restrict__ wts,
-                                          int lane) {
+__device__ __forceinline__ int route_row(const float* __restrict__ row, int E, int k, int renorm,
+                                         int* __restrict__ ids, float* __restrict__ wts,
+                                         int lane) {
   float p[kMaxExpertsPerLane];
   float m = -INFINITY;
 #pragma unroll
@@ -83,6 +84,7 @@ __device__ __forceinline__ void route_row(const float* __restrict__ row, int E, 
     ids[lane] = my_id;
     wts[lane] = renorm ? my_w / chosen_sum : my_w;
   }
+  return my_id;
 }
 
 // Rows grouped by expert, by one block: offsets[e] .. offsets[e+1] are the
@@ -157,15 +159,18 @@ __global__ __launch_bounds__(1024) void moe_route_small_kernel(
     const float* __restrict__ logits, int ld, int T, int E, int k, int renorm,
     int* __restrict__ ids, float* __restrict__ wts, int* __restrict__ offsets,
     int* __restrict__ order, int* __restrict__ tiles16, int* __restrict__ tiles64,
-    int* __restrict__ tile_counts, int big) {
-  extern __shared__ int cnt[];
+    int* __restrict__ tile_counts, int big, int ids_in_lds) {
+  extern __shared__ int cnt[];   // E + 1 counters, then (if they fit) a copy of the chosen ids
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
-  for (int t = wave; t < T; t += waves)
-    route_row(logits + (int64_t)t * ld, E, k, renorm, ids + (int64_t)t * k, wts + (int64_t)t * k,
-              lane);
-  __threadfence();
-  __syncthreads();  // the ids written above are read below by other threads of this block
-  align_block(ids, T * k, E, offsets, order, tiles16, tiles64, tile_counts, big, cnt);
+  int* ids_s = ids_in_lds ? cnt + E + 1 : nullptr;
+  for (int t = wave; t < T; t += waves) {
+    const int mine = route_row(logits + (int64_t)t * ld, E, k, renorm, ids + (int64_t)t * k,
+                               wts + (int64_t)t * k, lane);
+    // the grouping below reads the ids from LDS: no trip through global memory in between
+    if (ids_s && lane < k) ids_s[t * k + lane] = mine;
+  }
+  __syncthreads();  // what this block wrote above is read below by other threads of this block
+  align_block(ids_s ? ids_s : ids, T * k, E, offsets, order, tiles16, tiles64, tile_counts, big, cnt);
 }
 
 }  // namespace ninfer
@@ -216,9 +221,10 @@ extern "C" int ninfer_moe_route_small(const float* logits, int ld, int T, int E,
   NINFER_REQUIRE((!tiles16) == (!tiles64) && (!tiles16) == (!tile_counts),
                  "moe_route_small: tile lists come together or not at all");
   int threads = T >= 16 ? 1024 : 64 * T;
-  moe_route_small_kernel<<<1, threads, (E + 1) * sizeof(int), stream>>>(
+  const int ids_in_lds = T * k <= 4096;
+  moe_route_small_kernel<<<1, threads, (E + 1 + (ids_in_lds ? T * k : 0)) * sizeof(int), stream>>>(
       logits, ld, T, E, k, renorm, ids, wts, offsets, order, tiles16, tiles64, tile_counts,
-      big_rows);
+      big_rows, ids_in_lds);
   NINFER_LAUNCH_CHECK();
   return 0;
 }
