@@ -132,3 +132,28 @@ def test_toy_mixer_with_state_of_its_own(tmp_path):
     got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=3, max_live=3))
     for k in reqs:
         torch.testing.assert_close(got[k], ref[k], atol=2e-5, rtol=1e-4)
+
+
+def test_toy_routed_feed_forward_and_another_position_encoding(tmp_path):
+    """A feed-forward with routing of its own (a router bias from the checkpoint,
+    one expert per token) and a position encoding with other angles and a
+    partial rotation, both defined in the tests, run through the framework's
+    attention, cache, routing and grouped products, whole and in portions."""
+    import ninfer_amd
+    toy.register_routed()
+    d = str(tmp_path / "toy_routed")
+    ninfer_amd.write_random_model(d, toy.TOY_ROUTED_CONFIG, 9, std=0.3)
+    cfg, w = util.read_folder(d)
+    assert "layers.1.ff.router.bias" in w and "layers.0.ff.experts.4.down_proj.weight" in w
+    runner = runner_for(d, seqs=3)
+    assert len(runner.cache.pools) == 2          # one windowed cache per layer
+    reqs = {f"r{i}": util.random_tokens(n, 83, 40 + i) for i, n in enumerate([7, 26, 15, 33])}
+    ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
+    for k, v in reqs.items():
+        for sched in (util.schedule_whole(k, v), util.schedule_tail(k, v, 5),
+                      util.schedule_portions(k, v, 2)):
+            torch.testing.assert_close(util.run_schedule(runner, sched)[k], ref[k],
+                                       atol=3e-5, rtol=1e-4)
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=4, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)

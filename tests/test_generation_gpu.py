@@ -108,6 +108,28 @@ def test_toy_mixer_on_the_gpu(tmp_path):
         torch.testing.assert_close(got[k], ref[k], atol=2e-5, rtol=1e-4)
 
 
+def test_toy_routed_feed_forward_and_position_on_the_gpu(tmp_path):
+    """The second toy (a routed feed-forward with a router bias, another position
+    encoding with a partial rotation, a window) on the kernels, 32-bit."""
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, load_model
+    toy.register_routed()
+    d = str(tmp_path / "toy_routed")
+    ninfer_amd.write_random_model(d, toy.TOY_ROUTED_CONFIG, 9, std=0.3)
+    cfg, w = util.read_folder(d)
+    runner = load_model(d, EngineOptions(dtype="float32", max_context=64, num_sequences=3,
+                                         page_size=4))
+    reqs = {f"r{i}": util.random_tokens(n, 83, 40 + i) for i, n in enumerate([7, 26, 15, 33])}
+    ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=4, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+    k0 = "r1"
+    torch.testing.assert_close(
+        util.run_schedule(runner, util.schedule_tail(k0, reqs[k0], 6))[k0], ref[k0],
+        atol=3e-5, rtol=1e-4)
+
+
 @pytest.mark.parametrize("plan", [[(0, None), (1, 0), (2, None)],
                                   [(0, None), (1, None), (1, None), (2, None)]])
 def test_layer_plan_on_the_gpu(model_dirs, plan):

@@ -1,6 +1,7 @@
-"""A toy architecture defined in the tests, to show that a mixer with state of
-its own can be registered, built, loaded and stepped without a change to the
-framework's files. It is no model of anyone's.
+"""Toy architectures defined in the tests, to show that parts of other kinds
+can be registered, built, loaded and stepped without a change to the
+framework's files: a mixer with state of its own; a feed-forward with routing
+of its own; another position encoding. They are no models of anyone's.
 
 The mixer keeps one vector of `hidden` numbers per request (fixed size, in the
 request's state slot): s <- decay * s + (1 - decay) * x_t for every token in
@@ -14,7 +15,9 @@ from typing import Dict, List
 import torch
 
 from ninfer_amd.models.spec import ModelSpec
-from ninfer_amd.parts import (LMHead, Mixer, PreNormBlock, RMSNorm, SwiGLU, TokenEmbedding)
+from ninfer_amd.parts import (Attention, FeedForward, LMHead, Mixer, PendingRows, PositionEncoding,
+                              PreNormBlock, RMSNorm, RoutedExperts, SwiGLU, TokenEmbedding)
+from ninfer_amd.parts.moe import Routing
 from ninfer_amd.registry import register_architecture, register_part
 from ninfer_amd.weights import TensorSpec
 
@@ -101,3 +104,128 @@ def plain_forward(w: Dict[str, torch.Tensor], cfg: dict, tokens: List[int]) -> t
         x = x + pm.swiglu_mlp(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                               w[p + "mlp.down_proj.weight"])
     return pm.rms_norm(x, w["norm.weight"], cfg["rms_norm_eps"]) @ w["head.weight"].float().T
+
+
+# ---- a second toy: a feed-forward with routing of its own, another position encoding ----
+
+class HarmonicPosition(PositionEncoding):
+    """Rotation by the angles pos * slope / (1 + i), i < rot_dim / 2: no geometric
+    series, and only the first rot_dim dims of a head turn."""
+
+    def __init__(self, rot_dim: int, slope: float):
+        self.rot_dim, self.slope = rot_dim, slope
+        self._table = None
+
+    def inv_freq(self) -> torch.Tensor:
+        return torch.tensor([self.slope / (1 + i) for i in range(self.rot_dim // 2)],
+                            dtype=torch.float64).to(torch.float32)
+
+    def bind(self, w) -> None:
+        self._table = self.inv_freq().to(w.device)
+
+    def table(self):
+        return self._table
+
+
+class BiasedSwitch(FeedForward):
+    """Every token goes to the one expert with the largest (logit + bias), where the bias
+    is a tensor of the checkpoint; the expert's output is scaled by the softmax weight
+    of the biased logits. No shared expert."""
+
+    def __init__(self, prefix: str, hidden: int, inner: int, experts: int):
+        self.prefix, self.hidden, self.n = prefix, hidden, experts
+        self.experts = RoutedExperts(prefix + "experts.", hidden, inner, experts)
+        self.w_router = self.bias = None
+
+    def children(self):
+        return [self.experts]
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.prefix + "router.weight": TensorSpec((self.n, self.hidden)),
+                self.prefix + "router.bias": TensorSpec((self.n,), role="bias")}
+
+    def bind(self, w) -> None:
+        self.w_router = w.matrix(self.prefix + "router.weight")
+        self.bias = w.float32(self.prefix + "router.bias")
+
+    def forward(self, ctx, x, residual):
+        t, e = x.shape[0], self.n
+        logits = ctx.empty((t, e), torch.float32)
+        ctx.ops.linear(x, self.w_router, logits, bias=self.bias)
+        i32 = lambda *shape: ctx.empty(shape, torch.int32)
+        r = Routing(i32(t, 1), ctx.empty((t, 1), torch.float32), i32(e + 1), i32(t),
+                    i32(min(t, t // 16 + e), 4), i32(t // 64 + e, 4), i32(2))
+        ctx.ops.moe_route(logits, e, 1, False, r)
+        return PendingRows(self.experts.run(ctx, x, r), r.weights)
+
+
+@dataclass
+class ToyRoutedConfig:
+    raw: dict
+
+    @staticmethod
+    def from_dict(raw: dict) -> "ToyRoutedConfig":
+        return ToyRoutedConfig(dict(raw))
+
+
+def build_toy_routed(cfg: ToyRoutedConfig) -> ModelSpec:
+    c = cfg.raw
+    h = c["hidden_size"]
+    blocks = []
+    for l in range(c["num_hidden_layers"]):
+        p = f"layers.{l}."
+        attn = Attention(p + "attn.", h, c["heads"], c["kv_heads"], c["head_dim"],
+                         HarmonicPosition(c["rot_dim"], c["slope"]), qkv_bias=False,
+                         window=c["window"])
+        blocks.append(PreNormBlock(RMSNorm(p + "norm1.", h, c["rms_norm_eps"]), attn,
+                                   RMSNorm(p + "norm2.", h, c["rms_norm_eps"]),
+                                   BiasedSwitch(p + "ff.", h, c["inner"], c["experts"])))
+    return ModelSpec(TokenEmbedding("embed.", c["vocab_size"], h), blocks,
+                     RMSNorm("norm.", h, c["rms_norm_eps"]), LMHead("head.", c["vocab_size"], h))
+
+
+def register_routed() -> None:
+    register_part("position", "harmonic", HarmonicPosition)
+    register_part("feed_forward", "biased_switch", BiasedSwitch)
+    register_architecture("ToyRoutedForCausalLM", ToyRoutedConfig.from_dict, build_toy_routed)
+
+
+TOY_ROUTED_CONFIG = {"architectures": ["ToyRoutedForCausalLM"], "vocab_size": 83, "hidden_size": 48,
+                     "num_hidden_layers": 2, "heads": 3, "kv_heads": 1, "head_dim": 16, "rot_dim": 8,
+                     "slope": 0.7, "window": 11, "inner": 24, "experts": 5, "rms_norm_eps": 1e-5}
+
+
+def plain_forward_routed(w: Dict[str, torch.Tensor], c: dict, tokens: List[int]) -> torch.Tensor:
+    """Whole-sequence reference of the second toy (32-bit, no cache)."""
+    import plain_model as pm
+    t = len(tokens)
+    pos = torch.arange(t)
+    hq, hkv, d, rot = c["heads"], c["kv_heads"], c["head_dim"], c["rot_dim"]
+    f = torch.tensor([c["slope"] / (1 + i) for i in range(rot // 2)], dtype=torch.float64).float()
+    phi = pos.float()[:, None] * f[None, :]
+    cos, sin = torch.cos(phi)[:, None, :], torch.sin(phi)[:, None, :]
+
+    def turn(v):   # [T, heads, D]: the first rot dims in half-split pairs, the rest as they are
+        a, b, rest = v[..., :rot // 2], v[..., rot // 2:rot], v[..., rot:]
+        return torch.cat([a * cos - b * sin, a * sin + b * cos, rest], dim=-1)
+
+    x = w["embed.weight"][torch.tensor(tokens)].float()
+    for l in range(c["num_hidden_layers"]):
+        p = f"layers.{l}."
+        a = pm.rms_norm(x, w[p + "norm1.weight"], c["rms_norm_eps"])
+        q = turn((a @ w[p + "attn.q_proj.weight"].float().T).view(t, hq, d))
+        k = turn((a @ w[p + "attn.k_proj.weight"].float().T).view(t, hkv, d))
+        v = (a @ w[p + "attn.v_proj.weight"].float().T).view(t, hkv, d)
+        o = pm.attention_core(q, k, v, pos, pos, c["window"]).reshape(t, hq * d)
+        x = x + o @ w[p + "attn.o_proj.weight"].float().T
+        m = pm.rms_norm(x, w[p + "norm2.weight"], c["rms_norm_eps"])
+        logits = m @ w[p + "ff.router.weight"].float().T + w[p + "ff.router.bias"].float()
+        prob = torch.softmax(logits, dim=-1)
+        y = torch.zeros_like(m)
+        for r in range(t):
+            e = int(torch.argmax(prob[r]))        # the first maximum: ties to the lower index
+            pe = f"{p}ff.experts.{e}."
+            y[r] = prob[r, e] * pm.swiglu_mlp(m[r:r + 1], w[pe + "gate_proj.weight"],
+                                              w[pe + "up_proj.weight"], w[pe + "down_proj.weight"])[0]
+        x = x + y
+    return pm.rms_norm(x, w["norm.weight"], c["rms_norm_eps"]) @ w["head.weight"].float().T
