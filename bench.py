@@ -8,7 +8,7 @@ The default run has the layer sizes of Qwen1.5-MoE-A2.7B (24 layers, hidden
 requests and a context of 8192 tokens each (the cache is filled with random
 keys and values; token ids are seeded random). A step is one decode step: one
 new token for every request of the batch through the engine's step function
-and its device sampler. One JSON line is printed: decoded tokens a second as
+(replayed from a captured HIP graph unless --no-graph) and its device sampler. One JSON line is printed: decoded tokens a second as
 `value`; the 2,048-token prefill under "prefill"; the decode step's memory
 roofline under "roofline"; decode at batch 1 and 64 under "points".
 Peaks: HBM 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s (fp32 157.3 TFLOP/s).
@@ -57,7 +57,10 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
     ap.add_argument("--no-prefill", action="store_true")
-    ap.add_argument("--graph", action="store_true", help="decode through a captured HIP graph")
+    ap.add_argument("--graph", dest="graph", action="store_true", default=True,
+                    help="decode steps replayed from a captured HIP graph (the default)")
+    ap.add_argument("--no-graph", dest="graph", action="store_false",
+                    help="every decode step launched kernel by kernel")
     ap.add_argument("--model", default="a2.7b", choices=sorted(MODELS),
                     help="layer sizes: a2.7b (the default and the headline) or 57b-a14b")
     ap.add_argument("--scenario", default="decode", choices=["decode", "long"])
