@@ -345,8 +345,6 @@ def _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, n_pages):
     [(390, 300), (0, 129)]], ids=["long", "short", "deep"])
 def test_paged_attention(ops_mode, gen, dtype, n_q, n_kv, d, page_size, window, seqs):
     ops = ops_mode
-    if dtype == torch.float32 and seqs[0][1] == 300 and d > 64:
-        pytest.skip("the plain twin is slow at this size; bfloat16 covers the kernel")
     ctx, qkv, k_pool, v_pool, bt = _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, 80)
     if window:
         # pages a window has wholly passed are given back: the kernel must not need them
