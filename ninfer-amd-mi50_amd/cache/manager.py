@@ -37,6 +37,9 @@ class CacheGroup:
     instances: List[int] = field(default_factory=list)   # plan entries with pools in this group
     tables: Dict[int, List[int]] = field(default_factory=dict)  # slot -> page of each logical page
     window_freed: int = 0
+    # the same tables as rows of one array [slots, pages a request can hold], -1 where no page
+    # is held: what a step copies its block table from
+    rows: Optional[np.ndarray] = None
 
 
 class CacheManager:
@@ -63,6 +66,8 @@ class CacheManager:
             g = by_window[need.window]
             self.groups[g].instances.append(i)
             self.group_of_instance[i] = g
+        for g in self.groups:
+            g.rows = np.full((max_seqs, self.max_pages_per_request), -1, dtype=np.int32)
         self._free_slots: List[int] = list(range(max_seqs - 1, -1, -1))
         self._length: Dict[int, int] = {}
         self.pools: Dict[int, Tuple[object, object]] = {}
@@ -97,6 +102,7 @@ class CacheManager:
         self._length[slot] = 0
         for g in self.groups:
             g.tables[slot] = []
+            g.rows[slot, :] = -1
         if self.state is not None and self.state_floats:
             self.state[slot].zero_()
         return slot
@@ -134,7 +140,11 @@ class CacheManager:
                 raise OutOfPages(f"need {n} pages in the group with window {g.window}, "
                                  f"{g.allocator.free_pages} are free")
         for n, g in zip(need, self.groups):
-            g.tables[slot].extend(g.allocator.alloc(n))
+            if n:
+                table = g.tables[slot]
+                pages = g.allocator.alloc(n)
+                g.rows[slot, len(table):len(table) + n] = pages
+                table.extend(pages)
 
     def reserve_all(self, wants: Sequence[Tuple[int, int]]) -> None:
         """`reserve` for several (slot, new_len) at once: all or nothing."""
@@ -169,6 +179,7 @@ class CacheManager:
                 if table[p] >= 0:
                     gone.append(table[p])
                     table[p] = -1
+                    g.rows[slot, p] = -1
             if gone:
                 g.allocator.free(gone)
                 g.window_freed += len(gone)
@@ -180,11 +191,7 @@ class CacheManager:
         g = self.groups[group]
         if width is None:
             width = max([len(g.tables[s]) for s in slots] + [1])
-        out = np.full((len(slots), width), -1, dtype=np.int32)
-        for i, s in enumerate(slots):
-            t = g.tables[s]
-            out[i, :len(t)] = t
-        return out
+        return g.rows[np.asarray(slots, dtype=np.intp), :width]   # a copy
 
     # ---- introspection -------------------------------------------------------
     def kv_bytes_per_token(self, bytes_per_element: int) -> int:
@@ -207,3 +214,6 @@ class CacheManager:
             held = [p for t in g.tables.values() for p in t if p >= 0]
             assert len(held) == len(set(held)), "a page is in two block tables"
             assert len(held) == g.allocator.in_use, "allocator and block tables disagree"
+            for slot, t in g.tables.items():
+                assert g.rows[slot, :len(t)].tolist() == t and (g.rows[slot, len(t):] == -1).all(), \
+                    "the array of block-table rows has drifted from the tables"
