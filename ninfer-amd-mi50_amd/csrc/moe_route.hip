@@ -11,26 +11,30 @@ constexpr int kMaxExpertsPerLane = 16;  // up to 1024 experts
 // descending order, ties to the lower expert index; weights p (renorm: p / sum
 // of the chosen). Reference formulas: src/ops/moe.hip:65-82.
 // Returns the expert that lane j < k chose as its j-th (the same value it writes to ids[j]).
+// NPL: experts a lane looks after (64 NPL >= E).
+template <int NPL>
 __device__ __forceinline__ int route_row(const float* __restrict__ row, int E, int k, int renorm,
                                          int* __restrict__ ids, float* __restrict__ wts, int lane);
 
+template <int NPL>
 __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict__ logits, int ld,
                                                          int E, int k, int renorm,
                                                          int* __restrict__ ids,
                                                          float* __restrict__ wts) {
   const int t = blockIdx.x;
-  route_row(logits + (int64_t)t * ld, E, k, renorm, ids + (int64_t)t * k, wts + (int64_t)t * k,
-            threadIdx.x);
+  route_row<NPL>(logits + (int64_t)t * ld, E, k, renorm, ids + (int64_t)t * k, wts + (int64_t)t * k,
+                 threadIdx.x);
 }
 
 // One row's softmax + top-k by one wave (shared by the two routing kernels).
+template <int NPL>
 __device__ __forceinline__ int route_row(const float* __restrict__ row, int E, int k, int renorm,
                                          int* __restrict__ ids, float* __restrict__ wts,
                                          int lane) {
-  float p[kMaxExpertsPerLane];
+  float p[NPL];
   float m = -INFINITY;
 #pragma unroll
-  for (int i = 0; i < kMaxExpertsPerLane; ++i) {
+  for (int i = 0; i < NPL; ++i) {
     int e = lane + i * 64;
     p[i] = e < E ? row[e] : -INFINITY;
     m = fmaxf(m, p[i]);
@@ -38,14 +42,14 @@ __device__ __forceinline__ int route_row(const float* __restrict__ row, int E, i
   m = wave_max(m);
   float sum = 0.f;
 #pragma unroll
-  for (int i = 0; i < kMaxExpertsPerLane; ++i) {
+  for (int i = 0; i < NPL; ++i) {
     int e = lane + i * 64;
     p[i] = e < E ? expf(p[i] - m) : 0.f;
     sum += p[i];
   }
   sum = wave_sum(sum);
 #pragma unroll
-  for (int i = 0; i < kMaxExpertsPerLane; ++i) {
+  for (int i = 0; i < NPL; ++i) {
     int e = lane + i * 64;
     p[i] = e < E ? p[i] / sum : -1.f;  // -1 marks "not a candidate"
   }
@@ -55,7 +59,7 @@ __device__ __forceinline__ int route_row(const float* __restrict__ row, int E, i
     float best = -1.f;
     int best_e = 0x7fffffff;
 #pragma unroll
-    for (int i = 0; i < kMaxExpertsPerLane; ++i) {
+    for (int i = 0; i < NPL; ++i) {
       int e = lane + i * 64;
       if (p[i] > best) {  // ascending e within a lane: the first maximum is the lowest index
         best = p[i];
@@ -72,7 +76,7 @@ __device__ __forceinline__ int route_row(const float* __restrict__ row, int E, i
       }
     }
 #pragma unroll
-    for (int i = 0; i < kMaxExpertsPerLane; ++i)
+    for (int i = 0; i < NPL; ++i)
       if (lane + i * 64 == best_e) p[i] = -1.f;
     chosen_sum += best;
     if (lane == j) {  // lane j keeps choice j
@@ -155,6 +159,7 @@ __global__ void moe_align_kernel(const int* __restrict__ ids, int n, int E,
 
 // Few rows (decode): softmax + top-k of every row and the grouping by expert
 // in one launch of one block.
+template <int NPL>
 __global__ __launch_bounds__(1024) void moe_route_small_kernel(
     const float* __restrict__ logits, int ld, int T, int E, int k, int renorm,
     int* __restrict__ ids, float* __restrict__ wts, int* __restrict__ offsets,
@@ -164,8 +169,8 @@ __global__ __launch_bounds__(1024) void moe_route_small_kernel(
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
   int* ids_s = ids_in_lds ? cnt + E + 1 : nullptr;
   for (int t = wave; t < T; t += waves) {
-    const int mine = route_row(logits + (int64_t)t * ld, E, k, renorm, ids + (int64_t)t * k,
-                               wts + (int64_t)t * k, lane);
+    const int mine = route_row<NPL>(logits + (int64_t)t * ld, E, k, renorm, ids + (int64_t)t * k,
+                                    wts + (int64_t)t * k, lane);
     // the grouping below reads the ids from LDS: no trip through global memory in between
     if (ids_s && lane < k) ids_s[t * k + lane] = mine;
   }
@@ -184,7 +189,13 @@ extern "C" int ninfer_router_topk(const float* logits, int ld, int T, int E, int
                  64 * kMaxExpertsPerLane);
   NINFER_REQUIRE(k >= 1 && k <= E && k <= 64, "router_topk: k=%d not in [1, min(%d, 64)]", k, E);
   NINFER_REQUIRE(ld >= E, "router_topk: row stride %d < %d experts", ld, E);
-  router_topk_kernel<<<T, 64, 0, stream>>>(logits, ld, E, k, renorm, ids, wts);
+  // a lane looks after 1, 4 or 16 experts: the loops of the common sizes stay short
+  if (E <= 64)
+    router_topk_kernel<1><<<T, 64, 0, stream>>>(logits, ld, E, k, renorm, ids, wts);
+  else if (E <= 256)
+    router_topk_kernel<4><<<T, 64, 0, stream>>>(logits, ld, E, k, renorm, ids, wts);
+  else
+    router_topk_kernel<kMaxExpertsPerLane><<<T, 64, 0, stream>>>(logits, ld, E, k, renorm, ids, wts);
   NINFER_LAUNCH_CHECK();
   return 0;
 }
@@ -222,9 +233,18 @@ extern "C" int ninfer_moe_route_small(const float* logits, int ld, int T, int E,
                  "moe_route_small: tile lists come together or not at all");
   int threads = T >= 16 ? 1024 : 64 * T;
   const int ids_in_lds = T * k <= 4096;
-  moe_route_small_kernel<<<1, threads, (E + 1 + (ids_in_lds ? T * k : 0)) * sizeof(int), stream>>>(
-      logits, ld, T, E, k, renorm, ids, wts, offsets, order, tiles16, tiles64, tile_counts,
-      big_rows, ids_in_lds);
+  const size_t lds = (E + 1 + (ids_in_lds ? T * k : 0)) * sizeof(int);
+#define NINFER_ROUTE_SMALL(NPL)                                                                \
+  moe_route_small_kernel<NPL><<<1, threads, lds, stream>>>(logits, ld, T, E, k, renorm, ids, wts, \
+                                                           offsets, order, tiles16, tiles64,  \
+                                                           tile_counts, big_rows, ids_in_lds)
+  if (E <= 64)
+    NINFER_ROUTE_SMALL(1);
+  else if (E <= 256)
+    NINFER_ROUTE_SMALL(4);
+  else
+    NINFER_ROUTE_SMALL(kMaxExpertsPerLane);
+#undef NINFER_ROUTE_SMALL
   NINFER_LAUNCH_CHECK();
   return 0;
 }

@@ -231,7 +231,8 @@ def test_router_align_experts_combine(ops_mode, gen, dtype, t, e, k, h, inner):
 
 
 @pytest.mark.parametrize("t,e,k", [(1, 60, 4), (8, 60, 4), (64, 64, 8), (200, 8, 3), (300, 60, 4),
-                                   (1000, 5, 2)])
+                                   (1000, 5, 2), (7, 130, 6), (40, 300, 5), (16, 65, 64),
+                                   (3, 1000, 9)])
 def test_routing_in_one_call_with_tile_lists(ops, gen, t, e, k):
     """moe_route (one launch for few rows, two for many) against the twins; the
     tile lists cover every routed row exactly once, expert by expert."""
