@@ -200,7 +200,8 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
       v1 = to_f32(row[base + d1]) + (bias ? bias[base + d1] : 0.f);
       if (is_q || is_k) {
         float phi = (float)pos * inv_freq[i];
-        float c = cosf(phi), s = sinf(phi);
+        float c, s;
+        sincosf(phi, &s, &c);   // one range reduction for both
         float r0 = v0 * c - v1 * s, r1 = v0 * s + v1 * c;
         v0 = r0;
         v1 = r1;
@@ -265,8 +266,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_rows_kernel(
   const int slot = pos % page_size;
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     const float phi = (float)pos * inv_freq[i];
-    trig[i] = cosf(phi);
-    trig[half + i] = sinf(phi);
+    sincosf(phi, &trig[half + i], &trig[i]);   // one range reduction for both
   }
   __syncthreads();
   const int rot_items = half / 8, pass_items = (D - rot) / 8;   // of a rotated head
