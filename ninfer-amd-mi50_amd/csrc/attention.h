@@ -41,6 +41,8 @@ int attention_generic(const void* q, int q_stride, const void* kpool, const void
 int64_t attention_decode_workspace_floats(int T, int Hq, int D, int max_kv_len);
 bool attention_decode_takes(const AttnArgs& a);
 int attention_decode(const AttnArgs& a, hipStream_t stream);
+bool attention_decode_heads_takes(const AttnArgs& a);
+int attention_decode_heads(const AttnArgs& a, int chunk, int n_chunks, hipStream_t stream);
 bool attention_prefill_takes(const AttnArgs& a);
 int attention_prefill(const AttnArgs& a, hipStream_t stream);
 

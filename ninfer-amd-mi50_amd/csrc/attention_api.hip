@@ -13,6 +13,7 @@ extern "C" int ninfer_paged_attention(const AttnArgs* a, int force_generic, hipS
   NINFER_REQUIRE(a->D > 0 && a->D % 2 == 0, "paged_attention: head size %d must be even", a->D);
   NINFER_REQUIRE(a->page_size > 0 && a->bt_stride > 0, "paged_attention: bad page size %d or "
                  "table width %d", a->page_size, a->bt_stride);
+  NINFER_REQUIRE(a->scale > 0.f, "paged_attention: scale %g must be positive", (double)a->scale);
   NINFER_REQUIRE(a->window >= 0, "paged_attention: window %d must be >= 0", a->window);
   NINFER_REQUIRE(a->dtype == kF32 || a->dtype == kBF16, "paged_attention: unknown dtype %d",
                  a->dtype);

@@ -285,17 +285,32 @@ static void launch_decode_chunk(const AttnArgs& a, int chunk, int n_chunks, hipS
 }
 
 int attention_decode(const AttnArgs& a, hipStream_t stream) {
-  const int chunk = decode_chunk(a.T, a.Hkv, a.max_kv_len);
+  int chunk = decode_chunk(a.T, a.Hkv, a.max_kv_len);
+  if (attention_decode_heads_takes(a)) {
+    // the matrix-core kernel has a start-up of several tiles: the largest chunk that still
+    // gives every CU two blocks
+    chunk = 128;
+    for (int c = 1024; c > 128; c /= 2)
+      if ((long)a.T * a.Hkv * ((a.max_kv_len + c - 1) / c) >= 512) {
+        chunk = c;
+        break;
+      }
+  }
   const int n_chunks = (a.max_kv_len + chunk - 1) / chunk;
   NINFER_REQUIRE(a.workspace_floats >= attention_decode_workspace_floats(a.T, a.Hq, a.D, a.max_kv_len),
                  "paged_attention: workspace of %lld floats is too small", (long long)a.workspace_floats);
-  switch (a.D) {
-    case 16: launch_decode_chunk<2>(a, chunk, n_chunks, stream); break;
-    case 32: launch_decode_chunk<4>(a, chunk, n_chunks, stream); break;
-    case 64: launch_decode_chunk<8>(a, chunk, n_chunks, stream); break;
-    case 128: launch_decode_chunk<16>(a, chunk, n_chunks, stream); break;
-    case 256: launch_decode_chunk<32>(a, chunk, n_chunks, stream); break;
-    default: return set_error(-1, "paged_attention: decode kernel does not take head size %d", a.D);
+  if (attention_decode_heads_takes(a)) {
+    // three or more query heads per kv head: their products go to the matrix cores
+    if (int rc = attention_decode_heads(a, chunk, n_chunks, stream)) return rc;
+  } else {
+    switch (a.D) {
+      case 16: launch_decode_chunk<2>(a, chunk, n_chunks, stream); break;
+      case 32: launch_decode_chunk<4>(a, chunk, n_chunks, stream); break;
+      case 64: launch_decode_chunk<8>(a, chunk, n_chunks, stream); break;
+      case 128: launch_decode_chunk<16>(a, chunk, n_chunks, stream); break;
+      case 256: launch_decode_chunk<32>(a, chunk, n_chunks, stream); break;
+      default: return set_error(-1, "paged_attention: decode kernel does not take head size %d", a.D);
+    }
   }
   NINFER_LAUNCH_CHECK();
   const size_t merge_lds = (2 * (size_t)n_chunks + kMergeThreads) * sizeof(float);

@@ -26,6 +26,14 @@
 // A row at position p sees keys lo..p, lo = max(0, p - window + 1). Pages that
 // a window has passed may be gone (block-table entry -1): their keys are never
 // visible and are loaded as zeros.
+//
+// The same kernel serves decoding for models whose kv heads are shared by three
+// or more query heads (HEADS): the 32 "rows" of a block are then the query
+// heads of one kv head for one decoded token, all at one position, and the block
+// walks one chunk of CHUNK keys and writes its running max, sum and output to the
+// workspace, which the decode path's merge kernel adds up. Each key and value is
+// then read once for all heads of its group, and the products run on the matrix
+// cores instead of one scalar FMA per head, key and dim.
 #include "attention.h"
 #include "gemm.h"
 
@@ -37,10 +45,11 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int PK = 64;   // keys per tile
 
-template <int D, int NQ>
-__global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
+template <int D, int NQ, bool HEADS>   // HEADS: rows are the query heads of one token (decode)
+__global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, int CHUNK) {
   constexpr int KH = 2;             // waves per group of 32 rows: each meets one half of a tile's keys
   constexpr int NT = NQ * KH * 64;
+  constexpr int NS = 2;              // tiles on their way in registers
   constexpr int NKB = 2 / KH;       // 32-key blocks of a tile that one wave meets
   constexpr int PQ = NQ * 32;       // query rows per block
   constexpr int KS = D / 16;        // k-steps of Q K^T
@@ -56,29 +65,45 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
   bf16* const vt_lds = k_lds + 2 * K_TILE;             // [2][V_TILE]
   __shared__ int tile_info[3];
 
-  // Blocks go to the 8 XCDs in turn (block id mod 8) and each XCD has its own L2: ids
-  // that are congruent mod 8 get neighbouring work, heads outermost, so that an XCD
-  // meets the keys and values of few heads; within a head the later row tiles, which
-  // see the most keys, come first.
-  int tile, h;
-  {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 31, j = lane >> 5;
+  const int group = a.Hq / a.Hkv;
+  int row0, n_rows, seq, g, h, pos_first, pos_last, lo_first, chunk_id = 0;
+  if constexpr (HEADS) {
+    // grid (kv heads, chunks, rows): heads fastest, so that blocks in flight share pages
+    row0 = blockIdx.z;
+    g = blockIdx.x;
+    chunk_id = blockIdx.y;
+    const int pos = a.positions[row0];
+    const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+    const int c0 = chunk_id * CHUNK;
+    if (c0 > pos || c0 + CHUNK <= lo) return;   // chunk outside the row's keys
+    n_rows = group;
+    seq = a.row_seq[row0];
+    h = g * group;                               // the lane's head is h + c
+    pos_first = pos;
+    pos_last = min(pos, c0 + CHUNK - 1);         // last key this block meets
+    lo_first = max(lo, c0);
+  } else {
+    // Blocks go to the 8 XCDs in turn (block id mod 8) and each XCD has its own L2: ids
+    // that are congruent mod 8 get neighbouring work, heads outermost, so that an XCD
+    // meets the keys and values of few heads; within a head the later row tiles, which
+    // see the most keys, come first.
     const int total = gridDim.x * gridDim.y;
     const int id = blockIdx.x + gridDim.x * blockIdx.y;
     const int x = id % 8, q = total / 8, rem8 = total % 8;
     const int w = x * q + min(x, rem8) + id / 8;   // a bijection: x < rem8 own one id more
     h = w / gridDim.x;
-    tile = gridDim.x - 1 - w % gridDim.x;
+    const int tile = gridDim.x - 1 - w % gridDim.x;
+    if (!find_tile(a.seq_row_start, a.S, PQ, tile, tile_info)) return;
+    row0 = tile_info[0];
+    seq = tile_info[2];
+    g = h / group;
+    pos_first = a.positions[row0];               // rows of a request are consecutive
+    n_rows = min(PQ, tile_info[1] - row0);
+    pos_last = pos_first + n_rows - 1;
+    lo_first = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
   }
-  if (!find_tile(a.seq_row_start, a.S, PQ, tile, tile_info)) return;
-  const int row0 = tile_info[0], row_end = tile_info[1], seq = tile_info[2];
-  const int g = h / (a.Hq / a.Hkv);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int c = lane & 31, j = lane >> 5;
-
-  const int pos_first = a.positions[row0];               // rows of a request are consecutive
-  const int n_rows = min(PQ, row_end - row0);
-  const int pos_last = pos_first + n_rows - 1;
-  const int lo_first = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
   const int* bt = a.block_table + (int64_t)seq * a.bt_stride;
   const bf16* kpool = (const bf16*)a.kpool;
   const bf16* vpool = (const bf16*)a.vpool;
@@ -91,15 +116,22 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
   const int q_local = qg * 32 + c;
   const bool q_valid = q_local < n_rows;
   const bool wave_live = qg * 32 < n_rows;    // a wave without rows only helps to load
-  const int q_pos = pos_first + q_local;
-  const int q_lo = a.window > 0 ? max(0, q_pos - a.window + 1) : 0;
+  const int q_pos = HEADS ? pos_first : pos_first + q_local;
+  const int q_lo = HEADS ? lo_first : (a.window > 0 ? max(0, q_pos - a.window + 1) : 0);
   // keys this wave's rows can see: tiles outside are loaded for the others but not multiplied
-  const int wave_pos_last = pos_first + min(qg * 32 + 31, n_rows - 1);
-  const int wave_lo = a.window > 0 ? max(0, pos_first + qg * 32 - a.window + 1) : 0;
+  const int wave_pos_last = HEADS ? pos_last : pos_first + min(qg * 32 + 31, n_rows - 1);
+  const int wave_lo = HEADS ? lo_first
+                            : (a.window > 0 ? max(0, pos_first + qg * 32 - a.window + 1) : 0);
+  // keys that every row of the wave sees, rows without a query included: a block of keys
+  // inside needs no mask
+  const int all_see_last = HEADS ? pos_first : pos_first + qg * 32;
+  const int all_see_first =
+      HEADS ? lo_first : (a.window > 0 ? max(0, pos_first + qg * 32 + 31 - a.window + 1) : 0);
   bf16x8 qf[KS];
   {
-    const bf16* qr = (const bf16*)a.q + (int64_t)(row0 + (q_valid ? q_local : 0)) * a.q_stride +
-                     h * D + 8 * j;
+    const int ql = q_valid ? q_local : 0;
+    const bf16* qr = (const bf16*)a.q + (int64_t)(row0 + (HEADS ? 0 : ql)) * a.q_stride +
+                     (h + (HEADS ? ql : 0)) * D + 8 * j;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const bf16x8*)(qr + 16 * ks);
   }
@@ -121,13 +153,13 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
   constexpr int V_PER_THREAD = (V_BLOCKS + NT - 1) / NT;
   static_assert(K_VECS % NT == 0, "tile does not divide over the block");
 
-  // A tile's keys and values travel global -> registers -> LDS. Tile i is
+  // A tile's keys and values travel global -> registers (stage i % NS) -> LDS. Tile i is
   // multiplied from LDS buffer i % 2 while tile i + 1 moves from its registers to
-  // the other buffer, the loads of tile i + 3 are issued into those registers,
-  // and the page numbers of tile i + 5 are fetched: no load waits for another
+  // the other buffer, the loads of tile i + 1 + NS are issued into those registers,
+  // and the page numbers of tile i + 1 + 2 NS are fetched: no load waits for another
   // inside the loop.
-  bf16x8 kreg[2][K_PER_THREAD], vreg[2][V_PER_THREAD][4];
-  int kpage[2][K_PER_THREAD], vpage[2][V_PER_THREAD];
+  bf16x8 kreg[NS][K_PER_THREAD], vreg[NS][V_PER_THREAD][4];
+  int kpage[NS][K_PER_THREAD], vpage[NS][V_PER_THREAD];
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   // Every load below is unconditional (a select replaces what is not there by zeros): a
   // load under a condition would have to be waited for where the condition ends.
@@ -149,10 +181,11 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
     for (int i = 0; i < K_PER_THREAD; ++i) {
       int vec = tid + i * NT;
       int kp = t0 + vec / (D / 8), dv = vec % (D / 8);
-      // a key that is not there is read from the pool's first page and replaced by zeros
+      // For a key that is not there, the last key (beyond it) or a row of the pool's first
+      // page (a page given back) is read in its place. Such a key lies in a block that is
+      // masked, and the mask replaces its scores whatever they are.
       const int page = kpage[st][i];
-      const bf16x8 got = *(const bf16x8*)(kpool + ((((int64_t)max(page, 0) * Hkv + g) << ps_shift) + (kp & ps_mask)) * D + 8 * dv);
-      kreg[st][i] = (page >= 0 && kp <= pos_last) ? got : zero8;
+      kreg[st][i] = *(const bf16x8*)(kpool + ((((int64_t)max(page, 0) * Hkv + g) << ps_shift) + (min(kp, pos_last) & ps_mask)) * D + 8 * dv);
     }
 #pragma unroll
     for (int i = 0; i < V_PER_THREAD; ++i) {
@@ -162,7 +195,7 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         int kp = t0 + 4 * kg + r;
-        const bf16x8 got = *(const bf16x8*)(vpool + ((((int64_t)max(page, 0) * Hkv + g) << ps_shift) + (kp & ps_mask)) * D + 8 * dv);
+        const bf16x8 got = *(const bf16x8*)(vpool + ((((int64_t)max(page, 0) * Hkv + g) << ps_shift) + (min(kp, pos_last) & ps_mask)) * D + 8 * dv);
         vreg[st][i][r] = (page >= 0 && kp <= pos_last) ? got : zero8;
       }
     }
@@ -210,15 +243,25 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
     }
     // lane holds, for query c, keys k0 + 32 kb + 8 (v / 4) + 4 j + v % 4
     float mx = -1e30f;
+    if (k0 + 32 * NKB - 1 > all_see_last || k0 < all_see_first) {
 #pragma unroll
-    for (int kb = 0; kb < NKB; ++kb)
+      for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        int kp = k0 + 32 * kb + 8 * (v >> 2) + 4 * j + (v & 3);
-        float val = (kp <= q_pos && kp >= q_lo) ? s[kb][v] * scale2 : -1e30f;
-        s[kb][v] = val;
-        mx = fmaxf(mx, val);
-      }
+        for (int v = 0; v < 16; ++v) {
+          int kp = k0 + 32 * kb + 8 * (v >> 2) + 4 * j + (v & 3);
+          // minus infinity, so that the probability is exactly 0 whatever the row's maximum
+          // (the maximum itself starts at -1e30 and stays finite)
+          float val = (kp <= q_pos && kp >= q_lo) ? s[kb][v] : -__builtin_inff();
+          s[kb][v] = val;
+          mx = fmaxf(mx, val);
+        }
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
+    }
+    mx *= scale2;   // the scale is positive: the largest score stays the largest
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m, mx);
     const float alpha = __builtin_amdgcn_exp2f(m - m_new);
@@ -229,7 +272,7 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
     for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        float p = __builtin_amdgcn_exp2f(s[kb][v] - m_new);
+        float p = __builtin_amdgcn_exp2f(fmaf(s[kb][v], scale2, -m_new));
         psum += p;
         pf[kb][v >> 3][v & 7] = (__bf16)p;
       }
@@ -254,31 +297,31 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
   };
 
   const int t_first = (lo_first / PK) * PK;
-  load_pages(0, t_first);
-  load_pages(1, t_first + PK);
-  load_regs(0, t_first);
-  load_regs(1, t_first + PK);
-  load_pages(0, t_first + 2 * PK);
-  load_pages(1, t_first + 3 * PK);
+#pragma unroll
+  for (int st = 0; st < NS; ++st) load_pages(st, t_first + st * PK);
+#pragma unroll
+  for (int st = 0; st < NS; ++st) {
+    load_regs(st, t_first + st * PK);
+    load_pages(st, t_first + (NS + st) * PK);
+  }
   store_regs(0, 0);
-  load_regs(0, t_first + 2 * PK);
-  load_pages(0, t_first + 4 * PK);
+  load_regs(0, t_first + NS * PK);
+  load_pages(0, t_first + 2 * NS * PK);
   lds_barrier();
-  // Two tiles per turn, so that the register stage and the buffer of each are constants.
+  // NS tiles per turn, so that the register stage and the buffer of each are constants.
   // Nothing in the loop stands under a condition: tiles beyond the last key are loaded as
   // zeros and skipped by the products, so the wait before a store counts exactly the loads
   // issued after the ones it needs.
-  for (int t0 = t_first; t0 <= pos_last; t0 += 2 * PK) {
-    store_regs(1, 1);
-    load_regs(1, t0 + 3 * PK);
-    load_pages(1, t0 + 5 * PK);
-    multiply(0, t0);
-    lds_barrier();   // tile t0 + PK is whole, tile t0 has been read by every wave
-    store_regs(0, 0);
-    load_regs(0, t0 + 4 * PK);
-    load_pages(0, t0 + 6 * PK);
-    multiply(1, t0 + PK);
-    lds_barrier();
+  for (int t0 = t_first; t0 <= pos_last; t0 += NS * PK) {
+#pragma unroll
+    for (int u = 0; u < NS; ++u) {
+      const int st = (u + 1) % NS;
+      store_regs(st, (u + 1) % 2);
+      load_regs(st, t0 + (u + 1 + NS) * PK);
+      load_pages(st, t0 + (u + 1 + 2 * NS) * PK);
+      multiply(u % 2, t0 + u * PK);
+      lds_barrier();   // the next tile is whole, this one has been read by every wave
+    }
   }
 
   // Merge the two key halves of every row group: the waves of the second half hand their
@@ -294,9 +337,10 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
   }
   __syncthreads();
   if (kh == 1) return;
+  float m_all;
   {
     const float m1 = mine[0], l1 = mine[1];
-    const float m_all = fmaxf(m, m1);
+    m_all = fmaxf(m, m1);
     const float a0 = __builtin_amdgcn_exp2f(m - m_all), a1 = __builtin_amdgcn_exp2f(m1 - m_all);
     l = l * a0 + l1 * a1;
 #pragma unroll
@@ -306,6 +350,26 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
   }
   // the two lanes of a query hold partial sums of l
   l += __shfl_xor(l, 32, 64);
+  if constexpr (HEADS) {
+    // the chunk's max (in natural-log units, as the merge kernel takes it), sum and
+    // unnormalised output of head h + c
+    if (q_valid) {
+      float* ws = a.workspace + (((int64_t)row0 * a.Hq + h + c) * gridDim.y + chunk_id) * (D + 2);
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          float* dst = ws + db * 32 + 8 * qd + 4 * j;   // D + 2 is even: 8-byte aligned
+          *(float2*)dst = make_float2(o[db][4 * qd], o[db][4 * qd + 1]);
+          *(float2*)(dst + 2) = make_float2(o[db][4 * qd + 2], o[db][4 * qd + 3]);
+        }
+      if (j == 0) {
+        ws[D] = m_all * 0.693147180559945f;
+        ws[D + 1] = l;
+      }
+    }
+    return;
+  }
   if (q_valid) {
     // lane holds, of its query's output, dims 32 db + 8 (v / 4) + 4 j + v % 4
     const float inv = 1.f / l;
@@ -321,6 +385,27 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a) {
   }
 }
 
+// Decoding with grouped heads: bf16, head size 64 or 128, 3 to 32 query heads per kv head.
+bool attention_decode_heads_takes(const AttnArgs& a) {
+  const int group = a.Hq / a.Hkv;
+  return a.dtype == kBF16 && (a.D == 64 || a.D == 128) && a.q_stride % 8 == 0 &&
+         PK % a.page_size == 0 && group >= 3 && group <= 32 && a.workspace != nullptr &&
+         a.row_seq != nullptr;
+}
+
+// Pass 1 of split-context decoding for grouped heads; the caller merges the chunks.
+int attention_decode_heads(const AttnArgs& a, int chunk, int n_chunks, hipStream_t stream) {
+  NINFER_REQUIRE(chunk > 0 && chunk % PK == 0, "paged_attention: chunks of %d keys are no "
+                 "multiple of %d", chunk, PK);
+  dim3 grid(a.Hkv, n_chunks, a.T);
+  if (a.D == 128)
+    attn_prefill_kernel<128, 1, true><<<grid, 128, 0, stream>>>(a, chunk);
+  else
+    attn_prefill_kernel<64, 1, true><<<grid, 128, 0, stream>>>(a, chunk);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
 bool attention_prefill_takes(const AttnArgs& a) {
   return a.dtype == kBF16 && (a.D == 64 || a.D == 128) && a.q_stride % 8 == 0 &&
          PK % a.page_size == 0 && a.seq_row_start != nullptr;
@@ -331,9 +416,9 @@ static int launch_prefill(const AttnArgs& a, hipStream_t stream) {
   constexpr int PQ = NQ * 32;
   dim3 grid((a.T + PQ - 1) / PQ + a.S, a.Hq);
   if (a.D == 128)
-    attn_prefill_kernel<128, NQ><<<grid, NQ * 128, 0, stream>>>(a);
+    attn_prefill_kernel<128, NQ, false><<<grid, NQ * 128, 0, stream>>>(a, 0);
   else
-    attn_prefill_kernel<64, NQ><<<grid, NQ * 128, 0, stream>>>(a);
+    attn_prefill_kernel<64, NQ, false><<<grid, NQ * 128, 0, stream>>>(a, 0);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

@@ -365,7 +365,9 @@ def test_paged_attention(ops_mode, gen, dtype, n_q, n_kv, d, page_size, window, 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_q,n_kv,d,page_size,window", [
     (4, 2, 16, 4, 0), (3, 1, 32, 8, 24), (16, 16, 128, 16, 0), (28, 4, 128, 16, 0),
-    (8, 8, 64, 16, 300), (10, 2, 64, 64, 0), (2, 2, 80, 16, 0), (4, 1, 256, 16, 0)])
+    (8, 8, 64, 16, 300), (10, 2, 64, 64, 0), (2, 2, 80, 16, 0), (4, 1, 256, 16, 0),
+    # three or more query heads to a kv head: the decode kernel on the matrix cores
+    (12, 4, 64, 16, 300), (32, 1, 128, 32, 100), (9, 3, 128, 64, 0), (33, 1, 64, 16, 0)])
 def test_paged_attention_decode_rows(ops_mode, gen, dtype, n_q, n_kv, d, page_size, window):
     """Single-token rows only: the split-context kernel's case. Contexts end at
     chunk and page edges and inside them."""
