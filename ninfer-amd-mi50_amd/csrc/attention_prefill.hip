@@ -394,14 +394,16 @@ bool attention_decode_heads_takes(const AttnArgs& a) {
 }
 
 // Pass 1 of split-context decoding for grouped heads; the caller merges the chunks.
+// Blocks of four waves: two multiply (the key halves of the one group of 32 rows), the
+// other two only help to load, which keeps each wave's staging registers few.
 int attention_decode_heads(const AttnArgs& a, int chunk, int n_chunks, hipStream_t stream) {
   NINFER_REQUIRE(chunk > 0 && chunk % PK == 0, "paged_attention: chunks of %d keys are no "
                  "multiple of %d", chunk, PK);
   dim3 grid(a.Hkv, n_chunks, a.T);
   if (a.D == 128)
-    attn_prefill_kernel<128, 1, true><<<grid, 128, 0, stream>>>(a, chunk);
+    attn_prefill_kernel<128, 2, true><<<grid, 256, 0, stream>>>(a, chunk);
   else
-    attn_prefill_kernel<64, 1, true><<<grid, 128, 0, stream>>>(a, chunk);
+    attn_prefill_kernel<64, 2, true><<<grid, 256, 0, stream>>>(a, chunk);
   NINFER_LAUNCH_CHECK();
   return 0;
 }
