@@ -176,27 +176,39 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
       vpage[st][i] = bt[min(kp, pos_last) >> ps_shift];
     }
   };
+  // A tile starts at a multiple of the page size, so the place of a thread's piece inside
+  // its page is the same in every tile: address = pool + page * page_stride + in_page.
+  const int64_t page_stride = ((int64_t)Hkv << ps_shift) * D;
+  int64_t k_in_page[K_PER_THREAD], v_in_page[V_PER_THREAD];
+#pragma unroll
+  for (int i = 0; i < K_PER_THREAD; ++i) {
+    const int vec = tid + i * NT;
+    k_in_page[i] = (((int64_t)g << ps_shift) + ((vec / (D / 8)) & ps_mask)) * D + 8 * (vec % (D / 8));
+  }
+#pragma unroll
+  for (int i = 0; i < V_PER_THREAD; ++i) {
+    const int blk = (tid + i * NT) % V_BLOCKS;
+    v_in_page[i] = (((int64_t)g << ps_shift) + ((4 * (blk % (PK / 4))) & ps_mask)) * D + 8 * (blk / (PK / 4));
+  }
   auto load_regs = [&](int st, int t0) {
 #pragma unroll
     for (int i = 0; i < K_PER_THREAD; ++i) {
-      int vec = tid + i * NT;
-      int kp = t0 + vec / (D / 8), dv = vec % (D / 8);
-      // For a key that is not there, the last key (beyond it) or a row of the pool's first
-      // page (a page given back) is read in its place. Such a key lies in a block that is
-      // masked, and the mask replaces its scores whatever they are.
-      const int page = kpage[st][i];
-      kreg[st][i] = *(const bf16x8*)(kpool + ((((int64_t)max(page, 0) * Hkv + g) << ps_shift) + (min(kp, pos_last) & ps_mask)) * D + 8 * dv);
+      // For a key that is not there, a row of the last key's page (beyond it) or of the
+      // pool's first page (a page given back) is read in its place. Such a key lies in a
+      // block that is masked, and the mask replaces its scores whatever they are.
+      kreg[st][i] = *(const bf16x8*)(kpool + max(kpage[st][i], 0) * page_stride + k_in_page[i]);
     }
 #pragma unroll
     for (int i = 0; i < V_PER_THREAD; ++i) {
-      int blk = (tid + i * NT) % V_BLOCKS;
-      int kg = blk % (PK / 4), dv = blk / (PK / 4);
+      const int blk = (tid + i * NT) % V_BLOCKS;
       const int page = vpage[st][i];
+      const bf16* vsrc = vpool + max(page, 0) * page_stride + v_in_page[i];
+      const int kp0 = t0 + 4 * (blk % (PK / 4));
+      // a value that is not there must be zero: its probability is, but 0 x anything is not
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        int kp = t0 + 4 * kg + r;
-        const bf16x8 got = *(const bf16x8*)(vpool + ((((int64_t)max(page, 0) * Hkv + g) << ps_shift) + (min(kp, pos_last) & ps_mask)) * D + 8 * dv);
-        vreg[st][i][r] = (page >= 0 && kp <= pos_last) ? got : zero8;
+        const bf16x8 got = *(const bf16x8*)(vsrc + r * D);
+        vreg[st][i][r] = (page >= 0 && kp0 + r <= pos_last) ? got : zero8;
       }
     }
   };
@@ -282,7 +294,10 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
     m = m_new;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      if (moved) o[db] *= alpha;
+      if (moved) {
+        asm volatile("" ::: "memory");   // a real branch: as selects the products would always run
+        o[db] *= alpha;
+      }
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
@@ -389,7 +404,7 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
 bool attention_decode_heads_takes(const AttnArgs& a) {
   const int group = a.Hq / a.Hkv;
   return a.dtype == kBF16 && (a.D == 64 || a.D == 128) && a.q_stride % 8 == 0 &&
-         PK % a.page_size == 0 && group >= 3 && group <= 32 && a.workspace != nullptr &&
+         PK % a.page_size == 0 && a.page_size % 4 == 0 && group >= 3 && group <= 32 && a.workspace != nullptr &&
          a.row_seq != nullptr;
 }
 
@@ -410,7 +425,7 @@ int attention_decode_heads(const AttnArgs& a, int chunk, int n_chunks, hipStream
 
 bool attention_prefill_takes(const AttnArgs& a) {
   return a.dtype == kBF16 && (a.D == 64 || a.D == 128) && a.q_stride % 8 == 0 &&
-         PK % a.page_size == 0 && a.seq_row_start != nullptr;
+         PK % a.page_size == 0 && a.page_size % 4 == 0 && a.seq_row_start != nullptr;
 }
 
 template <int NQ>
