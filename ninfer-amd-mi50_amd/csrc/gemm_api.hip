@@ -3,6 +3,12 @@
 
 using namespace ninfer;
 
+// many rows per weight matrix: 64-row tiles and taller; few: 16-row tiles that stream the
+// weights (a product with few output features has too few 128-wide tiles to fill the GPU)
+static bool many_rows(const GemmArgs& a) {
+  return a.offsets ? a.M >= 16 * a.groups : (a.M > 32 && a.N > 128);
+}
+
 // force_generic != 0 runs the plain tiled kernel whatever the shape (tests
 // compare the fast kernels with it).
 extern "C" int ninfer_gemm(const GemmArgs* args, int force_generic, hipStream_t stream) {
@@ -10,11 +16,23 @@ extern "C" int ninfer_gemm(const GemmArgs* args, int force_generic, hipStream_t 
   if (rc) return rc;
   const GemmArgs& a = *args;
   if (!force_generic) {
-    // many rows per weight matrix: 64-row tiles; few: 16-row tiles that stream the weights
-    // (a product with few output features has too few 128-wide tiles to fill the GPU)
-    bool many = a.offsets ? a.M >= 16 * a.groups : (a.M > 32 && a.N > 128);
-    if (many && gemm_tile_takes(a)) return gemm_tile(a, stream);
+    if (many_rows(a) && gemm_tile_takes(a)) return gemm_tile(a, stream);
     if (gemm_skinny_takes(a)) return gemm_skinny(a, stream);
   }
   return gemm_generic(a, stream);
+}
+
+// Two products that do not depend on each other. Pairs of few-row products that have a
+// kernel of their own run as one launch; all others one after the other.
+extern "C" int ninfer_gemm_pair(const GemmArgs* a, const GemmArgs* b, int force_generic,
+                                hipStream_t stream) {
+  int rc = gemm_check(*a);
+  if (rc) return rc;
+  rc = gemm_check(*b);
+  if (rc) return rc;
+  if (!force_generic && !many_rows(*a) && !many_rows(*b) && gemm_skinny_pair_takes(*a, *b))
+    return gemm_skinny_pair(*a, *b, stream);
+  rc = ninfer_gemm(a, force_generic, stream);
+  if (rc) return rc;
+  return ninfer_gemm(b, force_generic, stream);
 }

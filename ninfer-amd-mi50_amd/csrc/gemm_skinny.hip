@@ -32,27 +32,31 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int SM = 16;  // rows of A per tile
 
+// The work of one block: tile (bx, by) of the product `a`. WAVES > 0 fixes the waves that
+// share the K range at compile time; WAVES == 0 takes them from `waves_arg` (waves of the
+// block beyond that number must not call). `red` holds waves x (2 with SwiGLU, else 1) x 256
+// floats.
 template <int WAVES, bool FULL, bool SWIGLU, typename TC>
-__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a, int rows_arg) {
-  __shared__ float red[WAVES][SWIGLU ? 2 : 1][256];
-  __shared__ int tile_info[3];
-
+__device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, int waves_arg,
+                                             int bx, int by, float* red, int* tile_info) {
+  constexpr int HALVES = SWIGLU ? 2 : 1;
+  const int waves = WAVES > 0 ? WAVES : waves_arg;
   int row0, row_end, group = 0;
   if (a.offsets && a.tiles16) {
     // every thread reads the tile's entry itself: no barrier before the first loads
     int count = a.tile_counts[0];
-    int4 t = ((const int4*)a.tiles16)[blockIdx.y];
-    if ((int)blockIdx.y >= count) return;
+    int4 t = ((const int4*)a.tiles16)[by];
+    if (by >= count) return;
     group = t.x;
     row0 = t.y;
     row_end = t.z;
   } else if (a.offsets) {
-    if (!find_tile(a.offsets, a.groups, SM, blockIdx.y, tile_info)) return;
+    if (!find_tile(a.offsets, a.groups, SM, by, tile_info)) return;
     group = tile_info[2];
     row0 = tile_info[0];
     row_end = tile_info[1];
   } else {
-    row0 = blockIdx.y * SM;
+    row0 = by * SM;
     row_end = a.M;
     if (row0 >= row_end) return;
   }
@@ -60,7 +64,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a, int
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, j = lane >> 4;
   const int rows = FULL ? 16 : rows_arg;   // features per block, at most 16
-  const int n0 = blockIdx.x * rows;
+  const int n0 = bx * rows;
   const bool w_valid = FULL || r < rows;   // lanes of the empty rows load nothing
   const int K = a.K;
 
@@ -80,7 +84,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a, int
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
   const int steps = K / 32;
-  for (int c = wave; c * 4 < steps; c += WAVES) {
+  for (int c = wave; c * 4 < steps; c += waves) {
     const int s0 = c * 4;
     if (s0 + 4 <= steps) {
       bf16x8 w[4], u[4], x[4];
@@ -113,8 +117,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a, int
 #pragma unroll
   for (int v = 0; v < 4; ++v) {
     int f = 4 * j + v;
-    red[wave][0][r * 16 + f] = acc[v];
-    if (SWIGLU) red[wave][1][r * 16 + f] = accu[v];
+    red[(wave * HALVES) * 256 + r * 16 + f] = acc[v];
+    if (SWIGLU) red[(wave * HALVES + 1) * 256 + r * 16 + f] = accu[v];
   }
   __syncthreads();
   if (threadIdx.x < 256) {
@@ -123,9 +127,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a, int
     if (row < row_end && col < a.N && f < rows) {
       float v = 0.f, up = 0.f;
 #pragma unroll
-      for (int w = 0; w < WAVES; ++w) {
-        v += red[w][0][threadIdx.x];
-        if (SWIGLU) up += red[w][1][threadIdx.x];
+      for (int w = 0; w < (WAVES > 0 ? WAVES : 16); ++w) {
+        if (WAVES == 0 && w >= waves) break;
+        v += red[(w * HALVES) * 256 + threadIdx.x];
+        if (SWIGLU) up += red[(w * HALVES + 1) * 256 + threadIdx.x];
       }
       if (SWIGLU) {
         v = v / (1.f + __expf(-v)) * up;
@@ -138,10 +143,50 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a, int
   }
 }
 
+template <int WAVES, bool FULL, bool SWIGLU, typename TC>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a, int rows_arg) {
+  __shared__ float red[WAVES * (SWIGLU ? 2 : 1) * 256];
+  __shared__ int tile_info[3];
+  skinny_block<WAVES, FULL, SWIGLU, TC>(a, rows_arg, WAVES, blockIdx.x, blockIdx.y, red, tile_info);
+}
+
+// Two products that do not depend on each other in one launch: the first blocks are the
+// tiles of `b` (the dense product, whose blocks run longest), the rest the tiles of `a`.
+// With few rows every launch costs a fixed
+// time next to which the products themselves are short; together they pay it once and
+// their loads overlap. The block has the waves of the larger need; waves a problem
+// does not use leave at once.
+struct SkinnyPlan {
+  int waves;    // waves that share the K range
+  int rows;     // features per block
+  int grid_x;
+  int grid_y;
+};
+
+template <bool FULL_A, bool SW_A, typename TC_A, bool FULL_B, bool SW_B, typename TC_B>
+__global__ __launch_bounds__(1024) void gemm_skinny_pair_kernel(GemmArgs a, SkinnyPlan pa,
+                                                               GemmArgs b, SkinnyPlan pb) {
+  __shared__ float red[16 * 2 * 256];
+  __shared__ int tile_info[3];
+  const int wave = threadIdx.x >> 6;
+  int id = blockIdx.x;
+  const int blocks_b = pb.grid_x * pb.grid_y;
+  if (id < blocks_b) {
+    if (wave >= pb.waves) return;
+    skinny_block<0, FULL_B, SW_B, TC_B>(b, pb.rows, pb.waves, id % pb.grid_x, id / pb.grid_x, red,
+                                        tile_info);
+  } else {
+    id -= blocks_b;
+    if (wave >= pa.waves) return;
+    skinny_block<0, FULL_A, SW_A, TC_A>(a, pa.rows, pa.waves, id % pa.grid_x, id / pa.grid_x, red,
+                                        tile_info);
+  }
+}
+
 template <int WAVES>
 static void launch_skinny(const GemmArgs& a, int rows, hipStream_t stream) {
   int m_tiles = a.offsets ? min((a.M + SM - 1) / SM + a.groups, a.M) : (a.M + SM - 1) / SM;
-  dim3 grid((a.N + rows - 1) / rows, m_tiles);
+  dim3 grid((a.N + rows - 1) / rows, m_tiles);   // as plan_skinny counts them
   dim3 block(WAVES * 64);
   bool swiglu = a.epilogue == kEpilogueSwiGLU;
 #define NINFER_SKINNY(FULL)                                                                   \
@@ -168,25 +213,66 @@ bool gemm_skinny_takes(const GemmArgs& a) {
          ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0) && a.w_group_stride % 8 == 0;
 }
 
-int gemm_skinny(const GemmArgs& a, hipStream_t stream) {
-  // more waves per block when the grid alone would leave CUs idle
-  int m_tiles = a.offsets ? a.groups : (a.M + SM - 1) / SM;
+static SkinnyPlan plan_skinny(const GemmArgs& a) {
+  SkinnyPlan p;
+  // more waves per block when the grid alone would leave CUs idle (grouped: at most one tile
+  // per sorted row, and one partial tile per group)
+  p.grid_y = a.offsets ? min((a.M + SM - 1) / SM + a.groups, a.M) : (a.M + SM - 1) / SM;
+  int m_tiles = p.grid_y;
   long blocks = (long)((a.N + 15) / 16) * m_tiles;
   int chunks = a.K / 128;
   // features per block: 16, or for a dense product with few tiles the count that makes the
   // blocks a whole multiple of the CUs
-  int rows = 16;
+  p.rows = 16;
   const int cus = 256;
   if (!a.offsets && m_tiles == 1 && blocks < 8 * cus) {
     const int per_cu = (a.N + 16 * cus - 1) / (16 * cus);          // blocks each CU gets
-    rows = (a.N + per_cu * cus - 1) / (per_cu * cus);
+    p.rows = (a.N + per_cu * cus - 1) / (per_cu * cus);
   }
-  if (blocks < 512 && chunks >= 16)
-    launch_skinny<16>(a, rows, stream);
-  else if (blocks < 2048 && chunks >= 8)
-    launch_skinny<8>(a, rows, stream);
+  p.waves = (blocks < 512 && chunks >= 16) ? 16 : (blocks < 2048 && chunks >= 8) ? 8 : 4;
+  p.grid_x = (a.N + p.rows - 1) / p.rows;
+  return p;
+}
+
+int gemm_skinny(const GemmArgs& a, hipStream_t stream) {
+  const SkinnyPlan p = plan_skinny(a);
+  if (p.waves == 16)
+    launch_skinny<16>(a, p.rows, stream);
+  else if (p.waves == 8)
+    launch_skinny<8>(a, p.rows, stream);
   else
-    launch_skinny<4>(a, rows, stream);
+    launch_skinny<4>(a, p.rows, stream);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+// The pairs that have a kernel: (dense, 32-bit out) beside (dense SwiGLU), as a router's
+// logits beside a shared expert's gate and up; (grouped) beside (dense), as the experts'
+// down products beside the shared expert's. Both bf16 in, the second bf16 out.
+bool gemm_skinny_pair_takes(const GemmArgs& a, const GemmArgs& b) {
+  if (!gemm_skinny_takes(a) || !gemm_skinny_takes(b) || a.bias || b.bias) return false;
+  const bool dense_b = !b.offsets && b.out_dtype == kBF16;
+  const bool first = !a.offsets && a.out_dtype == kF32 && a.epilogue == kEpilogueNone &&
+                     dense_b && b.epilogue == kEpilogueSwiGLU;
+  const bool second = a.offsets && a.out_dtype == kBF16 && a.epilogue == kEpilogueNone &&
+                      dense_b && b.epilogue == kEpilogueNone;
+  return first || second;
+}
+
+int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream) {
+  SkinnyPlan pa = plan_skinny(a), pb = plan_skinny(b);
+  // beside a grouped product with many blocks, which are small, the dense one takes the same
+  // few waves: blocks as wide as the larger need would hold up the small blocks' places
+  if (a.offsets && (long)pa.grid_x * pa.grid_y >= 2048) pb.waves = pa.waves;
+  const int threads = 64 * max(pa.waves, pb.waves);
+  const long blocks = (long)pa.grid_x * pa.grid_y + (long)pb.grid_x * pb.grid_y;
+  NINFER_REQUIRE(blocks < (1L << 31), "gemm pair: %ld blocks are too many", blocks);
+  if (!a.offsets)
+    gemm_skinny_pair_kernel<false, false, float, false, true, bf16>
+        <<<(unsigned)blocks, threads, 0, stream>>>(a, pa, b, pb);
+  else
+    gemm_skinny_pair_kernel<true, false, bf16, false, false, bf16>
+        <<<(unsigned)blocks, threads, 0, stream>>>(a, pa, b, pb);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

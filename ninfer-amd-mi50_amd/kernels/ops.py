@@ -66,6 +66,23 @@ def _dev(t: torch.Tensor, name: str, dtype=None, dims: Optional[int] = None) -> 
         _need(t.dim() == dims, f"{name} must have {dims} dimensions, has {t.dim()}")
 
 
+class _Together:
+    def __init__(self, ops):
+        self.ops = ops
+
+    def __enter__(self):
+        if self.ops._held is not None:
+            raise KernelError("together(): already inside one")
+        self.ops._held = []
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        held, self.ops._held = self.ops._held, None
+        if exc_type is None:
+            self.ops._launch_held(held)
+        return False
+
+
 class HipOps:
     def __init__(self, lib_path: Optional[str] = None):
         self.lib_path = lib_path or ensure_built()
@@ -73,6 +90,7 @@ class HipOps:
         self.lib.ninfer_last_error.restype = ctypes.c_char_p
         self.lib.ninfer_attention_workspace_floats.restype = ctypes.c_longlong
         self.force_generic = False  # tests: run the plain kernels whatever the shape
+        self._held = None           # products held back inside `together()`
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
         self._attn_ws = None
 
@@ -208,8 +226,32 @@ class HipOps:
                          _ptr(a_index), _ptr(c_index), t16, t64, tc, w_group_stride, m, n, k,
                          a.shape[1],
                          c.shape[1], groups, a_div, _DT[a.dtype], _DT[c.dtype], epilogue, big)
+        if self._held is not None:
+            self._held.append((args, (a, w, c, bias, offsets, a_index, c_index, tiles)))
+            return
         self._ok(self.lib.ninfer_gemm(ctypes.byref(args), 1 if self.force_generic else 0,
                                       self._stream()))
+
+    def together(self):
+        """Context manager for products that do not depend on each other: the
+        hand-written ones called inside are held back and launched when it ends,
+        two at a time as one launch where such a pair has a kernel (few rows: a
+        launch's fixed time is paid once), otherwise one after the other. Outputs
+        are valid after the block, not inside it."""
+        return _Together(self)
+
+    def _launch_held(self, held):
+        force = 1 if self.force_generic else 0
+        i = 0
+        while i < len(held):
+            if i + 1 < len(held):
+                self._ok(self.lib.ninfer_gemm_pair(ctypes.byref(held[i][0]),
+                                                   ctypes.byref(held[i + 1][0]), force,
+                                                   self._stream()))
+                i += 2
+            else:
+                self._ok(self.lib.ninfer_gemm(ctypes.byref(held[i][0]), force, self._stream()))
+                i += 1
 
     def linear(self, x, w, out, bias=None):
         """out = x w^T (+ bias); out may be 32-bit whatever the inputs are."""

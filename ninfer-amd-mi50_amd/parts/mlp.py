@@ -39,12 +39,18 @@ class SwiGLU(FeedForward):
         w.matrix_into(p + "up_proj.weight", self.w_gate_up[self.inner:])
         self.w_down = w.matrix(p + "down_proj.weight")
 
-    def run(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
+    def gate_up(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
         h = ctx.empty((x.shape[0], self.inner))
         ctx.ops.swiglu_linear(x, self.w_gate_up, h)
-        out = ctx.empty((x.shape[0], self.hidden))
+        return h
+
+    def down(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
+        out = ctx.empty((h.shape[0], self.hidden))
         ctx.ops.linear(h, self.w_down, out)
         return out
+
+    def run(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
+        return self.down(ctx, self.gate_up(ctx, x))
 
     def forward(self, ctx: StepContext, x, residual):
         return self.run(ctx, x)

@@ -116,15 +116,23 @@ class RoutedExperts(Part):
             w.matrix_into(p + "up_proj.weight", self.w_gate_up[e, i:])
             w.matrix_into(p + "down_proj.weight", self.w_down[e])
 
-    def run(self, ctx: StepContext, x: torch.Tensor, routing: "Routing") -> torch.Tensor:
-        """Expert outputs [T*k, hidden], row t*k + j for the j-th choice of row t."""
+    def gate_up(self, ctx: StepContext, x: torch.Tensor, routing: "Routing") -> torch.Tensor:
+        """Activations [T*k, inner] in sorted order (row r belongs to the expert that
+        owns sorted position r)."""
         t, k = routing.ids.shape
         h = ctx.empty((t * k, self.inner))
         ctx.ops.grouped_swiglu(x, self.w_gate_up, routing.offsets, routing.order, k, h,
                                tiles=routing)
-        y = ctx.empty((t * k, self.hidden))
+        return h
+
+    def down(self, ctx: StepContext, h: torch.Tensor, routing: "Routing") -> torch.Tensor:
+        """Expert outputs [T*k, hidden], row t*k + j for the j-th choice of row t."""
+        y = ctx.empty((h.shape[0], self.hidden))
         ctx.ops.grouped_down(h, self.w_down, routing.offsets, routing.order, y, tiles=routing)
         return y
+
+    def run(self, ctx: StepContext, x: torch.Tensor, routing: "Routing") -> torch.Tensor:
+        return self.down(ctx, self.gate_up(ctx, x, routing), routing)
 
 
 class SparseMoE(FeedForward):
@@ -162,18 +170,23 @@ class SparseMoE(FeedForward):
             self.shared_gate = self.router_and_gate[e:]
 
     def forward(self, ctx: StepContext, x, residual):
-        shared = gate = None
-        if self.shared is not None:
-            logits = ctx.empty((x.shape[0], self.router.experts + 1), torch.float32)
+        if self.shared is None:
+            routing = self.router.route(ctx, self.router.logits(ctx, x))
+            self.last_ids = routing.ids
+            return PendingRows(self.experts.run(ctx, x, routing), routing.weights)
+        # The shared expert's two products wait for nothing the routed path makes: each goes
+        # together with the routed path's product of the same stage.
+        logits = ctx.empty((x.shape[0], self.router.experts + 1), torch.float32)
+        with ctx.ops.together():
             ctx.ops.linear(x, self.router_and_gate, logits)
-            gate = logits[:, self.router.experts]
-        else:
-            logits = self.router.logits(ctx, x)
+            h_shared = self.shared.gate_up(ctx, x)
+        gate = logits[:, self.router.experts]
         routing = self.router.route(ctx, logits)
         self.last_ids = routing.ids
-        y = self.experts.run(ctx, x, routing)
-        if self.shared is not None:
-            shared = self.shared.run(ctx, x)
+        h = self.experts.gate_up(ctx, x, routing)
+        with ctx.ops.together():
+            y = self.experts.down(ctx, h, routing)
+            shared = self.shared.down(ctx, h_shared)
         # not added here: the next norm's kernel adds it to the residual on the fly
         return PendingRows(y, routing.weights, shared, gate)
 

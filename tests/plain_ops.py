@@ -9,6 +9,7 @@ reference lines that tests/plain_model.py cites.
 """
 from __future__ import annotations
 
+import contextlib
 import math
 
 import torch
@@ -20,6 +21,10 @@ def _f(t):
 
 class PlainOps:
     force_generic = False
+
+    def together(self):
+        """Independent products: nothing to gain here, they run as they are called."""
+        return contextlib.nullcontext()
 
     def embed(self, tokens, table, out):
         out.copy_(_f(table[tokens.long()]))

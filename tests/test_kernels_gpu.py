@@ -294,6 +294,62 @@ def test_rmsnorm_adds_a_sum_of_rows_on_the_fly(ops, gen, dtype):
         assert torch.equal(x1, x)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("t,e,k,h,inner,shared_inner", [(1, 6, 2, 64, 32, 96), (8, 60, 4, 256, 160, 352),
+                                                        (5, 7, 3, 384, 96, 1000), (32, 8, 2, 128, 64, 2048),
+                                                        (3, 64, 8, 3584, 2560, 512), (40, 6, 2, 128, 64, 96)])
+def test_products_launched_together(ops_mode, gen, dtype, t, e, k, h, inner, shared_inner):
+    """Two independent products inside together(): 32-bit logits beside a SwiGLU,
+    and a grouped down product beside a dense one. Same results as one by one,
+    for few rows (one launch for both) and for more (the usual kernels)."""
+    ops = ops_mode
+    plain = PlainOps()
+    from ninfer_amd.parts.moe import Routing
+    x = rnd((t, h), dtype, gen)
+    w_router = rnd((e + 1, h), dtype, gen, 0.3)
+    w_gu = rnd((2 * shared_inner, h), dtype, gen, 0.3)
+    logits = torch.zeros(t, e + 1, device="cuda")
+    hs = torch.zeros(t, shared_inner, device="cuda", dtype=dtype)
+    with ops.together():
+        ops.linear(x, w_router, logits)
+        ops.swiglu_linear(x, w_gu, hs)
+    logits2, hs2 = torch.zeros_like(logits), torch.zeros_like(hs)
+    plain.linear(x, w_router, logits2)
+    plain.swiglu_linear(x, w_gu, hs2)
+    close(logits, logits2, torch.float32, scale=math.sqrt(h) * 0.3)
+    close(hs, hs2, dtype, scale=h * 0.3)
+
+    n = t * k
+    i32 = lambda *sh: torch.zeros(*sh, device="cuda", dtype=torch.int32)
+    r = Routing(i32(t, k), torch.zeros(t, k, device="cuda"), i32(e + 1), i32(n),
+                i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2))
+    ops.moe_route(logits2[:, :e].contiguous(), e, k, True, r)
+    hx = rnd((n, inner), dtype, gen)
+    wd = rnd((e, h, inner), dtype, gen, 0.3)
+    wsd = rnd((h, shared_inner), dtype, gen, 0.3)
+    for tiles in (r, None):
+        y = torch.zeros(n, h, device="cuda", dtype=dtype)
+        out = torch.zeros(t, h, device="cuda", dtype=dtype)
+        with ops.together():
+            ops.grouped_down(hx, wd, r.offsets, r.order, y, tiles=tiles)
+            ops.linear(hs2, wsd, out)
+        y2, out2 = torch.zeros_like(y), torch.zeros_like(out)
+        plain.grouped_down(hx, wd, r.offsets, r.order, y2)
+        plain.linear(hs2, wsd, out2)
+        close(y, y2, dtype, scale=math.sqrt(inner) * 0.3)
+        close(out, out2, dtype, scale=hs2.float().abs().max().item() * math.sqrt(shared_inner) * 0.3)
+    # an odd number of products, and an error inside leaves nothing held back
+    with ops.together():
+        ops.linear(x, w_router, logits)
+    close(logits, logits2, torch.float32, scale=math.sqrt(h) * 0.3)
+    with pytest.raises(ZeroDivisionError):
+        with ops.together():
+            ops.linear(x, w_router, logits)
+            1 / 0
+    ops.linear(x, w_router, logits)   # launches at once again
+    close(logits, logits2, torch.float32, scale=math.sqrt(h) * 0.3)
+
+
 def test_router_ties_go_to_the_lower_index(ops):
     logits = torch.zeros(2, 8, device="cuda")
     logits[1, 5] = 1.0
