@@ -49,7 +49,26 @@ CONFIG_B = {
     "hidden_act": "silu",
 }
 
-TINY = {"A": (CONFIG_A, 1234), "B": (CONFIG_B, 987)}
+# Heads of 64 in groups of three, so that the engine's bf16 steps run the matrix-core
+# attention kernels (prompt portions, and decoding with grouped heads); one layer sees all
+# keys, one a window.
+CONFIG_C = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe",
+    "num_hidden_layers": 2, "hidden_size": 128, "num_attention_heads": 6,
+    "num_key_value_heads": 2, "head_dim": 64, "intermediate_size": 160,
+    "moe_intermediate_size": 64, "shared_expert_intermediate_size": 96,
+    "num_experts": 6, "num_experts_per_tok": 2, "norm_topk_prob": True,
+    "decoder_sparse_step": 1, "mlp_only_layers": [], "vocab_size": 320,
+    "rope_theta": 500000.0, "use_sliding_window": True, "sliding_window": 40,
+    "max_window_layers": 1, "rms_norm_eps": 1e-5, "tie_word_embeddings": False,
+    "hidden_act": "silu",
+}
+
+TINY = {"A": (CONFIG_A, 1234), "B": (CONFIG_B, 987), "C": (CONFIG_C, 4321)}
+# Std of the random weights. With tiny widths, N(0, 0.02) leaves all logits and attention
+# scores near zero, which would hide faults: 0.1. C is wider, and 0.08 keeps its logits at
+# the size (std about 0.9) that the bf16 bounds of the tests were made for.
+TINY_STD = {"A": 0.1, "B": 0.1, "C": 0.08}
 
 
 @pytest.fixture(scope="session")
@@ -61,8 +80,6 @@ def model_dirs(tmp_path_factory):
         out[name] = {}
         for dtype in ("float32", "bfloat16"):
             d = str(tmp_path_factory.mktemp(f"tiny_{name}_{dtype}"))
-            # std 0.1 rather than 0.02: with tiny widths, N(0, 0.02) leaves all
-            # logits and attention scores near zero, which would hide faults
-            ninfer_amd.write_random_model(d, cfg, seed, dtype=dtype, std=0.1)
+            ninfer_amd.write_random_model(d, cfg, seed, dtype=dtype, std=TINY_STD[name])
             out[name][dtype] = d
     return out

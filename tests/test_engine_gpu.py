@@ -13,14 +13,14 @@ from conftest import TINY
 
 pytestmark = pytest.mark.gpu
 
-PROMPTS = {"A": [5, 11, 17, 60], "B": [3, 20, 33, 40, 75]}
+PROMPTS = {"A": [5, 11, 17, 60], "B": [3, 20, 33, 40, 75], "C": [7, 30, 70, 100]}
 
 
 def bound(dtype):
     return dict(atol=2e-5, rtol=1e-4) if dtype == "float32" else dict(atol=6e-2, rtol=5e-2)
 
 
-@pytest.fixture(scope="module", params=["A", "B"])
+@pytest.fixture(scope="module", params=["A", "B", "C"])
 def case(request, model_dirs):
     name = request.param
     cfg = TINY[name][0]

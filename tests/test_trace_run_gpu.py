@@ -16,7 +16,7 @@ from conftest import ROOT, TINY
 
 pytestmark = pytest.mark.gpu
 
-LENS = {"A": [17, 45, 60, 38], "B": [15, 52, 70, 45, 33]}
+LENS = {"A": [17, 45, 60, 38], "B": [15, 52, 70, 45, 33], "C": [20, 66, 90, 41]}
 
 
 def replay(model_dir, dtype, steps, out_dir, max_tokens, vocab):
@@ -31,7 +31,7 @@ def replay(model_dir, dtype, steps, out_dir, max_tokens, vocab):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_trace_replay_all_ways(model_dirs, tmp_path, name, dtype):
     d = model_dirs[name][dtype]
     cfg, w = util.read_folder(d)
