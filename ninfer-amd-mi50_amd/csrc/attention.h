@@ -31,6 +31,8 @@ struct AttnArgs {
   int dtype;
   int max_qlen;             // host-side bounds used to size launches
   int max_kv_len;
+  int single_rows;          // the first single_rows requests bring one row each: rows
+                            // 0 .. single_rows - 1 (0 when the caller does not sort them)
 };
 
 int attention_generic(const void* q, int q_stride, const void* kpool, const void* vpool,

@@ -20,8 +20,30 @@ extern "C" int ninfer_paged_attention(const AttnArgs* a, int force_generic, hipS
   NINFER_REQUIRE(a->q_stride >= a->Hq * a->D, "paged_attention: row stride %d < %d", a->q_stride,
                  a->Hq * a->D);
   NINFER_REQUIRE(a->max_qlen >= 1 && a->max_kv_len >= 1, "paged_attention: bad size hints");
+  NINFER_REQUIRE(a->single_rows >= 0 && a->single_rows <= a->S && a->single_rows <= a->T,
+                 "paged_attention: %d single rows of %d requests", a->single_rows, a->S);
   if (!force_generic && a->max_qlen == 1 && attention_decode_takes(*a))
     return attention_decode(*a, stream);
+  if (!force_generic && a->single_rows > 0 && a->single_rows < a->S &&
+      attention_decode_takes(*a) && attention_prefill_takes(*a)) {
+    // A step that mixes decoded tokens with prompt portions: the single rows, which come
+    // first, walk their contexts split over many blocks; in the prompt kernel each would be
+    // one block that walks its whole context alone.
+    const int n = a->single_rows;
+    AttnArgs d = *a;
+    d.T = n;
+    d.S = n;
+    d.max_qlen = 1;
+    if (int rc = attention_decode(d, stream)) return rc;
+    AttnArgs p = *a;   // rows and their positions stay where they are: only the requests move
+    p.seq_row_start += n;
+    p.seq_qlen += n;
+    p.seq_pos0 += n;
+    p.block_table += (int64_t)n * a->bt_stride;
+    p.S = a->S - n;
+    p.T = a->T - n;
+    return attention_prefill(p, stream);
+  }
   if (!force_generic && attention_prefill_takes(*a)) return attention_prefill(*a, stream);
   return attention_generic(a->q, a->q_stride, a->kpool, a->vpool, a->block_table, a->bt_stride,
                            a->positions, a->row_seq, a->out, a->T, a->Hq, a->Hkv, a->D,

@@ -87,13 +87,19 @@ class ModelRunner:
         if not chunks:
             return None
         cache = self.cache
+        for c in chunks:
+            if len(c.tokens) < 1:
+                raise ValueError("a request in a step brings at least one token")
+        # Requests that bring one token go first (a stable sort), so that their rows are the
+        # step's first: attention then runs them apart from the prompt portions. The wanted
+        # rows keep the order of the caller's chunks.
+        given = chunks
+        chunks = sorted(given, key=lambda c: len(c.tokens) != 1)
+        single_rows = sum(1 for c in chunks if len(c.tokens) == 1)
         slots = [c.slot for c in chunks]
         if len(set(slots)) != len(slots):
             raise ValueError("a request may appear once in a step")
         pos0 = [cache.length(c.slot) for c in chunks]
-        for c in chunks:
-            if len(c.tokens) < 1:
-                raise ValueError("a request in a step brings at least one token")
         T = sum(len(c.tokens) for c in chunks)
         S = len(chunks)
         tokens = np.empty(T, np.int32)
@@ -101,7 +107,7 @@ class ModelRunner:
         row_seq = np.empty(T, np.int32)
         row_start = np.empty(S + 1, np.int32)
         qlen = np.empty(S, np.int32)
-        want_rows: List[int] = []
+        first_row = {}
         r = 0
         for i, (c, p) in enumerate(zip(chunks, pos0)):
             n = len(c.tokens)
@@ -110,12 +116,16 @@ class ModelRunner:
             row_seq[r:r + n] = i
             row_start[i] = r
             qlen[i] = n
-            for w in c.want:
-                if not 0 <= w < n:
-                    raise ValueError(f"wanted row {w} is outside the request's {n} tokens")
-                want_rows.append(r + w)
+            first_row[c.slot] = r
             r += n
         row_start[S] = T
+        want_rows: List[int] = []
+        for c in given:
+            for w in c.want:
+                if not 0 <= w < len(c.tokens):
+                    raise ValueError(f"wanted row {w} is outside the request's "
+                                     f"{len(c.tokens)} tokens")
+                want_rows.append(first_row[c.slot] + w)
         if tokens.min() < 0 or tokens.max() >= self.vocab_size:
             raise ValueError(f"token id outside [0, {self.vocab_size})")
         # the batch is well formed: now pages for all its requests, or for none
@@ -135,7 +145,8 @@ class ModelRunner:
         sizes = [x.size for x in parts]
         host = torch.from_numpy(np.concatenate(parts))
         shape = dict(T=T, S=S, sizes=sizes, widths=[t.shape[1] for t in tables],
-                     max_qlen=int(qlen.max()), max_kv_len=max_kv_len, wants=bool(want_rows))
+                     max_qlen=int(qlen.max()), max_kv_len=max_kv_len, wants=bool(want_rows),
+                     single_rows=single_rows)
         if graph:
             logits = self._step_graph(host, shape)
         else:
@@ -163,7 +174,7 @@ class ModelRunner:
             tokens=views[0], positions=views[1], row_seq=views[2], seq_slots=views[3],
             seq_row_start=views[4], seq_qlen=views[5], seq_pos0=views[6],
             max_qlen=shape["max_qlen"], max_kv_len=shape["max_kv_len"],
-            all_decode=shape["max_qlen"] == 1)
+            all_decode=shape["max_qlen"] == 1, single_rows=shape["single_rows"])
         return self.spec.forward(ctx, self._call_infos(d_tables),
                                  views[7] if shape["wants"] else None)
 

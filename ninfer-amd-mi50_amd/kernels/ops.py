@@ -45,7 +45,7 @@ class _AttnArgs(ctypes.Structure):
                 ("S", ctypes.c_int), ("Hq", ctypes.c_int), ("Hkv", ctypes.c_int),
                 ("D", ctypes.c_int), ("page_size", ctypes.c_int), ("window", ctypes.c_int),
                 ("scale", ctypes.c_float), ("dtype", ctypes.c_int), ("max_qlen", ctypes.c_int),
-                ("max_kv_len", ctypes.c_int)]
+                ("max_kv_len", ctypes.c_int), ("single_rows", ctypes.c_int)]
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -410,9 +410,11 @@ class HipOps:
         _need(block_table.shape[0] == ctx.S, "paged_attention: block table rows != requests")
         _need(ctx.positions.shape[0] == t, "paged_attention: positions size")
         ws, ws_floats = None, 0
-        if ctx.max_qlen == 1 and qkv.dtype == torch.bfloat16 and not self.force_generic:
-            ws_floats = int(self.lib.ninfer_attention_workspace_floats(t, n_q, head_dim,
-                                                                       ctx.max_kv_len))
+        single = int(getattr(ctx, "single_rows", 0))
+        if (ctx.max_qlen == 1 or single > 0) and qkv.dtype == torch.bfloat16 \
+                and not self.force_generic:
+            ws_floats = int(self.lib.ninfer_attention_workspace_floats(
+                t if ctx.max_qlen == 1 else single, n_q, head_dim, ctx.max_kv_len))
             if self._attn_ws is None or self._attn_ws.numel() < ws_floats:
                 self._attn_ws = torch.empty(ws_floats, dtype=torch.float32, device=qkv.device)
             ws = self._attn_ws.data_ptr()
@@ -421,7 +423,7 @@ class HipOps:
             block_table.data_ptr(), ctx.positions.data_ptr(), ctx.row_seq.data_ptr(),
             ctx.seq_row_start.data_ptr(), ctx.seq_qlen.data_ptr(), ctx.seq_pos0.data_ptr(),
             ws, ws_floats, qkv.shape[1], block_table.shape[1], t, ctx.S, n_q, n_kv, head_dim, page_size,
-            int(window or 0), float(scale), _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len)
+            int(window or 0), float(scale), _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len, single)
         self._ok(self.lib.ninfer_paged_attention(ctypes.byref(args),
                                                  1 if self.force_generic else 0, self._stream()))
 

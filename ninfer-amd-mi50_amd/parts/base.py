@@ -72,6 +72,7 @@ class StepContext:
     max_qlen: int = 1
     max_kv_len: int = 1
     all_decode: bool = False
+    single_rows: int = 0          # the first single_rows requests bring one row each (rows 0 ..)
     scratch: Dict[str, Any] = field(default_factory=dict)
 
     def empty(self, shape, dtype=None) -> torch.Tensor:

@@ -440,6 +440,30 @@ def test_paged_attention_decode_rows(ops_mode, gen, dtype, n_q, n_kv, d, page_si
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_q,n_kv,d,page_size,window", [
+    (16, 16, 128, 16, 0), (28, 4, 128, 16, 0), (6, 2, 64, 32, 40), (4, 2, 64, 8, 300),
+    (3, 1, 32, 8, 24)])
+def test_paged_attention_single_rows_first(ops_mode, gen, dtype, n_q, n_kv, d, page_size, window):
+    """A mixed step whose single-token requests come first and are announced as such:
+    they run on the split-context kernel, the portions on the prompt kernel."""
+    ops = ops_mode
+    seqs = [(700, 1), (15, 1), (255, 1), (0, 37), (390, 300), (64, 64), (9, 2)]
+    ctx, qkv, k_pool, v_pool, bt = _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, 80)
+    scale = 1 / math.sqrt(d)
+    o2 = torch.empty(ctx.T, n_q * d, device="cuda", dtype=dtype)
+    PlainOps().paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, page_size, window,
+                               scale, o2)
+    for single in (3, 1, 0):
+        ctx.single_rows = single
+        o1 = torch.zeros(ctx.T, n_q * d, device="cuda", dtype=dtype)
+        ops.paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, page_size, window, scale, o1)
+        close(o1, o2, dtype)
+    ctx.single_rows = len(seqs) + 1
+    with pytest.raises(Exception):
+        ops.paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, page_size, window, scale, o1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_finds_a_far_key(ops_mode, gen, dtype):
     """One key among hundreds is made to dominate: the output must be its
     value, wherever it lies (a page's first or last slot, far back)."""
