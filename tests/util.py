@@ -228,3 +228,31 @@ def read_trace_output(out_dir: str, steps: List[Step], vocab: int) -> Dict[str, 
                 rows.setdefault(r, []).append(torch.from_numpy(arr[o:o + len(w)].copy()))
                 o += len(w)
     return {k: torch.cat(v) for k, v in rows.items()}
+
+
+def random_config(seed: int) -> dict:
+    """A seeded random configuration of the architecture: head sizes in steps of 16, head
+    counts and groups of every kind, widths and vocabularies that are no power of two,
+    one expert or many, with and without windows."""
+    rng = random.Random(seed)
+    nkv = rng.choice([1, 2, 3, 5])
+    group = rng.choice([1, 1, 2, 3, 4, 7])
+    experts = rng.choice([1, 2, 3, 5, 8, 17, 60, 70])
+    window = rng.choice([None, None, 8, 24, 40, 70])
+    layers = rng.randint(1, 3)
+    return {
+        "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe",
+        "num_hidden_layers": layers, "hidden_size": rng.choice([48, 64, 72, 96, 100, 128, 136, 160, 200]),
+        "num_attention_heads": nkv * group, "num_key_value_heads": nkv,
+        "head_dim": rng.choice([16, 32, 48, 64, 80, 96, 112, 128]),
+        "intermediate_size": rng.choice([40, 64, 100, 192]),
+        "moe_intermediate_size": rng.choice([16, 24, 32, 40, 64, 100]),
+        "shared_expert_intermediate_size": rng.choice([16, 48, 64, 96, 130]),
+        "num_experts": experts, "num_experts_per_tok": rng.randint(1, min(experts, 6)),
+        "norm_topk_prob": rng.random() < 0.5, "decoder_sparse_step": rng.choice([1, 1, 2]),
+        "mlp_only_layers": rng.choice([[], [0]]), "vocab_size": rng.choice([97, 256, 333, 1001]),
+        "rope_theta": rng.choice([10000.0, 1000000.0]), "use_sliding_window": window is not None,
+        "sliding_window": window or 4096, "max_window_layers": rng.randint(0, layers),
+        "rms_norm_eps": rng.choice([1e-6, 1e-5]), "tie_word_embeddings": rng.random() < 0.5,
+        "hidden_act": "silu",
+    }
