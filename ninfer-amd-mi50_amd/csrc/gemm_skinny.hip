@@ -228,6 +228,10 @@ static SkinnyPlan plan_skinny(const GemmArgs& a) {
   if (!a.offsets && m_tiles == 1 && blocks < 8 * cus) {
     const int per_cu = (a.N + 16 * cus - 1) / (16 * cus);          // blocks each CU gets
     p.rows = (a.N + per_cu * cus - 1) / (per_cu * cus);
+  } else if (a.offsets && a.M <= 8 && blocks < 8 * cus) {
+    // a single token's choices: one tile per sorted row (its experts differ), counted alike
+    const long per_cu = ((long)a.N * m_tiles + 16 * cus - 1) / (16 * cus);
+    p.rows = (int)(((long)a.N * m_tiles + per_cu * cus - 1) / (per_cu * cus));
   }
   p.waves = (blocks < 512 && chunks >= 16) ? 16 : (blocks < 2048 && chunks >= 8) ? 8 : 4;
   p.grid_x = (a.N + p.rows - 1) / p.rows;
@@ -263,6 +267,10 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream) {
   SkinnyPlan pa = plan_skinny(a), pb = plan_skinny(b);
   // beside a grouped product with many blocks, which are small, the dense one takes the same
   // few waves: blocks as wide as the larger need would hold up the small blocks' places
+  if (a.offsets) {   // the pair's grouped kernel has whole tiles of 16 features
+    pa.rows = 16;
+    pa.grid_x = (a.N + 15) / 16;
+  }
   if (a.offsets && (long)pa.grid_x * pa.grid_y >= 2048) pb.waves = pa.waves;
   const int threads = 64 * max(pa.waves, pb.waves);
   const long blocks = (long)pa.grid_x * pa.grid_y + (long)pb.grid_x * pb.grid_y;
