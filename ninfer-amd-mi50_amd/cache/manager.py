@@ -72,6 +72,10 @@ class CacheManager:
         self._length: Dict[int, int] = {}
         self.pools: Dict[int, Tuple[object, object]] = {}
         self.state = None
+        # debugging: pages given back are filled with NaN in every pool of their group, so
+        # that a read of a page that is no longer held (or of a slot not yet written in a page
+        # that is used again) shows in the logits
+        self.poison_freed = False
 
     # ---- device memory -----------------------------------------------------
     def allocate_pools(self, device, dtype) -> None:
@@ -112,9 +116,19 @@ class CacheManager:
         if slot not in self._length:
             raise RuntimeError(f"slot {slot} released but not held")
         for g in self.groups:
-            g.allocator.free([p for p in g.tables.pop(slot) if p >= 0])
+            self._give_back(g, [p for p in g.tables.pop(slot) if p >= 0])
         del self._length[slot]
         self._free_slots.append(slot)
+
+    def _give_back(self, g: CacheGroup, pages: List[int]) -> None:
+        g.allocator.free(pages)
+        if self.poison_freed and pages and self.pools:
+            import torch
+            for i in g.instances:
+                k_pool, v_pool = self.pools[i]
+                idx = torch.tensor(pages, dtype=torch.int64, device=k_pool.device)
+                k_pool.index_fill_(0, idx, float("nan"))
+                v_pool.index_fill_(0, idx, float("nan"))
 
     def length(self, slot: int) -> int:
         return self._length[slot]
@@ -181,7 +195,7 @@ class CacheManager:
                     table[p] = -1
                     g.rows[slot, p] = -1
             if gone:
-                g.allocator.free(gone)
+                self._give_back(g, gone)
                 g.window_freed += len(gone)
 
     # ---- what a step needs ---------------------------------------------------

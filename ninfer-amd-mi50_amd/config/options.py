@@ -19,6 +19,7 @@ class EngineOptions:
     page_size: int = 16            # tokens per cache page
     num_pages: Optional[int] = None  # pages per cache group; None: enough for every request at max_context
     use_graph: bool = False        # replay decode-only steps from a captured HIP graph
+    poison_freed_pages: bool = False  # debugging: fill pages that are given back with NaN
     device: str = "cuda:0"
 
     def validate(self) -> None:

@@ -66,6 +66,7 @@ class ModelRunner:
         self.cache = CacheManager(needs, options.page_size, options.pool_pages(),
                                   options.num_sequences, options.max_context, floats)
         self.cache.allocate_pools(self.device, self.act_dtype)
+        self.cache.poison_freed = options.poison_freed_pages
         self.vocab_size = spec.vocab_size
         self.steps_run = 0
         self._graphs: Dict[tuple, dict] = {}

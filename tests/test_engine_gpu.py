@@ -75,6 +75,27 @@ def test_mixed_with_page_reuse(case, dtype, page_size, num_pages):
         assert any(g.window_freed > 0 for g in runner.cache.groups)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_given_back_are_never_read(case, dtype):
+    """Pages that are given back (a finished request, a window that has passed them) are
+    filled with NaN: a kernel that read a page it no longer holds, or a slot of a reused
+    page that it has not written yet, would carry the NaN into the logits."""
+    from ninfer_amd import EngineOptions, load_model
+    for page_size, num_pages in ((4, 60), (16, 16)):
+        opt = EngineOptions(dtype=dtype, max_context=128, num_sequences=4, page_size=page_size,
+                            num_pages=num_pages, poison_freed_pages=True)
+        runner = load_model(case["dirs"][dtype], opt)
+        reqs = dict(case["reqs"])
+        for seed in (7, 8):   # the second pass starts on pages that the first has poisoned
+            got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=seed))
+            for rid in reqs:
+                assert torch.isfinite(got[rid]).all(), f"{case['name']} {rid}: NaN from a freed page"
+                torch.testing.assert_close(got[rid], case["ref"][dtype][rid], **bound(dtype),
+                                           msg=lambda m: f"{case['name']} {rid} poisoned: {m}")
+        k_pool = next(iter(runner.cache.pools.values()))[0]
+        assert torch.isnan(k_pool).any(), "pages were given back, so some are poisoned now"
+
+
 def test_32bit_does_not_depend_on_the_cut(case):
     """In 32-bit every way of cutting gives the same logits to the last bit or
     nearly so (far inside the bound against the plain implementation)."""
