@@ -487,6 +487,52 @@ def test_paged_attention_finds_a_far_key(ops_mode, gen, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_q,n_kv,d,ps", [(4, 2, 64, 16), (6, 2, 64, 8), (28, 4, 128, 16),
+                                           (3, 1, 32, 4)])
+def test_paged_attention_window_edge(ops_mode, gen, dtype, n_q, n_kv, d, ps):
+    """The key that a window has just passed is made to dominate every query: the output
+    must not change. Then the oldest key still inside is made to dominate: the output must
+    be its value. For a decoded row (both split-context kernels) and for the rows of a
+    portion (the prompt kernel)."""
+    ops = ops_mode
+    window, group = 37, n_q // n_kv
+    seqs = [(300, 1), (270, 70)]
+    scale = 1 / math.sqrt(d)
+
+    def run(ctx, qkv, k_pool, v_pool, bt):
+        out = torch.empty(ctx.T, n_q * d, device="cuda", dtype=dtype)
+        ops.paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, ps, window, scale, out)
+        return out
+
+    for seq, row, pos in ((0, 0, 300), (1, 1 + 69, 339), (1, 1 + 5, 275)):
+        ctx, qkv, k_pool, v_pool, bt = _attention_case(gen, dtype, seqs, n_q, n_kv, d, ps, 120)
+        base = run(ctx, qkv, k_pool, v_pool, bt)
+        outside, inside = pos - window, pos - window + 1
+        for key, seen in ((outside, False), (inside, True)):
+            page = int(bt[seq, key // ps])
+            k_pool[page, :, key % ps, :] = torch.sign(k_pool[page, :, key % ps, :].float()).to(dtype)
+            q = qkv.clone()
+            for h in range(n_q):
+                q[row, h * d:(h + 1) * d] = (8 * k_pool[page, h // group, key % ps, :].float()).to(dtype)
+            out = run(ctx, q, k_pool, v_pool, bt)
+            for h in range(n_q):
+                got = out[row, h * d:(h + 1) * d].float()
+                value = v_pool[page, h // group, key % ps, :].float()
+                if seen:
+                    torch.testing.assert_close(got, value, atol=2e-2, rtol=2e-2)
+                else:
+                    assert (got - value).abs().max() > 0.2, "a key outside the window was seen"
+            # rows other than the one whose queries were changed keep their output
+            keep = [r for r in range(ctx.T) if r != row]
+            if not seen:
+                # the changed key lies outside the window of every row at or after `pos`, and
+                # the earlier rows of the request may see it: compare only the later ones
+                keep = [r for r in keep if ctx.positions[r].item() >= pos or
+                        ctx.row_seq[r].item() != seq]
+                torch.testing.assert_close(out[keep].float(), base[keep].float(), atol=1e-6, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_q,n_kv,d,rot", [(4, 2, 16, 16), (3, 1, 32, 32), (16, 16, 128, 128),
                                             (5, 5, 48, 24), (2, 1, 64, 0), (3, 1, 64, 32),
                                             (28, 4, 128, 128)])
