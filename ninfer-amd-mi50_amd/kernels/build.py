@@ -8,6 +8,7 @@ is kept beside it); `build(force=True)` always compiles.
 from __future__ import annotations
 
 import concurrent.futures
+import fcntl
 import glob
 import hashlib
 import os
@@ -98,6 +99,17 @@ def build(force: bool = True, jobs: int = 8) -> str:
     srcs = sources()
     if not srcs:
         raise RuntimeError(f"no HIP sources under {CSRC}")
+    # one build at a time per folder: a second process waits, then finds the library made
+    with open(os.path.join(out_dir, ".lock"), "w") as lock:
+        fcntl.flock(lock, fcntl.LOCK_EX)
+        if not force:
+            lib = _matching_library()
+            if lib:
+                return lib
+        return _compile_and_link(srcs, out_dir, jobs)
+
+
+def _compile_and_link(srcs: List[str], out_dir: str, jobs: int) -> str:
     hipcc = _hipcc()
     _say(f"compiling {len(srcs)} HIP sources for {ARCH} into {out_dir}")
     t0 = time.time()
