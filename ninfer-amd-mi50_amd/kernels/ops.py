@@ -48,6 +48,17 @@ class _AttnArgs(ctypes.Structure):
                 ("max_kv_len", ctypes.c_int), ("single_rows", ctypes.c_int)]
 
 
+class _QkvRopeArgs(ctypes.Structure):
+    _fields_ = [("x", ctypes.c_void_p), ("w", ctypes.c_void_p), ("bias", ctypes.c_void_p),
+                ("qkv", ctypes.c_void_p), ("positions", ctypes.c_void_p),
+                ("row_seq", ctypes.c_void_p), ("inv_freq", ctypes.c_void_p),
+                ("kpool", ctypes.c_void_p), ("vpool", ctypes.c_void_p),
+                ("block_table", ctypes.c_void_p), ("T", ctypes.c_int), ("K", ctypes.c_int),
+                ("lda", ctypes.c_int), ("Hq", ctypes.c_int), ("Hkv", ctypes.c_int),
+                ("D", ctypes.c_int), ("bt_stride", ctypes.c_int), ("page_size", ctypes.c_int),
+                ("write_kv", ctypes.c_int)]
+
+
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
@@ -191,6 +202,44 @@ class HipOps:
             ctypes.c_void_p(k_pool.data_ptr()), ctypes.c_void_p(v_pool.data_ptr()),
             ctypes.c_void_p(block_table.data_ptr()), block_table.shape[1], page_size,
             1 if write_kv else 0, t, _DT[qkv.dtype], self._stream()))
+
+    def qkv_rope(self, x, w_qkv, bias, qkv, positions, row_seq, inv_freq, rot_dim, n_q, n_kv,
+                 head_dim, k_pool, v_pool, block_table, page_size, write_kv=True):
+        """qkv = x w_qkv^T, then what `rope_kv_write` does. Few bf16 rows with a full
+        rotation run as one kernel; everything else as the product and the rotation
+        kernel one after the other."""
+        t = x.shape[0]
+        fused = (not self.force_generic and x.dtype == torch.bfloat16 and x.dim() == 2
+                 and self.lib.ninfer_qkv_rope_takes(t, x.shape[1], x.shape[1], head_dim, rot_dim))
+        if not fused:
+            self.linear(x, w_qkv, qkv)
+            self.rope_kv_write(qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv,
+                               head_dim, k_pool, v_pool, block_table, page_size, write_kv)
+            return
+        width = (n_q + 2 * n_kv) * head_dim
+        _dev(x, "x", torch.bfloat16, 2)
+        _dev(w_qkv, "w_qkv", torch.bfloat16, 2)
+        _dev(qkv, "qkv", torch.bfloat16, 2)
+        _need(w_qkv.shape == (width, x.shape[1]) and qkv.shape == (t, width), "qkv_rope: shapes")
+        if bias is not None:
+            _dev(bias, "bias", torch.float32, 1)
+            _need(bias.shape[0] == width, "qkv_rope: bias has the wrong size")
+        _dev(positions, "positions", torch.int32, 1)
+        _dev(row_seq, "row_seq", torch.int32, 1)
+        _need(positions.shape[0] == t and row_seq.shape[0] == t, "qkv_rope: index sizes")
+        _dev(inv_freq, "inv_freq", torch.float32, 1)
+        _need(inv_freq.shape[0] == head_dim // 2, "qkv_rope: table size != head_dim / 2")
+        _dev(k_pool, "k_pool", torch.bfloat16, 4)
+        _dev(v_pool, "v_pool", torch.bfloat16, 4)
+        _need(k_pool.shape == v_pool.shape and k_pool.shape[1:] == (n_kv, page_size, head_dim),
+              "qkv_rope: pools do not fit the head layout")
+        _dev(block_table, "block_table", torch.int32, 2)
+        args = _QkvRopeArgs(x.data_ptr(), w_qkv.data_ptr(), _ptr(bias), qkv.data_ptr(),
+                            positions.data_ptr(), row_seq.data_ptr(), inv_freq.data_ptr(),
+                            k_pool.data_ptr(), v_pool.data_ptr(), block_table.data_ptr(), t,
+                            x.shape[1], x.shape[1], n_q, n_kv, head_dim, block_table.shape[1],
+                            page_size, 1 if write_kv else 0)
+        self._ok(self.lib.ninfer_qkv_rope(ctypes.byref(args), self._stream()))
 
     def moe_combine(self, residual, y, wts, shared=None, gate=None):
         _dev(residual, "residual", torch.float32, 2)

@@ -80,12 +80,11 @@ class Attention(Mixer):
         ops = ctx.ops
         cache = call.cache
         qkv = ctx.empty((ctx.T, self.qkv_width))
-        ops.linear(x, self.w_qkv, qkv)
-        # bias, rotation of q (in place) and k, and the write of k, v into pages
-        ops.rope_kv_write(qkv, self.b_qkv, ctx.positions, ctx.row_seq, self.position.table(),
-                          self.position.rot_dim, self.heads, self.kv_heads, self.head_dim,
-                          cache.k_pool, cache.v_pool, cache.block_table, cache.page_size,
-                          write_kv=call.writes_cache)
+        # the product, then bias, rotation of q and k, and the write of k, v into pages
+        ops.qkv_rope(x, self.w_qkv, self.b_qkv, qkv, ctx.positions, ctx.row_seq,
+                     self.position.table(), self.position.rot_dim, self.heads, self.kv_heads,
+                     self.head_dim, cache.k_pool, cache.v_pool, cache.block_table,
+                     cache.page_size, write_kv=call.writes_cache)
         attn = ctx.empty((ctx.T, self.heads * self.head_dim))
         ops.paged_attention(qkv, cache.k_pool, cache.v_pool, cache.block_table, ctx,
                             self.heads, self.kv_heads, self.head_dim,

@@ -48,6 +48,12 @@ class PlainOps:
         ms = (v * v).sum(-1, keepdim=True) / v.shape[-1]
         out.copy_((v * torch.rsqrt(ms + eps) * gain).to(out.dtype))
 
+    def qkv_rope(self, x, w_qkv, bias, qkv, positions, row_seq, inv_freq, rot_dim, n_q, n_kv,
+                 head_dim, k_pool, v_pool, block_table, page_size, write_kv=True):
+        self.linear(x, w_qkv, qkv)
+        self.rope_kv_write(qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv, head_dim,
+                           k_pool, v_pool, block_table, page_size, write_kv)
+
     def rope_kv_write(self, qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv, head_dim,
                       k_pool, v_pool, block_table, page_size, write_kv=True):
         t = qkv.shape[0]

@@ -561,6 +561,41 @@ def test_rope_kv_write(ops, gen, dtype, n_q, n_kv, d, rot, seqs):
                 assert torch.equal(k1, k_pool) and torch.equal(v1, v_pool)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_q,n_kv,d,rot,hidden", [(4, 2, 16, 16, 64), (16, 16, 128, 128, 256),
+                                                   (28, 4, 128, 128, 160), (3, 1, 48, 48, 96),
+                                                   (5, 5, 80, 80, 72), (6, 2, 64, 32, 64),
+                                                   (2, 1, 64, 0, 96)])
+@pytest.mark.parametrize("seqs", [[(1000, 1)], [(0, 1), (77, 1), (8, 1), (300, 1), (31, 1)],
+                                  [(5, 20), (40, 1), (300, 1)], [(0, 33), (9, 2)]],
+                         ids=["one", "five", "22", "35"])
+def test_qkv_rope(ops_mode, gen, dtype, n_q, n_kv, d, rot, hidden, seqs):
+    """The product, the rotation and the cache write as one call: few bf16 rows with a full
+    rotation run as one kernel, the rest as the two kernels; both against the twins."""
+    from ninfer_amd.parts.rotary import Rotary
+    ops = ops_mode
+    ps = 8
+    ctx, qkv, k_pool, v_pool, bt = _attention_case(gen, dtype, seqs, n_q, n_kv, d, ps, 200)
+    table = Rotary(rot, 1e4).inv_freq().cuda() if rot else None
+    x = rnd((ctx.T, hidden), dtype, gen)
+    w = rnd((qkv.shape[1], hidden), dtype, gen, 0.3)
+    bias = torch.randn(qkv.shape[1], generator=gen, device="cuda")
+    for b in (None, bias):
+        for write in (True, False):
+            q1, q2 = torch.zeros_like(qkv), torch.zeros_like(qkv)
+            k1, k2, v1, v2 = k_pool.clone(), k_pool.clone(), v_pool.clone(), v_pool.clone()
+            ops.qkv_rope(x, w, b, q1, ctx.positions, ctx.row_seq, table, rot, n_q, n_kv, d, k1, v1,
+                         bt, ps, write_kv=write)
+            PlainOps().qkv_rope(x, w, b, q2, ctx.positions, ctx.row_seq, table, rot, n_q, n_kv, d,
+                                k2, v2, bt, ps, write_kv=write)
+            scale = math.sqrt(hidden) * 0.3 + 3
+            close(q1[:, :n_q * d], q2[:, :n_q * d], dtype, scale=scale)
+            close(k1, k2, dtype, scale=scale)
+            close(v1, v2, dtype, scale=scale)
+            if not write:
+                assert torch.equal(k1, k_pool) and torch.equal(v1, v_pool)
+
+
 def test_sample_greedy_and_distribution(ops, gen):
     import plain_model
     v = 1000
