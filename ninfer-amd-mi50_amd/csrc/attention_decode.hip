@@ -15,6 +15,9 @@
 // them. Lane groups, then waves, are merged by the usual log-sum-exp rule and
 // the chunk's (m, l, acc) goes to the workspace.
 // Pass 2, grid (rows, query heads): merges the chunks of a row in a fixed order.
+// With three or more query heads per kv head (and heads of 64 or 128), pass 1 is the
+// matrix-core kernel of attention_prefill.hip with the heads of a kv head as its rows;
+// it writes the same (m, l, acc) per chunk, and pass 2 is the same.
 //
 // Scores, softmax and sums are 32-bit. A row sees keys lo..pos with
 // lo = max(0, pos - window + 1); chunks are aligned to absolute positions.
@@ -299,6 +302,9 @@ int attention_decode(const AttnArgs& a, hipStream_t stream) {
   const int n_chunks = (a.max_kv_len + chunk - 1) / chunk;
   NINFER_REQUIRE(a.workspace_floats >= attention_decode_workspace_floats(a.T, a.Hq, a.D, a.max_kv_len),
                  "paged_attention: workspace of %lld floats is too small", (long long)a.workspace_floats);
+  const size_t merge_lds = (2 * (size_t)n_chunks + kMergeThreads) * sizeof(float);
+  NINFER_REQUIRE(merge_lds <= 48 * 1024, "paged_attention: a context of %d keys has too many chunks to merge",
+                 a.max_kv_len);
   if (attention_decode_heads_takes(a)) {
     // three or more query heads per kv head: their products go to the matrix cores
     if (int rc = attention_decode_heads(a, chunk, n_chunks, stream)) return rc;
@@ -313,9 +319,6 @@ int attention_decode(const AttnArgs& a, hipStream_t stream) {
     }
   }
   NINFER_LAUNCH_CHECK();
-  const size_t merge_lds = (2 * (size_t)n_chunks + kMergeThreads) * sizeof(float);
-  NINFER_REQUIRE(merge_lds <= 48 * 1024, "paged_attention: a context of %d keys has too many chunks to merge",
-                 a.max_kv_len);
   attn_decode_merge_kernel<<<dim3(a.T, a.Hq), kMergeThreads, merge_lds, stream>>>(a, n_chunks, chunk);
   NINFER_LAUNCH_CHECK();
   return 0;
