@@ -10,7 +10,6 @@ become exceptions here.
 """
 from __future__ import annotations
 
-from collections import Counter
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
@@ -20,7 +19,7 @@ from ..engine.runner import Chunk
 from ..engine.scheduler import Request, Scheduler
 from ..loading import load_model, random_model
 from ..sampling.params import SamplingParams
-from ..sampling.sampler import SampleRow, Sampler, fresh_seed
+from ..sampling.sampler import History, SampleRow, Sampler, fresh_seed
 
 
 class Session:
@@ -147,7 +146,7 @@ class Ninfer:
             self.runner.device)
         params = SamplingParams(temperature, top_k, top_p, repetition_penalty, seed, 1)
         self._sample_calls += 1
-        r = SampleRow(params, Counter(recent), 0, 0 if seed else self._sample_calls,
+        r = SampleRow(params, History(recent), 0, 0 if seed else self._sample_calls,
                       seed or fresh_seed())
         return self.sampler.sample(row, [r])[0]
 

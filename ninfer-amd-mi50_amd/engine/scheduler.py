@@ -23,13 +23,13 @@ one. A request that could not fit even alone is finished with an error.
 """
 from __future__ import annotations
 
-from collections import Counter, deque
+from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, Dict, List, Optional, Sequence, Tuple
 
 from ..cache.pages import OutOfPages
 from ..sampling.params import SamplingParams
-from ..sampling.sampler import SampleRow, fresh_seed
+from ..sampling.sampler import History, SampleRow, fresh_seed
 from .runner import Chunk
 
 
@@ -48,7 +48,7 @@ class Request:
     preemptions: int = 0
     seed: int = 0
     key: int = 0
-    history: Counter = field(default_factory=Counter)
+    history: History = field(default_factory=History)
 
     @property
     def tokens(self) -> List[int]:
@@ -105,7 +105,7 @@ class Scheduler:
         request.seed = request.params.seed if request.params.seed != 0 else fresh_seed()
         request.key = self._next_key
         self._next_key += 1
-        request.history = Counter(request.prompt)
+        request.history = History(request.prompt)
         request.status = "waiting"
         self.waiting.append(request)
 
@@ -232,7 +232,7 @@ class Scheduler:
                     done.append(req)
                     continue
                 req.output.append(tok)
-                req.history[tok] += 1
+                req.history.add(tok)
                 if len(req.output) >= req.params.max_new_tokens:
                     self._finish(req)
                     done.append(req)

@@ -11,9 +11,9 @@ the request gets a seed from the operating system when it is added.
 from __future__ import annotations
 
 import os
-from collections import Counter
-from typing import List, Sequence
+from typing import Dict, Iterable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from .params import SamplingParams
@@ -38,12 +38,58 @@ def fresh_seed() -> int:
     return int.from_bytes(os.urandom(8), "little") | 1
 
 
+class History:
+    """How often a request has seen each token (prompt + generated), for the
+    repetition penalty. Kept as two growing arrays (distinct tokens, counts), so
+    that a step hands them to the device as they are: the work per generated
+    token does not grow with the length of the history."""
+
+    def __init__(self, tokens: Iterable[int] = ()):
+        toks, counts = np.unique(np.asarray(list(tokens), dtype=np.int64), return_counts=True)
+        n = int(toks.shape[0])
+        cap = max(64, 2 * n)
+        self._tok = np.zeros(cap, np.int32)
+        self._cnt = np.zeros(cap, np.int32)
+        self._tok[:n] = toks
+        self._cnt[:n] = counts
+        self._n = n
+        self._where: Optional[Dict[int, int]] = None   # token -> index, made at the first add
+
+    def add(self, token: int) -> None:
+        if self._where is None:
+            self._where = {int(t): i for i, t in enumerate(self._tok[:self._n])}
+        i = self._where.get(token)
+        if i is not None:
+            self._cnt[i] += 1
+            return
+        if self._n == self._tok.shape[0]:
+            self._tok = np.concatenate([self._tok, np.zeros_like(self._tok)])
+            self._cnt = np.concatenate([self._cnt, np.zeros_like(self._cnt)])
+        self._tok[self._n] = token
+        self._cnt[self._n] = 1
+        self._where[token] = self._n
+        self._n += 1
+
+    def arrays(self) -> Tuple[np.ndarray, np.ndarray]:
+        """(distinct tokens, their counts), int32 views of equal length."""
+        return self._tok[:self._n], self._cnt[:self._n]
+
+    def count(self, token: int) -> int:
+        toks, cnts = self.arrays()
+        hit = np.nonzero(toks == token)[0]
+        return int(cnts[hit[0]]) if hit.size else 0
+
+    def __len__(self) -> int:
+        return self._n
+
+
 class SampleRow:
     """What the sampler needs of one row: options, history counts, RNG stream."""
 
-    def __init__(self, params: SamplingParams, history: Counter, key: int, draw: int, seed: int):
+    def __init__(self, params: SamplingParams, history: History, key: int, draw: int, seed: int):
         self.params = params
-        self.history = history
+        self.history = history if isinstance(history, History) else History(
+            t for t, c in dict(history).items() for _ in range(c))
         self.key = key
         self.draw = draw
         self.seed = seed
@@ -63,21 +109,26 @@ class Sampler:
         top_p = [row.params.top_p for row in rows]
         rp = [row.params.repetition_penalty for row in rows]
         u = [uniform(row.seed, row.key, row.draw) for row in rows]
-        pen_t: List[int] = []
-        pen_c: List[int] = []
+        pen_t: List[np.ndarray] = []
+        pen_c: List[np.ndarray] = []
         pen_o = [0]
         for row in rows:
+            n = 0
             if row.params.repetition_penalty != 1.0:
-                for tok, cnt in row.history.items():
-                    pen_t.append(tok)
-                    pen_c.append(cnt)
-            pen_o.append(len(pen_t))
+                toks, cnts = row.history.arrays()
+                pen_t.append(toks)
+                pen_c.append(cnts)
+                n = toks.shape[0]
+            pen_o.append(pen_o[-1] + n)
         dev = self.device
         f32 = lambda v: torch.tensor(v, dtype=torch.float32, device=dev)
         i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
         out = torch.empty(r, dtype=torch.int32, device=dev)
-        pen = dict(pen_tokens=i32(pen_t), pen_counts=i32(pen_c), pen_offsets=i32(pen_o)) \
-            if pen_t else {}
+        pen = {}
+        if pen_o[-1] > 0:
+            pen = dict(pen_tokens=torch.from_numpy(np.concatenate(pen_t)).to(dev),
+                       pen_counts=torch.from_numpy(np.concatenate(pen_c)).to(dev),
+                       pen_offsets=i32(pen_o))
         self.ops.sample(logits, f32(temp), f32(u), out, top_k=i32(top_k), top_p=f32(top_p),
                         rep_penalty=f32(rp), **pen)
         return out.tolist()

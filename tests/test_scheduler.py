@@ -172,3 +172,21 @@ def test_next_tokens_spans_prompt_and_output():
         for n in range(1, 8 - cached):
             r.cached = cached
             assert r.next_tokens(n) == r.tokens[cached:cached + n]
+
+
+def test_history_counts_like_a_counter():
+    """The sampler's history (distinct tokens and counts as growing arrays) against
+    collections.Counter, from a prompt and from nothing, beyond its first capacity."""
+    import random
+    from collections import Counter
+    from ninfer_amd.sampling.sampler import History
+    rng = random.Random(3)
+    toks = [rng.randrange(400) for _ in range(1500)]
+    for start in (0, 100):
+        h = History(toks[:start])
+        for t in toks[start:]:
+            h.add(t)
+        a, n = h.arrays()
+        assert dict(zip(a.tolist(), n.tolist())) == dict(Counter(toks))
+        assert len(h) == len(set(toks)) and h.count(toks[0]) == Counter(toks)[toks[0]]
+        assert h.count(100000) == 0
