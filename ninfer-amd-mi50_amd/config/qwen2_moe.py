@@ -5,8 +5,8 @@ Keys and defaults the reference reads: src/models/config.cpp:12-43
 (`num_key_value_heads` defaults to the head count :21-23, `head_dim` to
 hidden/heads :25-27, `rope_theta` to 1e6 :29-30, `tie_word_embeddings` to
 false :31-32). The keys it does not read (shared expert size, `norm_topk_prob`,
-`decoder_sparse_step`, `mlp_only_layers`, the sliding-window keys) are read
-here because the architecture has them.
+`decoder_sparse_step`, `mlp_only_layers`, the sliding-window keys, `qkv_bias`)
+are read here because the architecture has them.
 """
 from __future__ import annotations
 
@@ -38,6 +38,7 @@ class Qwen2MoeConfig:
     use_sliding_window: bool = False
     sliding_window: Optional[int] = None
     max_window_layers: int = 0
+    qkv_bias: bool = True
     eos_token_id: Optional[int] = None
     architecture: str = "Qwen2MoeForCausalLM"
 
@@ -81,11 +82,26 @@ class Qwen2MoeConfig:
         eps = r.need_float("rms_norm_eps")
         if not eps > 0:
             raise ConfigError(f"config.json: key 'rms_norm_eps' must be > 0, got {eps}")
-        theta = r.opt_float("rope_theta", 1e6)
+        # the rotation's base stands at the top level or inside 'rope_parameters'; of the
+        # scaling kinds only the plain one ("default": none) is built
+        rope = {}
+        for key in ("rope_scaling", "rope_parameters"):
+            sub = r.opt_raw(key)
+            if sub is None:
+                continue
+            if not isinstance(sub, dict):
+                raise ConfigError(f"config.json: key '{key}' must be an object or null")
+            kind = sub.get("rope_type", sub.get("type", "default"))
+            if kind != "default":
+                raise ConfigError(f"config.json: key '{key}' asks for rope scaling of type "
+                                  f"{kind!r}; only 'default' (none) is supported")
+            rope.update(sub)
+        if "rope_theta" in raw and raw["rope_theta"] is not None:
+            theta = r.opt_float("rope_theta", 1e6)
+        else:
+            theta = KeyReader(rope, "config.json: rope_parameters").opt_float("rope_theta", 1e6)
         if not theta > 0:
             raise ConfigError(f"config.json: key 'rope_theta' must be > 0, got {theta}")
-        if r.opt_raw("rope_scaling") is not None:
-            raise ConfigError("config.json: key 'rope_scaling' is not supported (must be null)")
         act = r.opt_str("hidden_act", "silu")
         if act != "silu":
             raise ConfigError(f"config.json: key 'hidden_act' must be 'silu', got {act!r}")
@@ -124,4 +140,5 @@ class Qwen2MoeConfig:
             norm_topk_prob=r.opt_bool("norm_topk_prob", False),
             decoder_sparse_step=sparse_step, mlp_only_layers=mlp_only,
             use_sliding_window=use_win, sliding_window=window,
-            max_window_layers=max_win_layers, eos_token_id=eos)
+            max_window_layers=max_win_layers, qkv_bias=r.opt_bool("qkv_bias", True),
+            eos_token_id=eos)

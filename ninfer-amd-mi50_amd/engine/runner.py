@@ -50,7 +50,7 @@ class ModelRunner:
             from ..kernels import load_ops
             ops = load_ops()
         self.ops = ops
-        check_tensors(source.shapes(), spec.tensor_specs(), where)
+        check_tensors(source.shapes(), spec.tensor_specs(), where, spec.unused_tensor_specs())
         spec.bind(WeightBinder(source, self.device, self.act_dtype))
 
         # one cache instance per plan entry that writes keys and values

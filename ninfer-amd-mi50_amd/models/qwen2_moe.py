@@ -1,6 +1,6 @@
 """Qwen2-MoE put together from parts, layer by layer from its configuration.
 
-Per layer: RMSNorm -> attention (q/k/v bias, rotary, window on layers >=
+Per layer: RMSNorm -> attention (q/k/v bias unless `qkv_bias` is false, rotary, window on layers >=
 max_window_layers when use_sliding_window) -> RMSNorm -> feed-forward, which
 is sparse (router, routed experts, gated shared expert) or a dense SwiGLU of
 `intermediate_size` according to `mlp_only_layers` and `decoder_sparse_step`.
@@ -29,7 +29,7 @@ def build_qwen2_moe(cfg: Qwen2MoeConfig) -> ModelSpec:
     for l in range(cfg.num_hidden_layers):
         p = f"model.layers.{l}."
         mixer = Attention(p + "self_attn.", h, cfg.num_attention_heads, cfg.num_key_value_heads,
-                          cfg.head_dim, rotary, qkv_bias=True, window=cfg.layer_window(l))
+                          cfg.head_dim, rotary, qkv_bias=cfg.qkv_bias, window=cfg.layer_window(l))
         if cfg.layer_is_sparse(l):
             ff = SparseMoE(p + "mlp.", h, cfg.num_experts, cfg.num_experts_per_tok,
                            cfg.moe_intermediate_size, cfg.norm_topk_prob,

@@ -63,6 +63,12 @@ class ModelSpec:
             out.update(p.all_tensor_specs())
         return out
 
+    def unused_tensor_specs(self) -> Dict[str, TensorSpec]:
+        out: Dict[str, TensorSpec] = {}
+        for p in self.parts():
+            out.update(p.all_unused_tensor_specs())
+        return out
+
     def bind(self, w: WeightBinder) -> None:
         for p in self.parts():
             p.bind_all(w)

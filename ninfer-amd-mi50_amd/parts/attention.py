@@ -64,6 +64,12 @@ class Attention(Mixer):
             specs[p + "v_proj.bias"] = TensorSpec((self.kv_heads * d,), "bias")
         return specs
 
+    def unused_tensor_specs(self) -> Dict[str, TensorSpec]:
+        # older checkpoints store the rotation's frequency table, which is computed here
+        if self.position.rot_dim > 0:
+            return {self.prefix + "rotary_emb.inv_freq": TensorSpec((self.position.rot_dim // 2,))}
+        return {}
+
     def bind(self, w: WeightBinder) -> None:
         p, d = self.prefix, self.head_dim
         nq, nk = self.heads * d, self.kv_heads * d

@@ -133,6 +133,12 @@ class Part:
         """Full checkpoint names this part needs -> expected shape and role."""
         return {}
 
+    def unused_tensor_specs(self) -> Dict[str, TensorSpec]:
+        """Checkpoint names that may be there and that this part does not read
+        (a copy of a tied table, a stored table of constants): present with the
+        shape given they are passed over, absent they are not missed."""
+        return {}
+
     def bind(self, w: WeightBinder) -> None:
         """Read this part's tensors (fusing or stacking them as its kernels
         want them)."""
@@ -144,6 +150,12 @@ class Part:
         out = dict(self.tensor_specs())
         for c in self.children():
             out.update(c.all_tensor_specs())
+        return out
+
+    def all_unused_tensor_specs(self) -> Dict[str, TensorSpec]:
+        out = dict(self.unused_tensor_specs())
+        for c in self.children():
+            out.update(c.all_unused_tensor_specs())
         return out
 
     def bind_all(self, w: WeightBinder) -> None:

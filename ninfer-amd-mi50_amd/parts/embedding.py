@@ -49,6 +49,12 @@ class LMHead(Part):
             return {}
         return {self.prefix + "weight": TensorSpec((self.vocab, self.hidden))}
 
+    def unused_tensor_specs(self) -> Dict[str, TensorSpec]:
+        # a checkpoint of a tied model may still carry the head: a copy of the table
+        if self.tied_to is not None:
+            return {self.prefix + "weight": TensorSpec((self.vocab, self.hidden))}
+        return {}
+
     def bind(self, w: WeightBinder) -> None:
         if self.tied_to is None:
             self.weight = w.matrix(self.prefix + "weight")

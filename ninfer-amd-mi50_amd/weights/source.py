@@ -11,7 +11,7 @@ import hashlib
 import json
 import os
 from dataclasses import dataclass
-from typing import Dict, List, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import torch
 
@@ -110,14 +110,17 @@ class RandomSource:
 
 
 def check_tensors(have: Dict[str, Tuple[int, ...]], want: Dict[str, TensorSpec],
-                  where: str) -> None:
+                  where: str, unused: Optional[Dict[str, TensorSpec]] = None) -> None:
     """One error that lists every missing tensor, every unexpected tensor and
     every tensor of the wrong shape (the reference stops at the first missing
-    name, src/models/model.hip:115-119, and checks no shapes)."""
+    name, src/models/model.hip:115-119, and checks no shapes). Names in
+    `unused` may be there or not; if there, their shape is checked too."""
+    known = dict(unused or {})
+    known.update(want)
     missing = sorted(n for n in want if n not in have)
-    unexpected = sorted(n for n in have if n not in want)
-    wrong = sorted((n, tuple(have[n]), tuple(want[n].shape)) for n in want
-                   if n in have and tuple(have[n]) != tuple(want[n].shape))
+    unexpected = sorted(n for n in have if n not in known)
+    wrong = sorted((n, tuple(have[n]), tuple(known[n].shape)) for n in known
+                   if n in have and tuple(have[n]) != tuple(known[n].shape))
     if not (missing or unexpected or wrong):
         return
     lines = [f"{where}: checkpoint does not match the model"]

@@ -110,12 +110,17 @@ def attention_qkv(x: Tensor, w: Dict[str, Tensor], prefix: str, n_heads: int, n_
     """q, k, v = x W^T + b, split into heads, q and k rotated.
 
     Weights: reference src/models/model.hip:530-532; the biases are this
-    architecture's (the reference loads none).
+    architecture's (the reference loads none) and are added where the weights
+    hold them (a model with `qkv_bias` false has none).
     """
     t = x.shape[0]
-    q = x @ w[prefix + "q_proj.weight"].float().T + w[prefix + "q_proj.bias"].float()
-    k = x @ w[prefix + "k_proj.weight"].float().T + w[prefix + "k_proj.bias"].float()
-    v = x @ w[prefix + "v_proj.weight"].float().T + w[prefix + "v_proj.bias"].float()
+
+    def project(name: str) -> Tensor:
+        y = x @ w[prefix + name + ".weight"].float().T
+        b = w.get(prefix + name + ".bias")
+        return y if b is None else y + b.float()
+
+    q, k, v = project("q_proj"), project("k_proj"), project("v_proj")
     q = apply_rope(q.view(t, n_heads, head_dim), positions, theta)
     k = apply_rope(k.view(t, n_kv, head_dim), positions, theta)
     return q, k, v.view(t, n_kv, head_dim)

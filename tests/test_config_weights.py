@@ -55,6 +55,29 @@ def test_configuration_errors_name_the_key(change, word):
         Qwen2MoeConfig.from_dict(raw)
 
 
+def test_rope_keys_and_qkv_bias():
+    """The rotation's base may stand inside 'rope_parameters'; scaling of the plain kind is
+    no scaling; another kind is refused. Without `qkv_bias` the model asks for no biases."""
+    from ninfer_amd import ConfigError, Qwen2MoeConfig
+    from ninfer_amd.loading import build_spec
+    raw = dict(CONFIG_A)
+    del raw["rope_theta"]
+    raw["rope_parameters"] = {"rope_type": "default", "rope_theta": 12345.0}
+    assert Qwen2MoeConfig.from_dict(raw).rope_theta == 12345.0
+    raw = dict(CONFIG_A, rope_scaling={"type": "default"})
+    assert Qwen2MoeConfig.from_dict(raw).rope_theta == CONFIG_A["rope_theta"]
+    with pytest.raises(ConfigError, match="rope_parameters"):
+        Qwen2MoeConfig.from_dict(dict(CONFIG_A, rope_parameters={"rope_type": "linear", "factor": 2.0}))
+    with pytest.raises(ConfigError, match="qkv_bias"):
+        Qwen2MoeConfig.from_dict(dict(CONFIG_A, qkv_bias=1))
+    assert Qwen2MoeConfig.from_dict(CONFIG_A).qkv_bias is True
+    _, with_bias = build_spec(CONFIG_A)
+    _, without = build_spec(dict(CONFIG_A, qkv_bias=False))
+    dropped = set(with_bias.tensor_specs()) - set(without.tensor_specs())
+    assert len(dropped) == 3 * CONFIG_A["num_hidden_layers"]
+    assert all(n.endswith("_proj.bias") for n in dropped)
+
+
 def test_registry_resolves_by_architecture_name():
     import ninfer_amd
     from ninfer_amd.loading import build_spec
@@ -148,6 +171,38 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(model_dirs, tmp_pat
     assert "unexpected tensors (1)" in msg and "model.layers.0.extra.weight" in msg
     assert "wrong shapes (2)" in msg and "has [65], expected [64]" in msg
     assert "has [64, 4], expected [4, 64]" in msg
+
+
+def test_tensors_a_checkpoint_may_hold_unread(model_dirs, tmp_path):
+    """A tied model's checkpoint may carry a copy of the head, an older one the rotation's
+    frequency tables: passed over when their shapes are right, reported when not."""
+    from ninfer_amd.loading import build_spec
+    from ninfer_amd.weights import CheckpointSource, WeightError, check_tensors
+    cfg, spec = build_spec(CONFIG_B)
+    half = CONFIG_B["head_dim"] // 2
+
+    def edit(t):
+        t["lm_head.weight"] = t["model.embed_tokens.weight"].clone()
+        t["model.layers.1.self_attn.rotary_emb.inv_freq"] = torch.zeros(half)
+
+    d = str(tmp_path / "extra")
+    _rewrite(model_dirs["B"]["float32"], d, edit)
+    check_tensors(CheckpointSource(d).shapes(), spec.tensor_specs(), d, spec.unused_tensor_specs())
+    with pytest.raises(WeightError, match="unexpected tensors \\(2\\)"):
+        check_tensors(CheckpointSource(d).shapes(), spec.tensor_specs(), d)
+
+    def edit_wrong(t):
+        t["lm_head.weight"] = torch.zeros(3, CONFIG_B["hidden_size"])
+
+    d2 = str(tmp_path / "extra_wrong")
+    _rewrite(model_dirs["B"]["float32"], d2, edit_wrong)
+    with pytest.raises(WeightError, match="wrong shapes \\(1\\)"):
+        check_tensors(CheckpointSource(d2).shapes(), spec.tensor_specs(), d2,
+                      spec.unused_tensor_specs())
+    # an untied model reads its head: nothing of it is passed over
+    _, untied = build_spec(CONFIG_A)
+    assert "lm_head.weight" in untied.tensor_specs()
+    assert "lm_head.weight" not in untied.unused_tensor_specs()
 
 
 def test_file_level_errors(tmp_path):

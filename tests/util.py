@@ -254,5 +254,5 @@ def random_config(seed: int) -> dict:
         "rope_theta": rng.choice([10000.0, 1000000.0]), "use_sliding_window": window is not None,
         "sliding_window": window or 4096, "max_window_layers": rng.randint(0, layers),
         "rms_norm_eps": rng.choice([1e-6, 1e-5]), "tie_word_embeddings": rng.random() < 0.5,
-        "hidden_act": "silu",
+        "hidden_act": "silu", "qkv_bias": rng.random() < 0.75,
     }
