@@ -31,6 +31,11 @@ struct GemmArgs {
   int out_dtype;         // of C
   int epilogue;
   int big_rows;          // rows of a big grouped tile: 64, 128 or 256 (0: 64)
+  int k_parts;           // the K range is cut into this many parts, one per blockIdx.z, part z
+                         // writing its sums to C + z * M * ldc (0 or 1: no cut); set by
+                         // gemm_split, not by callers
+  float* workspace;      // 32-bit scratch for a product cut along K, or null
+  int64_t workspace_floats;
 };
 
 // Which rows does tile `ti` of the grouped enumeration cover? Tiles of
@@ -96,5 +101,9 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream);
 bool gemm_tile_takes(const GemmArgs& a);
 int gemm_tile(const GemmArgs& a, hipStream_t stream);
 int gemm_generic(const GemmArgs& a, hipStream_t stream);
+// Dense products of 33 to 128 rows whose output tiles are too few to fill the GPU: cut
+// along K over more blocks, partial sums in the workspace, then added up in a fixed order.
+int gemm_split_parts(const GemmArgs& a);   // parts the product would be cut into (< 2: not cut)
+int gemm_split(const GemmArgs& a, hipStream_t stream);
 
 }  // namespace ninfer

@@ -16,10 +16,17 @@ extern "C" int ninfer_gemm(const GemmArgs* args, int force_generic, hipStream_t 
   if (rc) return rc;
   const GemmArgs& a = *args;
   if (!force_generic) {
+    if (gemm_split_parts(a) >= 2) return gemm_split(a, stream);
     if (many_rows(a) && gemm_tile_takes(a)) return gemm_tile(a, stream);
     if (gemm_skinny_takes(a)) return gemm_skinny(a, stream);
   }
   return gemm_generic(a, stream);
+}
+
+// Into how many parts along K ninfer_gemm would cut this product (< 2: it would not).
+extern "C" int ninfer_gemm_split_parts(const GemmArgs* args) {
+  if (gemm_check(*args)) return 0;
+  return gemm_split_parts(*args);
 }
 
 // Two products that do not depend on each other. Pairs of few-row products that have a

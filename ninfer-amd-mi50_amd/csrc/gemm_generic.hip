@@ -145,6 +145,9 @@ int gemm_check(const GemmArgs& a) {
   NINFER_REQUIRE(a.epilogue == kEpilogueNone || a.epilogue == kEpilogueSwiGLU,
                  "gemm: unknown epilogue %d", a.epilogue);
   NINFER_REQUIRE(!(a.epilogue == kEpilogueSwiGLU && a.bias), "gemm: SwiGLU epilogue takes no bias");
+  NINFER_REQUIRE(a.k_parts <= 1, "gemm: k_parts is set by the library, not by callers");
+  NINFER_REQUIRE(!a.workspace || a.workspace_floats > 0, "gemm: a workspace of %ld floats",
+                 (long)a.workspace_floats);
   return 0;
 }
 

@@ -54,6 +54,15 @@ __global__ __launch_bounds__(NW * 64, OCC) void gemm_tile_kernel(GemmArgs a) {
   const int wm = wave % WGM, wn = wave / WGM;
   const int K = a.K, N = a.N;
   const bf16* W = (const bf16*)a.W + (int64_t)group * a.w_group_stride;
+  // a product cut along K: this block's k tiles are kt_first .. kt_first + nk - 1, and its
+  // sums go to part blockIdx.z of C
+  int nk = K / TK, kt_first = 0;
+  if (a.k_parts > 1) {
+    const int per = (nk + a.k_parts - 1) / a.k_parts;
+    kt_first = blockIdx.z * per;
+    nk = min(per, nk - kt_first);
+    a.C = (TC*)a.C + (int64_t)blockIdx.z * a.M * a.ldc;
+  }
   constexpr int OUT_PER_BLOCK = SWIGLU ? TN / 2 : TN;
   constexpr int OUT_PER_WAVE = OUT_PER_BLOCK / WGM;
   const int out0 = by * OUT_PER_BLOCK;
@@ -69,12 +78,12 @@ __global__ __launch_bounds__(NW * 64, OCC) void gemm_tile_kernel(GemmArgs a) {
     // rows beyond the tile's last read its first row: their results are never stored
     int rr = r < rows_here ? row0 + r : row0;
     int64_t ar = a.a_index ? a.a_index[rr] / a.a_div : rr;
-    xsrc[i] = (const bf16*)a.A + ar * a.lda + 8 * kv;
+    xsrc[i] = (const bf16*)a.A + ar * a.lda + 8 * kv + kt_first * TK;
   }
 #pragma unroll
   for (int i = 0; i < WV; ++i) {
     int v = tid + i * NT, r = v / VPR, kv = v % VPR;
-    wsrc[i] = W + (int64_t)staged_w_row<TN, WGM, SWIGLU>(r, out0, N) * K + 8 * kv;
+    wsrc[i] = W + (int64_t)staged_w_row<TN, WGM, SWIGLU>(r, out0, N) * K + 8 * kv + kt_first * TK;
   }
   // P register stages: the loads of k tile t + P are issued while tile t is multiplied
   bf16x8 xreg[P][XV], wreg[P][WV];
@@ -111,7 +120,6 @@ __global__ __launch_bounds__(NW * 64, OCC) void gemm_tile_kernel(GemmArgs a) {
   const int tok0 = wn * COL;
 
   const int lr = lane & 31, lk = lane >> 5;
-  const int nk = K / TK;
   // products of one k tile from LDS buffer `buf`; NJ token blocks are live (a
   // compile-time count, so the loop body is straight-line code)
   auto multiply = [&](int buf, auto nj_tag) {
@@ -199,6 +207,7 @@ bool gemm_tile_takes(const GemmArgs& a) {
 }
 
 static int g_tile_variant = 0;   // tests: 0 = choose by shape
+static int64_t g_split_min_bytes = 48 << 20;   // tests lower it to cut small products too
 
 template <int TM, int TN, int TK, int NW, int WGM, int P, int OCC = 2>
 static int launch_tile(const GemmArgs& a, hipStream_t stream) {
@@ -207,7 +216,7 @@ static int launch_tile(const GemmArgs& a, hipStream_t stream) {
   const bool swiglu = a.epilogue == kEpilogueSwiGLU;
   const int m_tiles = (a.M + TM - 1) / TM + (a.offsets ? a.groups : 0);
   const int per_block = swiglu ? TN / 2 : TN;
-  const dim3 grid(m_tiles, (a.N + per_block - 1) / per_block);
+  const dim3 grid(m_tiles, (a.N + per_block - 1) / per_block, a.k_parts > 1 ? a.k_parts : 1);
   const size_t lds = 2 * (TM + TN) * (TK + 8) * sizeof(bf16);
 #define NINFER_TILE_LAUNCH(SW, TYPE)                                                        \
   do {                                                                                      \
@@ -251,6 +260,69 @@ int gemm_tile(const GemmArgs& a, hipStream_t stream) {
   return launch_tile<64, 128, 64, 4, 2, 2>(a, stream);
 }
 
+// out[m][n] = sum over the parts, in their order, of ws[z][m][n] (+ bias[n]); four features a thread.
+template <typename TC>
+__global__ void sum_parts_kernel(const float* __restrict__ ws, int parts, int M, int N,
+                                 const float* __restrict__ bias, TC* __restrict__ out, int ldc) {
+  const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // quad of features
+  const int quads = N / 4;
+  if (q >= (int64_t)M * quads) return;
+  const int m = q / quads, n = 4 * (q % quads);
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int z = 0; z < parts; ++z) {
+    const float4 v = *(const float4*)(ws + ((int64_t)z * M + m) * N + n);
+    s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+  }
+  if (bias) {
+    s.x += bias[n]; s.y += bias[n + 1]; s.z += bias[n + 2]; s.w += bias[n + 3];
+  }
+  const float v[4] = {s.x, s.y, s.z, s.w};
+  store_quad(out + (int64_t)m * ldc + n, v);
+}
+
+// The cut along K pays where 64 x 128 tiles of the output are fewer than the CUs, K is
+// long, and the weights are many enough (48 MB and more) that their stream outweighs the
+// second launch that adds the parts up (measured: 41 against 99 us for the library's product
+// at 64 rows, 3584 x 20480; no gain at 25 MB). Parts so that about two blocks per CU
+// exist, each with at least four k tiles, and no part is empty.
+int gemm_split_parts(const GemmArgs& a) {
+  if (a.offsets || a.epilogue != kEpilogueNone || !a.workspace || !gemm_tile_takes(a)) return 1;
+  if (a.M <= 32 || a.M > 128 || a.N % 4 || a.ldc % 4 || ((uintptr_t)a.C & 15)) return 1;
+  if ((int64_t)a.N * a.K * 2 < g_split_min_bytes) return 1;
+  const int cus = 256, tk = 64;
+  const int tiles = ((a.M + 63) / 64) * ((a.N + 127) / 128), nk = a.K / tk;
+  if (tiles >= cus) return 1;
+  const int64_t fit = a.workspace_floats / ((int64_t)a.M * a.N);
+  int parts = (int)min((int64_t)min(min(16, 2 * cus / tiles), nk / 4), fit);
+  if (parts < 2) return 1;
+  const int per = (nk + parts - 1) / parts;
+  return (nk + per - 1) / per;
+}
+
+int gemm_split(const GemmArgs& a, hipStream_t stream) {
+  const int parts = gemm_split_parts(a);
+  NINFER_REQUIRE(parts >= 2, "gemm: this product is not cut along K");
+  GemmArgs b = a;
+  b.C = a.workspace;
+  b.ldc = a.N;
+  b.out_dtype = kF32;
+  b.bias = nullptr;
+  b.k_parts = parts;
+  int rc = launch_tile<64, 128, 64, 4, 2, 2>(b, stream);
+  if (rc) return rc;
+  const int64_t quads = (int64_t)a.M * (a.N / 4);
+  const unsigned blocks = (unsigned)((quads + 255) / 256);
+  if (a.out_dtype == kF32)
+    sum_parts_kernel<float><<<blocks, 256, 0, stream>>>(a.workspace, parts, a.M, a.N, a.bias,
+                                                        (float*)a.C, a.ldc);
+  else
+    sum_parts_kernel<bf16><<<blocks, 256, 0, stream>>>(a.workspace, parts, a.M, a.N, a.bias,
+                                                       (bf16*)a.C, a.ldc);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
 }  // namespace ninfer
 
 extern "C" void ninfer_set_tile_variant(int v) { ninfer::g_tile_variant = v; }
+extern "C" void ninfer_set_split_min_bytes(long long v) { ninfer::g_split_min_bytes = v; }

@@ -31,7 +31,9 @@ class _GemmArgs(ctypes.Structure):
                 ("M", ctypes.c_int), ("N", ctypes.c_int), ("K", ctypes.c_int),
                 ("lda", ctypes.c_int), ("ldc", ctypes.c_int), ("groups", ctypes.c_int),
                 ("a_div", ctypes.c_int), ("in_dtype", ctypes.c_int), ("out_dtype", ctypes.c_int),
-                ("epilogue", ctypes.c_int), ("big_rows", ctypes.c_int)]
+                ("epilogue", ctypes.c_int), ("big_rows", ctypes.c_int),
+                ("k_parts", ctypes.c_int), ("workspace", ctypes.c_void_p),
+                ("workspace_floats", ctypes.c_int64)]
 
 
 class _AttnArgs(ctypes.Structure):
@@ -103,7 +105,12 @@ class HipOps:
         self.force_generic = False  # tests: run the plain kernels whatever the shape
         self._held = None           # products held back inside `together()`
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
+        # ... a SwiGLU's gate/up product only beyond this many: up to here the tile kernel with
+        # the activation in its epilogue beats the library's product followed by a kernel for
+        # the activation (measured at 33, 64 and 128 rows: 70 against 98 us at 40960 x 3584)
+        self.library_min_rows_fused = 128
         self._attn_ws = None
+        self._split_ws = None   # 32 MB of 32-bit scratch for products cut along K, made at first use
 
     # ---- helpers ----------------------------------------------------------------
     def _stream(self) -> ctypes.c_void_p:
@@ -264,7 +271,7 @@ class HipOps:
 
     # ---- products ---------------------------------------------------------------
     def _gemm(self, a, w, c, *, n, k, m, bias=None, offsets=None, a_index=None, c_index=None,
-              a_div=1, groups=1, epilogue=0, w_group_stride=0, tiles=None):
+              a_div=1, groups=1, epilogue=0, w_group_stride=0, tiles=None, only_if_split=False):
         t16 = t64 = tc = None
         big = 0
         if tiles is not None and tiles.tiles16 is not None:
@@ -275,6 +282,17 @@ class HipOps:
                          _ptr(a_index), _ptr(c_index), t16, t64, tc, w_group_stride, m, n, k,
                          a.shape[1],
                          c.shape[1], groups, a_div, _DT[a.dtype], _DT[c.dtype], epilogue, big)
+        if only_if_split:
+            # a dense product of few dozen rows: the library's unless the kernels here cut it
+            # along K (its output tiles alone would not fill the GPU)
+            if self._split_ws is None:
+                self._split_ws = torch.empty(1 << 23, dtype=torch.float32, device=a.device)
+            args.workspace = self._split_ws.data_ptr()
+            args.workspace_floats = self._split_ws.numel()
+            if self.lib.ninfer_gemm_split_parts(ctypes.byref(args)) < 2:
+                return False
+            self._ok(self.lib.ninfer_gemm(ctypes.byref(args), 0, self._stream()))
+            return True
         if self._held is not None:
             self._held.append((args, (a, w, c, bias, offsets, a_index, c_index, tiles)))
             return
@@ -314,7 +332,9 @@ class HipOps:
             _dev(bias, "bias", torch.float32, 1)
             _need(bias.shape[0] == w.shape[0], "linear: bias has the wrong size")
         if self._use_library(x, out) and bias is None:
-            torch.matmul(x, w.t(), out=out)
+            if x.shape[0] > self.library_min_rows_fused or not self._gemm(
+                    x, w, out, m=x.shape[0], n=w.shape[0], k=x.shape[1], only_if_split=True):
+                torch.matmul(x, w.t(), out=out)
             return
         self._gemm(x, w, out, m=x.shape[0], n=w.shape[0], k=x.shape[1], bias=bias)
 
@@ -342,7 +362,7 @@ class HipOps:
         inner = w_gate_up.shape[0] // 2
         _need(w_gate_up.shape == (2 * inner, x.shape[1]), "swiglu_linear: weight shape")
         _need(out.shape == (x.shape[0], inner), "swiglu_linear: out has the wrong shape")
-        if self._use_library(x, out):
+        if self._use_library(x, out) and x.shape[0] > self.library_min_rows_fused:
             gu = torch.empty((x.shape[0], 2 * inner), dtype=x.dtype, device=x.device)
             torch.matmul(x, w_gate_up.t(), out=gu)
             self.silu_mul(gu, out)

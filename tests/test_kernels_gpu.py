@@ -2,6 +2,7 @@
 and in bfloat16, at sizes other than the engine's tiny models: widths and
 vocabularies that are no power of two, odd row counts, experts without rows,
 contexts that end inside a page."""
+import ctypes
 import math
 from types import SimpleNamespace
 
@@ -141,6 +142,31 @@ def test_tile_product_every_tile_height(ops, gen, variant, m, n, k):
         close(h1, h2, torch.bfloat16, scale=k * 0.2)
     finally:
         ops.lib.ninfer_set_tile_variant(0)
+
+
+@pytest.mark.parametrize("m,n,k", [(33, 2048, 5632), (64, 3584, 20480), (100, 300, 512),
+                                   (128, 2048, 2048), (64, 136, 4096), (40, 6144, 1024)])
+def test_linear_cut_along_k(ops, gen, m, n, k):
+    """Dense bf16 products of 33 to 128 rows whose output tiles would not fill the GPU are cut
+    along K over more blocks and summed in a fixed order: against the plain product, the
+    same result twice, and (the sizes say so) cut indeed."""
+    x, w = rnd((m, k), torch.bfloat16, gen), rnd((n, k), torch.bfloat16, gen)
+    o1 = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
+    o2, o3 = torch.empty_like(o1), torch.empty_like(o1)
+    ops.lib.ninfer_set_split_min_bytes(ctypes.c_longlong(0))   # products of any size
+    try:
+        assert ops._gemm(x, w, o1, m=m, n=n, k=k, only_if_split=True), "not cut along K"
+        PlainOps().linear(x, w, o2)
+        close(o1, o2, torch.bfloat16, scale=math.sqrt(k))
+        if not ops.force_generic:   # (another test's fixture may have switched the fast kernels off)
+            ops.linear(x, w, o3)
+        else:
+            ops._gemm(x, w, o3, m=m, n=n, k=k, only_if_split=True)
+        assert torch.equal(o1, o3)
+    finally:
+        ops.lib.ninfer_set_split_min_bytes(ctypes.c_longlong(48 << 20))
+    if n * k * 2 < (48 << 20):   # by default only long weight streams are cut
+        assert not ops._gemm(x, w, o3, m=m, n=n, k=k, only_if_split=True)
 
 
 def test_linear_row_result_does_not_depend_on_batch(ops, gen):
