@@ -10,7 +10,9 @@ keys and values; token ids are seeded random). A step is one decode step: one
 new token for every request of the batch through the engine's step function
 (replayed from a captured HIP graph unless --no-graph) and its device sampler. One JSON line is printed: decoded tokens a second as
 `value`; the 2,048-token prefill under "prefill"; the decode step's memory
-roofline under "roofline"; decode at batch 1 and 64 under "points".
+roofline under "roofline"; decode at batch 1 and 64 under "points"; and under
+"graph_check" the largest difference between replayed and eager decode steps at
+those batches (untimed; 0.0 when the replays are exact).
 Peaks: HBM 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s (fp32 157.3 TFLOP/s).
 
     python bench.py --scenario long [--model 57b-a14b] [--requests 8] [--prompt 32768] [--new 256]
@@ -57,6 +59,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-check", action="store_true",
+                    help="skip the comparison of replayed with eager decode steps (untimed)")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
                     help="length of the timed prefill (the contract's figure is at 2,048)")
     ap.add_argument("--graph", dest="graph", action="store_true", default=True,
@@ -159,6 +163,37 @@ def main() -> int:
                              + 3 * Is * H + H) + L * 2 * Hq * D * T * T + 2 * V * H
         return dt, flops
 
+    def graph_check(batch: int) -> float:
+        """Replayed steps against the same steps launched kernel by kernel, at this batch (so
+        with the same library products inside the graph): `batch` requests with a real
+        64-token prompt each, then four decode steps of fixed tokens, once with replays and
+        once with the graphs forgotten before every step (the first step of a shape runs
+        eagerly, under the same context bound as its graph), with an eager step of another
+        shape between the replays. Largest difference of any logit (0.0: replays are exact)."""
+        prompts = [torch.randint(0, V, (64,), generator=gen).tolist() for _ in range(batch)]
+        feed = [torch.randint(0, V, (batch,), generator=gen).tolist() for _ in range(4)]
+        outs = []
+        for replay in (True, False):
+            runner._graphs.clear()
+            slots = [runner.open() for _ in range(batch)]
+            for i in range(0, batch, 16):
+                runner.step([Chunk(s, p, []) for s, p in zip(slots[i:i + 16], prompts[i:i + 16])])
+            got = []
+            for n, toks in enumerate(feed):
+                if not replay:
+                    runner._graphs.clear()
+                logits = runner.step([Chunk(s, [t], [0]) for s, t in zip(slots, toks)])
+                got.append(logits.float().clone())
+                if n == 1 and batch < max_b:
+                    extra = runner.open()
+                    runner.step([Chunk(extra, prompts[0][:9], [8])])
+                    runner.close(extra)
+            outs.append(got)
+            for s in slots:
+                runner.close(s)
+        runner._graphs.clear()
+        return max(float((a - b).abs().max()) for a, b in zip(*outs))
+
     dt, nbytes, n_exp = decode_run(args.batch, args.steps, args.warmup)
     result = {
         "metric": f"decode tok/s at batch {args.batch} ({model_name} shapes, context {ctx})",
@@ -190,6 +225,13 @@ def main() -> int:
             d, _, _ = decode_run(b, steps, max(2, args.warmup // 2))
             points[f"decode_b{b}"] = round(b / d, 2)
         result["points"] = points
+    if args.graph and not args.no_check:
+        batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+        worst = max(graph_check(b) for b in batches)
+        result["graph_check"] = {"batches": batches, "max_abs_diff": worst}
+        if worst != 0.0:
+            print(f"[bench] WARNING: replayed steps differ from eager steps by {worst}",
+                  file=sys.stderr, flush=True)
     print(json.dumps(result), flush=True)
     return 0
 

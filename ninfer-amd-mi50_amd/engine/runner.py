@@ -194,16 +194,16 @@ class ModelRunner:
                                  "meta": torch.empty(host.numel(), dtype=torch.int32,
                                                      device=self.device), "graph": None}
             entry = self._graphs[key]
+            entry["copied"] = torch.cuda.Event()
             entry["pinned"].copy_(host)
             entry["meta"].copy_(entry["pinned"], non_blocking=True)
+            entry["copied"].record()
             return self._forward(entry["meta"], shape)
-        # the pinned staging buffer is reused: wait until the last copy from it is done
-        if entry.get("copied") is not None:
-            entry["copied"].synchronize()
+        # the pinned staging buffer is reused: wait until the last copy from it is done (a
+        # caller that does not read the logits of a step back runs ahead of the device)
+        entry["copied"].synchronize()
         entry["pinned"].copy_(host)
         entry["meta"].copy_(entry["pinned"], non_blocking=True)
-        if entry.get("copied") is None:
-            entry["copied"] = torch.cuda.Event()
         entry["copied"].record()
         if entry["graph"] is None:
             torch.cuda.synchronize()

@@ -140,6 +140,34 @@ def test_graph_replay_equals_eager(case, dtype):
         assert torch.equal(a, b)
 
 
+def test_graph_steps_of_a_caller_that_runs_ahead(model_dirs):
+    """A caller that reads no logits back between steps runs ahead of the device: the second
+    step of a shape must not refill the staging buffer before the first step's copy from it
+    has run (work is queued in front so that the device lags)."""
+    from ninfer_amd import Chunk, EngineOptions, load_model
+    d = model_dirs["C"]["bfloat16"]
+    vocab = TINY["C"][0]["vocab_size"]
+    prompts = [util.random_tokens(9 + i, vocab, 50 + i) for i in range(3)]
+    feed = [util.random_tokens(3, vocab, 70 + i) for i in range(4)]
+    outs = []
+    for use_graph in (False, True):
+        runner = load_model(d, EngineOptions(dtype="bfloat16", max_context=64, num_sequences=4,
+                                             page_size=8, use_graph=use_graph))
+        slots = [runner.open() for _ in prompts]
+        runner.step([Chunk(s, p, []) for s, p in zip(slots, prompts)])
+        torch.cuda.synchronize()
+        busy = torch.randn(4096, 4096, device="cuda")
+        for _ in range(40):          # tens of milliseconds of queued work
+            busy = busy @ busy * 1e-3
+        got = [runner.step([Chunk(s, [t], [0]) for s, t in zip(slots, toks)]) for toks in feed[:2]]
+        got = [g.clone() for g in got[-1:]]          # (a graph's logits live until the next step)
+        for toks in feed[2:]:
+            got.append(runner.step([Chunk(s, [t], [0]) for s, t in zip(slots, toks)]).clone())
+        outs.append([g.float().cpu() for g in got])
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+
+
 def test_graph_replay_with_many_requests(model_dirs):
     """40 requests decode together: dense products of more than 32 rows go to the
     vendor library, also inside the captured graph. Every replay must equal the
