@@ -110,6 +110,7 @@ class HipOps:
         # the activation (measured at 33, 64 and 128 rows: 70 against 98 us at 40960 x 3584)
         self.library_min_rows_fused = 128
         self._attn_ws = None
+        self._outgrown = []     # workspaces that captured graphs may still point to
         self._split_ws = None   # 32 MB of 32-bit scratch for products cut along K, made at first use
 
     # ---- helpers ----------------------------------------------------------------
@@ -485,7 +486,15 @@ class HipOps:
             ws_floats = int(self.lib.ninfer_attention_workspace_floats(
                 t if ctx.max_qlen == 1 else single, n_q, head_dim, ctx.max_kv_len))
             if self._attn_ws is None or self._attn_ws.numel() < ws_floats:
+                # A captured graph may hold the address of the workspace it was recorded
+                # with: an outgrown one is kept, never given back (a replay would write
+                # into whatever took its place), and growth at least doubles, which bounds
+                # what is kept to the size of the largest.
+                if self._attn_ws is not None:
+                    self._outgrown.append(self._attn_ws)
+                    ws_floats = max(ws_floats, 2 * self._attn_ws.numel())
                 self._attn_ws = torch.empty(ws_floats, dtype=torch.float32, device=qkv.device)
+            ws_floats = self._attn_ws.numel()
             ws = self._attn_ws.data_ptr()
         args = _AttnArgs(
             qkv.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), out.data_ptr(),
