@@ -196,6 +196,55 @@ def test_graph_replay_with_many_requests(model_dirs):
         assert torch.equal(a, b)
 
 
+# Wide enough, with a prompt long enough, that the engine's steps run the kernels for many rows:
+# prompt attention on the matrix cores over hundreds of keys with a window that ends inside
+# them, grouped products in tiles of 256, 128 and 64 rows, dense products by the library.
+CONFIG_WIDE = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe",
+    "num_hidden_layers": 2, "hidden_size": 256, "num_attention_heads": 4,
+    "num_key_value_heads": 2, "head_dim": 64, "intermediate_size": 384,
+    "moe_intermediate_size": 192, "shared_expert_intermediate_size": 256,
+    "num_experts": 4, "num_experts_per_tok": 2, "norm_topk_prob": False,
+    "decoder_sparse_step": 1, "mlp_only_layers": [], "vocab_size": 512,
+    "rope_theta": 10000.0, "use_sliding_window": True, "sliding_window": 300,
+    "max_window_layers": 1, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
+    "hidden_act": "silu",
+}
+
+
+@pytest.fixture(scope="module")
+def wide_case(tmp_path_factory):
+    import ninfer_amd
+    dirs = {}
+    for dt in ("float32", "bfloat16"):
+        dirs[dt] = str(tmp_path_factory.mktemp(f"wide_{dt}"))
+        ninfer_amd.write_random_model(dirs[dt], CONFIG_WIDE, 77, dtype=dt, std=0.06)
+    rcfg, w16 = util.read_folder(dirs["bfloat16"])
+    return dirs, util.safe_prompt(w16, rcfg, 640, 5)
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_long_prompt_on_the_many_row_kernels(wide_case, dtype):
+    from ninfer_amd import EngineOptions, load_model
+    from ninfer_amd.parts.moe import big_tile_rows
+    cfg = CONFIG_WIDE
+    dirs, toks = wide_case
+    rcfg, w = util.read_folder(dirs[dtype])
+    ref = plain_model.forward(w, rcfg, toks)
+    k, e = cfg["num_experts_per_tok"], cfg["num_experts"]
+    assert {big_tile_rows(n * k, e) for n in (640, 200, 60)} == {256, 128, 64}
+    runner = load_model(dirs[dtype], EngineOptions(dtype=dtype, max_context=704, prefill_chunk=640,
+                                                   num_sequences=2, page_size=16))
+    whole = util.run_schedule(runner, util.schedule_whole("a", toks))["a"]
+    torch.testing.assert_close(whole, ref, **bound(dtype), msg=lambda m: f"whole: {m}")
+    cut = [("b", toks[:200], list(range(200))), ("b", toks[200:260], list(range(60))),
+           ("b", toks[260:], list(range(380)))]
+    steps = [([entry], ["b"] if i == len(cut) - 1 else []) for i, entry in enumerate(cut)]
+    parts = util.run_schedule(runner, steps)["b"]
+    torch.testing.assert_close(parts, ref, **bound(dtype), msg=lambda m: f"portions: {m}")
+    assert any(g.window_freed > 0 for g in runner.cache.groups)
+
+
 @pytest.mark.parametrize("seed", [0, 10, 16, 28, 35])
 def test_random_configurations(tmp_path, seed):
     """Configurations drawn at random (head sizes that only the plain kernels take, heads in
