@@ -243,6 +243,16 @@ def test_long_prompt_on_the_many_row_kernels(wide_case, dtype):
     parts = util.run_schedule(runner, steps)["b"]
     torch.testing.assert_close(parts, ref, **bound(dtype), msg=lambda m: f"portions: {m}")
     assert any(g.window_freed > 0 for g in runner.cache.groups)
+    # decoding over a context of several chunks of keys, two requests at different lengths
+    # in a step, from a replayed graph: the few-row kernels at this width
+    runner = load_model(dirs[dtype], EngineOptions(dtype=dtype, max_context=704, prefill_chunk=640,
+                                                   num_sequences=2, page_size=16, use_graph=True))
+    steps = [([("c", toks[:600], []), ("d", toks[:333], [])], [])]
+    steps += [([("c", [toks[600 + i]], [0]), ("d", [toks[333 + i]], [0])], []) for i in range(24)]
+    got = util.run_schedule(runner, steps)
+    torch.testing.assert_close(got["c"], ref[600:624], **bound(dtype), msg=lambda m: f"decode c: {m}")
+    torch.testing.assert_close(got["d"], ref[333:357], **bound(dtype), msg=lambda m: f"decode d: {m}")
+    assert any(e["graph"] is not None for e in runner._graphs.values())
 
 
 @pytest.mark.parametrize("seed", [0, 10, 16, 28, 35])
