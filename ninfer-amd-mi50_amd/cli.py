@@ -1,11 +1,15 @@
 """Command line in the reference's manner: `ninfer <model_dir> [options]`
 (src/apps/ninfer.cpp:55-119). Option names and meanings are the reference's
 where it has them: --max-context, --prefill-chunk, --max-new, --temperature
-(0 = greedy), --top-k, --top-p, --repeat-penalty, --seed (0 = not fixed),
+(0 = greedy), --top-k, --top-p, --repeat-penalty, --seed,
 --graph, --log-level. Prompts are token ids (there is no tokenizer here):
 --prompt-ids, --prompt-file, --random-prompts. Generated ids go to stdout, one
 line per request; diagnostics go to stderr (src/apps/ninfer.cpp:1-2). An
-unknown option is an error (:114-116).
+unknown option is an error (:114-116). Without a prompt it is the reference's
+interactive loop (:222-233): every line of standard input is a turn of token
+ids, the answer is generated from all turns and answers so far, until the
+input ends. A one-shot run with --seed 0 samples from the fixed seed 1234, as
+the reference's does (:205); the loop draws a seed per turn.
 """
 from __future__ import annotations
 
@@ -31,7 +35,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--top-k", type=int, default=50)
     ap.add_argument("--top-p", type=float, default=0.95)
     ap.add_argument("--repeat-penalty", type=float, default=1.05)
-    ap.add_argument("--seed", type=int, default=0, help="sampling seed (0 = not fixed)")
+    ap.add_argument("--seed", type=int, default=0, help="sampling seed (0: 1234 for a one-shot run, a fresh one per turn of the loop)")
     ap.add_argument("--graph", action="store_true", help="replay decode steps from a HIP graph")
     ap.add_argument("--log-level", choices=["debug", "info", "warn", "error"], default="info")
     ap.add_argument("--dtype", choices=["bf16", "fp32", "bfloat16", "float32"], default="bf16")
@@ -67,10 +71,6 @@ def main(argv: Optional[List[str]] = None) -> int:
         rng = random.Random(args.seed or 1234)
         for n in args.random_prompts.split(","):
             prompts.append([rng.randrange(raw["vocab_size"]) for _ in range(int(n))])
-    if not prompts:
-        print("ninfer: no prompt given (--prompt-ids, --prompt-file or --random-prompts)",
-              file=sys.stderr)
-        return 2
     t0 = time.time()
     common = dict(max_context=args.max_context, prefill_chunk=args.prefill_chunk,
                   num_sequences=args.max_seqs, dtype=dtype, page_size=args.page_size,
@@ -82,9 +82,11 @@ def main(argv: Optional[List[str]] = None) -> int:
             eng = Ninfer(args.model_dir, **common)
         log(f"engine ready in {time.time() - t0:.1f} s: vocab={eng.vocab} ctx={args.max_context} "
             f"chunk={args.prefill_chunk} seqs={args.max_seqs} dtype={dtype}")
-        params = SamplingParams(args.temperature, args.top_k, args.top_p, args.repeat_penalty,
-                                args.seed, args.max_new)
         stop = [args.eos_id] if args.eos_id is not None else None
+        if not prompts:
+            return _interactive(eng, args, stop)
+        params = SamplingParams(args.temperature, args.top_k, args.top_p, args.repeat_penalty,
+                                args.seed or 1234, args.max_new)
         t1 = time.time()
         outs = eng.generate(prompts, params, stop)
         dt = time.time() - t1
@@ -95,6 +97,26 @@ def main(argv: Optional[List[str]] = None) -> int:
     except Exception as e:  # the reference exits 1 with the message (src/apps/ninfer.cpp:234-237)
         print(f"ninfer: error: {e}", file=sys.stderr)
         return 1
+    return 0
+
+
+def _interactive(eng, args, stop) -> int:
+    """Turn after turn from standard input: a line of comma-separated token ids is added to
+    what has been said, the answer is generated from all of it and added too."""
+    from .sampling.params import SamplingParams
+    print("ninfer ready: one line of comma-separated token ids per turn, end of input to exit",
+          file=sys.stderr, flush=True)
+    said: List[int] = []
+    for line in sys.stdin:
+        ids = [int(x) for x in line.replace(",", " ").split()]
+        if not ids:
+            continue
+        said += ids
+        params = SamplingParams(args.temperature, args.top_k, args.top_p, args.repeat_penalty,
+                                args.seed, args.max_new)
+        answer = eng.generate([said], params, stop)[0]
+        print(",".join(map(str, answer)), flush=True)
+        said += answer
     return 0
 
 

@@ -88,6 +88,17 @@ def test_command_line(model_dirs):
     lines = proc.stdout.strip().splitlines()
     assert len(lines) == 3
     assert [int(x) for x in lines[0].split(",")] == plain_model.greedy_generate(w, cfg, prompt, 6)
+    # without a prompt: turns from standard input, each answered from everything said so far
+    second = util.random_tokens(4, cfg["vocab_size"], 4)
+    turns = ",".join(map(str, prompt)) + "\n\n" + " ".join(map(str, second)) + "\n"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "ninfer"), d, "--max-new", "5", "--temperature",
+         "0", "--dtype", "fp32", "--max-context", "64", "--eos-id", "-1", "--repeat-penalty", "1"],
+        input=turns, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    answers = [[int(x) for x in l.split(",")] for l in proc.stdout.strip().splitlines()]
+    first = plain_model.greedy_generate(w, cfg, prompt, 5)
+    assert answers == [first, plain_model.greedy_generate(w, cfg, prompt + first + second, 5)]
     bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "ninfer"), d, "--no-such-flag"],
                          capture_output=True, text=True, timeout=120)
     assert bad.returncode != 0
