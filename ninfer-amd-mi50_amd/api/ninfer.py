@@ -103,6 +103,11 @@ class Ninfer:
         return self.options.num_sequences
 
     @property
+    def devices(self) -> int:
+        """GPUs the engine runs on (reference tools/ninfer_ctypes.py:177): always one."""
+        return 1
+
+    @property
     def kv_bytes_per_token(self) -> int:
         return self.runner.cache.kv_bytes_per_token(2 if self.options.dtype == "bfloat16" else 4)
 
@@ -149,6 +154,12 @@ class Ninfer:
         r = SampleRow(params, History(recent), 0, 0 if seed else self._sample_calls,
                       seed or fresh_seed())
         return self.sampler.sample(row, [r])[0]
+
+    def close(self) -> None:
+        """Give the model and its cache back (reference tools/ninfer_ctypes.py:238-241);
+        the object cannot be used afterwards."""
+        self.runner = None
+        self.sampler = None
 
     # ---- generation -----------------------------------------------------------------
     def generate(self, prompts: Sequence[Sequence[int]], params: Optional[SamplingParams] = None,
