@@ -107,6 +107,46 @@ def test_32bit_does_not_depend_on_the_cut(case):
     assert torch.equal(a, b) and torch.equal(a, c)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_schedules_give_the_same_bits(model_dirs, seed):
+    """32-bit: schedules drawn at random (cuts, batches, order of entries, wanted rows), with a
+    random page size and a pool that just suffices, pages given back filled with NaN: every
+    wanted row equals the whole-sequence run of its request to the last bit."""
+    import random
+    from ninfer_amd import Chunk, EngineOptions, load_model
+    rng = random.Random(seed)
+    name = "ABC"[seed % 3]
+    d = model_dirs[name]["float32"]
+    vocab = TINY[name][0]["vocab_size"]
+    lens = [rng.randint(1, 120) for _ in range(rng.randint(2, 7))]
+    reqs = {f"r{i}": util.random_tokens(n, vocab, seed * 100 + i) for i, n in enumerate(lens)}
+    page, max_live = rng.choice([4, 8, 16, 32]), rng.randint(1, 4)
+    pages = sum(sorted((-(-n // page) for n in lens), reverse=True)[:max_live]) + rng.randint(0, 2)
+    whole = load_model(d, EngineOptions(dtype="float32", max_context=128, num_sequences=4,
+                                        page_size=16, num_pages=64))
+    ref = {r: util.run_schedule(whole, util.schedule_whole(r, t))[r] for r, t in reqs.items()}
+    runner = load_model(d, EngineOptions(dtype="float32", max_context=128, num_sequences=4,
+                                         page_size=page, num_pages=pages, poison_freed_pages=True,
+                                         use_graph=seed % 4 == 3))
+    slots, fed = {}, {r: 0 for r in reqs}
+    for entries, end in util.schedule_random(reqs, seed, max_live):
+        for r, _, _ in entries:
+            if r not in slots:
+                slots[r] = runner.open()
+        logits = runner.step([Chunk(slots[r], t, w) for r, t, w in entries])
+        o = 0
+        for r, t, w in entries:
+            for i in w:
+                assert torch.equal(logits[o].cpu(), ref[r][fed[r] + i]), \
+                    f"{name} seed {seed} page {page}: {r} at position {fed[r] + i}"
+                o += 1
+            fed[r] += len(t)
+        for r in end:
+            runner.close(slots.pop(r))
+    runner.cache.check()
+    assert all(g.allocator.in_use == 0 for g in runner.cache.groups)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_graph_replay_equals_eager(case, dtype):
     """Decode-only steps replayed from a HIP graph give the logits of the same

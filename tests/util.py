@@ -138,6 +138,36 @@ def schedule_mixed(requests: Dict[str, Sequence[int]], seed: int = 0, max_live: 
     return steps
 
 
+def schedule_random(requests: Dict[str, Sequence[int]], seed: int, max_live: int = 4) -> List[Step]:
+    """A schedule drawn at random: requests start in any order, up to `max_live` live; a live
+    request brings 1 to 64 tokens to a step or is left out of it; the entries of a step come
+    in any order; logits are wanted at a random subset of the rows."""
+    rng = random.Random(seed)
+    waiting = list(requests)
+    rng.shuffle(waiting)
+    live: Dict[str, int] = {}
+    steps: List[Step] = []
+    while waiting or live:
+        while waiting and len(live) < max_live and rng.random() < 0.6:
+            live[waiting.pop()] = 0
+        entries, end = [], []
+        for rid in list(live):
+            if rng.random() < 0.2 and len(live) > 1:
+                continue
+            toks, done = requests[rid], live[rid]
+            m = min(len(toks) - done, rng.choice([1, 1, 1, 2, 3, 4, 7, 16, 17, 33, 64]))
+            want = sorted(rng.sample(range(m), rng.randint(0, m)))
+            entries.append((rid, list(toks[done:done + m]), want))
+            live[rid] = done + m
+            if live[rid] == len(toks):
+                end.append(rid)
+                del live[rid]
+        if entries:
+            rng.shuffle(entries)
+            steps.append((entries, end))
+    return steps
+
+
 def run_schedule(runner, steps: List[Step]) -> Dict[str, torch.Tensor]:
     """Feed a schedule through a ModelRunner; returns id -> logits [n, vocab]
     (rows in position order) on the CPU."""
