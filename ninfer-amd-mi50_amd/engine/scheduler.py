@@ -23,6 +23,7 @@ one. A request that could not fit even alone is finished with an error.
 """
 from __future__ import annotations
 
+import hashlib
 from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, Dict, List, Optional, Sequence, Tuple
@@ -47,7 +48,8 @@ class Request:
     error: Optional[str] = None
     preemptions: int = 0
     seed: int = 0
-    key: int = 0
+    key: int = 0                    # of its stream of random numbers: from its id (see add)
+    order: int = 0                  # of its arrival at the scheduler
     history: History = field(default_factory=History)
 
     @property
@@ -103,7 +105,12 @@ class Scheduler:
             self.finished.append(request)
             return
         request.seed = request.params.seed if request.params.seed != 0 else fresh_seed()
-        request.key = self._next_key
+        # The stream of random numbers is named by (seed, id), not by the order of arrival:
+        # the same request draws the same tokens alone and in a crowd, and requests that
+        # share a seed still draw differently.
+        digest = hashlib.sha256(str(request.id).encode("utf-8")).digest()
+        request.key = int.from_bytes(digest[:8], "little")
+        request.order = self._next_key
         self._next_key += 1
         request.history = History(request.prompt)
         request.status = "waiting"
@@ -176,7 +183,7 @@ class Scheduler:
             chunks.append((req, n, n == left))
             budget -= n
         # preempted requests go back to the front, oldest first
-        for req in sorted(preempted, key=lambda r: -r.key):
+        for req in sorted(preempted, key=lambda r: -r.order):
             self.waiting.appendleft(req)
         # 3: admissions
         while self.waiting and budget > 0 and len(self.running) < self.max_seqs \

@@ -31,6 +31,58 @@ def test_greedy_generation_through_the_entry_point(model_dirs):
         assert eng.kv_pages()["free"] == eng.kv_pages()["total"]
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_a_crowd_under_a_tight_pool_generates_what_each_request_does_alone(model_dirs, seed):
+    """32-bit, requests drawn at random, greedy or at a temperature: through a scheduler with
+    few slots and a pool that just fits the largest request (so requests are preempted and
+    recomputed), every request gets the tokens it gets alone. Its random numbers are named by
+    its seed and id, not by its place in the queue."""
+    import random
+    from ninfer_amd import EngineOptions, Request, SamplingParams, Scheduler, load_model
+    from ninfer_amd.sampling import Sampler
+    rng = random.Random(seed)
+    name = "ABC"[seed % 3]
+    d = model_dirs[name]["float32"]
+    vocab = TINY[name][0]["vocab_size"]
+    n = rng.randint(3, 8)
+    prompts = [util.random_tokens(rng.randint(1, 60), vocab, seed * 50 + i) for i in range(n)]
+    news = [rng.randint(1, 24) for _ in range(n)]
+    temp = 0.8 if seed % 2 else 0.0
+
+    def requests():
+        return [Request(f"q{i}", list(p), SamplingParams(temperature=temp, top_k=0, top_p=1.0,
+                                                         repetition_penalty=1.0, seed=7 + i % 2,
+                                                         max_new_tokens=m), [])
+                for i, (p, m) in enumerate(zip(prompts, news))]
+
+    alone = load_model(d, EngineOptions(dtype="float32", max_context=96, num_sequences=1,
+                                        page_size=16, prefill_chunk=64))
+    sampler = Sampler(alone.ops, alone.device)
+    want = []
+    for r in reversed(requests()):        # one scheduler each, in another order
+        s = Scheduler(alone, sampler)
+        s.add(r)
+        s.run()
+        want.insert(0, r.output)
+    page = rng.choice([4, 8, 16])
+    pages = max(-(-(len(p) + m) // page) for p, m in zip(prompts, news)) + rng.randint(0, 4)
+    runner = load_model(d, EngineOptions(dtype="float32", max_context=96, num_sequences=3,
+                                         page_size=page, num_pages=pages,
+                                         prefill_chunk=rng.choice([8, 16, 64]),
+                                         poison_freed_pages=True, use_graph=seed % 3 == 0))
+    sched = Scheduler(runner, Sampler(runner.ops, runner.device))
+    crowd = requests()
+    for r in crowd:
+        sched.add(r)
+    sched.run()
+    for r, w in zip(crowd, want):
+        assert r.status == "finished" and r.output == w, f"{name} seed {seed}: {r.id}"
+    if temp > 0:   # requests that share a seed still draw their own numbers
+        assert len({tuple(o[:4]) for o in want if len(o) >= 4}) > 1
+    runner.cache.check()
+    assert all(g.allocator.in_use == 0 for g in runner.cache.groups)
+
+
 def test_sessions_like_the_reference_binding(model_dirs):
     import ninfer_amd
     d = model_dirs["A"]["float32"]
