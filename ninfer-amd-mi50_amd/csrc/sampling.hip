@@ -6,8 +6,10 @@
 // Differences, all deliberate: the penalty arrives as (token, count) pairs
 // (a token seen c times is penalised c times, as the reference's loop over
 // the history does); top-k and top-p are found by radix selection on the
-// ordered bit pattern of the scaled logits instead of a sort, so ties at a
-// threshold are all kept; probabilities are held as 32.32 fixed-point
+// ordered bit pattern of the scaled logits instead of a sort, and of the tokens
+// tied at the threshold the first ones in index order are kept, so the kept set
+// is the prefix a stable sort by descending logit would give (top_k = 1 is the
+// greedy choice, ties included); probabilities are held as 32.32 fixed-point
 // integers so every sum is exact and the draw does not depend on the order of
 // additions; the draw walks the kept tokens in index order with a uniform
 // number `u` in [0,1) that the caller derives from (seed, request, draw
@@ -21,6 +23,7 @@ constexpr int kSampleThreads = 1024;
 
 __device__ __forceinline__ uint32_t ordered_key(float v) {
   uint32_t b = __float_as_uint(v);
+  if (b == 0x80000000u) b = 0;   // -0 and +0 are one value, as in a comparison of floats
   return (b & 0x80000000u) ? ~b : (b | 0x80000000u);  // ascending with the float order
 }
 
@@ -147,87 +150,116 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
 
   const float inv_t = 1.f / temp;
   const float m = best * inv_t;  // max of the scaled logits (temp > 0)
+  typedef unsigned long long u64;
   auto key = [&](int i) { return ordered_key(w[i] * inv_t); };
-
-  // top-k: keep keys >= the k-th largest
-  uint32_t floor_key = 0;
-  int k = top_k ? top_k[r] : 0;
-  if (k > 0 && k < V)
-    floor_key = radix_select(V, (unsigned long long)k, hist, sel, key,
-                             [](int, uint32_t) { return 1ull; });
-
-  // probabilities of the kept tokens as 32.32 fixed point
-  auto mass = [&](int i, uint32_t kk) -> unsigned long long {
-    if (kk < floor_key) return 0ull;
-    return (unsigned long long)(expf(w[i] * inv_t - m) * 4294967296.f);
+  // probability of a token as 32.32 fixed point; tokens of equal key have equal mass
+  auto mass_of = [&](int i) -> u64 { return (u64)(expf(w[i] * inv_t - m) * 4294967296.f); };
+  auto mass_at = [&](uint32_t kk) -> u64 {
+    const uint32_t bits = (kk & 0x80000000u) ? (kk & 0x7fffffffu) : ~kk;   // ordered_key's inverse
+    return (u64)(expf(__uint_as_float(bits) - m) * 4294967296.f);
   };
-  auto block_total = [&](uint32_t lowest) {
-    unsigned long long s = 0;
-    for (int i = tid; i < V; i += blockDim.x) {
-      uint32_t kk = key(i);
-      if (kk >= lowest) s += mass(i, kk);
-    }
-    sums[tid] = s;
+  auto block_sum = [&](u64 v) -> u64 {
+    sums[tid] = v;
     __syncthreads();
     for (int off = kSampleThreads / 2; off > 0; off >>= 1) {
       if (tid < off) sums[tid] += sums[tid + off];
       __syncthreads();
     }
-    unsigned long long t = sums[0];
+    const u64 t = sums[0];
     __syncthreads();
     return t;
   };
-  unsigned long long total = block_total(floor_key);
-
-  // top-p: the smallest set of most probable tokens whose mass reaches top_p
-  float pp = top_p ? top_p[r] : 1.f;
-  if (pp < 1.f) {
-    unsigned long long target = (unsigned long long)((double)pp * (double)total);
-    if (target < 1) target = 1;
-    uint32_t pk = radix_select(V, target, hist, sel, key, mass);
-    if (pk > floor_key) {
-      floor_key = pk;
-      total = block_total(floor_key);
+  // tokens with a key above t (their count and mass) and with key t (their count)
+  auto stats = [&](uint32_t t, u64& cnt_gt, u64& mass_gt, u64& cnt_eq) {
+    u64 c = 0, ms = 0, e = 0;
+    for (int i = tid; i < V; i += blockDim.x) {
+      const uint32_t kk = key(i);
+      if (kk > t) {
+        ++c;
+        ms += mass_of(i);
+      } else if (kk == t) {
+        ++e;
+      }
     }
+    cnt_gt = block_sum(c);
+    mass_gt = block_sum(ms);
+    cnt_eq = block_sum(e);
+  };
+
+  // The kept set is a prefix of the tokens ordered by (logit descending, index ascending),
+  // as a sort would give it: every token with a key above `thr`, and of the tokens with key
+  // `thr` the first `quota` in index order. Keeping all is thr = 0 with no token at it.
+  uint32_t thr = 0;
+  u64 cnt_gt, mass_gt, cnt_eq;
+  const int k = top_k ? top_k[r] : 0;
+  if (k > 0 && k < V)   // top-k: the k-th largest key
+    thr = radix_select(V, (u64)k, hist, sel, key, [](int, uint32_t) { return 1ull; });
+  stats(thr, cnt_gt, mass_gt, cnt_eq);
+  u64 quota = (k > 0 && k < V) ? (u64)k - cnt_gt : cnt_eq;   // 1 .. cnt_eq with top-k
+  u64 mass_thr = mass_at(thr);
+  u64 total = mass_gt + quota * mass_thr;
+
+  // top-p: the shortest prefix of that order whose mass reaches top_p of the total
+  const float pp = top_p ? top_p[r] : 1.f;
+  if (pp < 1.f) {
+    u64 target = (u64)((double)pp * (double)total);
+    if (target < 1) target = 1;
+    if (target <= mass_gt) {   // it ends among the keys above thr
+      const uint32_t floor_key = thr;
+      thr = radix_select(V, target, hist, sel, key, [&](int i, uint32_t kk) -> u64 {
+        return kk > floor_key ? mass_of(i) : 0ull;
+      });
+      stats(thr, cnt_gt, mass_gt, cnt_eq);
+      mass_thr = mass_at(thr);
+      quota = cnt_eq;
+    }
+    // mass_gt < target <= mass_gt + quota * mass_thr
+    if (mass_thr > 0) {
+      const u64 need = (target - mass_gt + mass_thr - 1) / mass_thr;
+      if (need < quota) quota = need;
+    }
+    total = mass_gt + quota * mass_thr;
   }
 
-  // inverse CDF over the kept tokens in index order
-  unsigned long long goal = (unsigned long long)((double)uniform[r] * (double)total);
+  // inverse CDF over the kept tokens in index order; a thread owns a run of indices
+  u64 goal = (u64)((double)uniform[r] * (double)total);
   if (goal >= total) goal = total - 1;
   const int chunk = (V + blockDim.x - 1) / blockDim.x;
-  const int c0 = tid * chunk, c1 = min(V, c0 + chunk);
-  unsigned long long mine = 0;
-  for (int i = c0; i < c1; ++i) {
-    uint32_t kk = key(i);
-    if (kk >= floor_key) mine += mass(i, kk);
-  }
-  sums[tid] = mine;
-  __syncthreads();
-  if (tid == 0) {
-    unsigned long long run = 0;
-    for (int i = 0; i < (int)blockDim.x; ++i) {
-      unsigned long long s = sums[i];
-      sums[i] = run;
-      run += s;
-    }
-
-  }
-  __syncthreads();
-  unsigned long long before = sums[tid];
-  if (mine > 0 && goal >= before && goal < before + mine) {
-    unsigned long long run = before;
-    int pick = c1 - 1;
-    for (int i = c0; i < c1; ++i) {
-      uint32_t kk = key(i);
-      unsigned long long ms = kk >= floor_key ? mass(i, kk) : 0ull;
-      if (ms && goal < run + ms) {
-        pick = i;
-        break;
+  const int c0 = min(V, tid * chunk), c1 = min(V, c0 + chunk);
+  auto scan = [&](u64 mine) -> u64 {   // sum over the threads before this one
+    sums[tid] = mine;
+    __syncthreads();
+    if (tid == 0) {
+      u64 run = 0;
+      for (int i = 0; i < (int)blockDim.x; ++i) {
+        const u64 v = sums[i];
+        sums[i] = run;
+        run += v;
       }
+    }
+    __syncthreads();
+    const u64 before = sums[tid];
+    __syncthreads();
+    return before;
+  };
+  u64 eq_mine = 0;
+  for (int i = c0; i < c1; ++i) eq_mine += key(i) == thr;
+  const u64 eq_before = scan(eq_mine);
+  auto walk = [&](u64 start, bool pick_it) -> u64 {   // mass of the run; or the token at `goal`
+    u64 run = start, rank = eq_before;
+    for (int i = c0; i < c1; ++i) {
+      const uint32_t kk = key(i);
+      u64 ms = 0;
+      if (kk > thr) ms = mass_of(i);
+      else if (kk == thr && rank++ < quota) ms = mass_thr;
+      if (pick_it && ms && goal < run + ms) return (u64)i;
       run += ms;
     }
-    out[r] = pick;
-  }
+    return pick_it ? (u64)(c1 - 1) : run - start;
+  };
+  const u64 mine = walk(0, false);
+  const u64 before = scan(mine);
+  if (mine > 0 && goal >= before && goal < before + mine) out[r] = (int)walk(before, true);
 }
 
 }  // namespace ninfer

@@ -655,3 +655,41 @@ def test_sample_greedy_and_distribution(ops, gen):
         # a grid of u's samples the inverse CDF: frequencies follow p
         freq = torch.bincount(torch.tensor(draws[i]), minlength=v).float() / len(us)
         assert (freq - p).abs().max() < 3.0 / len(us) + 1e-3
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_sample_ties_keep_the_sorted_prefix(ops, seed):
+    """Logits in a few tiers, so that top-k and top-p cut inside a run of equal values: the
+    kept set is the prefix of the tokens sorted by (logit descending, index ascending), as
+    the plain sampler's sort gives it; top_k = 1 is the greedy choice whatever ties there are.
+    Vocabularies that are no power of two, the penalty applied to tokens seen several times."""
+    import random
+    from collections import Counter
+    import plain_model
+    rng = random.Random(seed)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    v = [2, 17, 97, 1000, 4099, 32000][seed % 6]
+    logits = ((torch.randn(1, v, generator=g, device="cuda") * rng.choice([0.5, 3.0])) * 2).round() / 2
+    temp = rng.choice([0.3, 0.7, 1.0, 2.0])
+    top_k = rng.choice([1, 2, 7, 50, v + 5]) if seed % 4 else 1
+    top_p = rng.choice([1.0, 0.9, 0.5, 0.1, 0.01])
+    rp = rng.choice([1.0, 1.3, 2.0])
+    recent = [rng.randrange(v) for _ in range(rng.choice([0, 5, 40]))]
+    seen = Counter(recent)
+    i32 = lambda x: torch.tensor(x, device="cuda", dtype=torch.int32)
+    f32 = lambda x: torch.tensor([x], device="cuda", dtype=torch.float32)
+    p = plain_model.sample_distribution(logits[0].cpu(), temp, top_k, top_p, rp, recent)
+    n = 300
+    out = torch.empty(1, device="cuda", dtype=torch.int32)
+    draws = []
+    for i in range(n):
+        ops.sample(logits, f32(temp), f32((i + 0.5) / n), out, top_k=i32([top_k]), top_p=f32(top_p),
+                   rep_penalty=f32(rp), pen_tokens=i32(list(seen.keys()) or [0]),
+                   pen_counts=i32(list(seen.values()) or [0]), pen_offsets=i32([0, len(seen)]))
+        draws.append(int(out[0]))
+    assert set(draws) <= set(torch.nonzero(p).flatten().tolist())
+    freq = torch.bincount(torch.tensor(draws), minlength=v).float() / n
+    assert (freq - p).abs().max() < 3.0 / n + 2e-3
+    if top_k == 1:
+        assert len(set(draws)) == 1
