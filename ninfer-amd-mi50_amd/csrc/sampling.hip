@@ -226,25 +226,32 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   if (goal >= total) goal = total - 1;
   const int chunk = (V + blockDim.x - 1) / blockDim.x;
   const int c0 = min(V, tid * chunk), c1 = min(V, c0 + chunk);
-  auto scan = [&](u64 mine) -> u64 {   // sum over the threads before this one
-    sums[tid] = mine;
-    __syncthreads();
-    if (tid == 0) {
-      u64 run = 0;
-      for (int i = 0; i < (int)blockDim.x; ++i) {
-        const u64 v = sums[i];
-        sums[i] = run;
-        run += v;
-      }
-    }
-    __syncthreads();
-    const u64 before = sums[tid];
-    __syncthreads();
-    return before;
+  auto shfl_up64 = [](u64 v, int d) -> u64 {
+    const uint32_t lo = __shfl_up((uint32_t)v, d, 64), hi = __shfl_up((uint32_t)(v >> 32), d, 64);
+    return ((u64)hi << 32) | lo;
   };
-  u64 eq_mine = 0;
-  for (int i = c0; i < c1; ++i) eq_mine += key(i) == thr;
-  const u64 eq_before = scan(eq_mine);
+  auto scan = [&](u64 mine) -> u64 {   // sum over the threads before this one
+    const int lane = tid & 63, wv = tid >> 6;
+    u64 incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const u64 o = shfl_up64(incl, d);
+      if (lane >= d) incl += o;
+    }
+    if (lane == 63) sums[wv] = incl;
+    __syncthreads();
+    u64 base = 0;
+    for (int i = 0; i < wv; ++i) base += sums[i];   // at most 15 wave totals
+    __syncthreads();
+    return base + incl - mine;
+  };
+  // ranks among the tokens tied at the threshold are needed only when not all of them are kept
+  u64 eq_before = 0;
+  if (quota < cnt_eq) {
+    u64 eq_mine = 0;
+    for (int i = c0; i < c1; ++i) eq_mine += key(i) == thr;
+    eq_before = scan(eq_mine);
+  }
   auto walk = [&](u64 start, bool pick_it) -> u64 {   // mass of the run; or the token at `goal`
     u64 run = start, rank = eq_before;
     for (int i = c0; i < c1; ++i) {
