@@ -104,31 +104,38 @@ class Sampler:
         """One token per row of `logits` [R, vocab]."""
         r = len(rows)
         assert logits.shape[0] == r
-        temp = [row.params.temperature for row in rows]
-        top_k = [row.params.top_k for row in rows]
-        top_p = [row.params.top_p for row in rows]
-        rp = [row.params.repetition_penalty for row in rows]
-        u = [uniform(row.seed, row.key, row.draw) for row in rows]
+        # Everything the kernel needs of the rows travels in one array and one copy: four
+        # 32-bit floats and one int per row, the offsets of the penalties, then their tokens
+        # and counts. (Copies queue behind the step that makes the logits, one after the other:
+        # every further one would add its latency to the step.)
         pen_t: List[np.ndarray] = []
         pen_c: List[np.ndarray] = []
-        pen_o = [0]
-        for row in rows:
+        pen_o = np.zeros(r + 1, np.int32)
+        for i, row in enumerate(rows):
             n = 0
             if row.params.repetition_penalty != 1.0:
                 toks, cnts = row.history.arrays()
                 pen_t.append(toks)
                 pen_c.append(cnts)
                 n = toks.shape[0]
-            pen_o.append(pen_o[-1] + n)
-        dev = self.device
-        f32 = lambda v: torch.tensor(v, dtype=torch.float32, device=dev)
-        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
-        out = torch.empty(r, dtype=torch.int32, device=dev)
+            pen_o[i + 1] = pen_o[i] + n
+        floats = np.empty((4, r), np.float32)
+        floats[0] = [row.params.temperature for row in rows]
+        floats[1] = [row.params.top_p for row in rows]
+        floats[2] = [row.params.repetition_penalty for row in rows]
+        floats[3] = [uniform(row.seed, row.key, row.draw) for row in rows]
+        top_k = np.asarray([row.params.top_k for row in rows], np.int32)
+        n_pen = int(pen_o[-1])
+        packed = np.concatenate([floats.reshape(-1).view(np.int32), top_k, pen_o] + pen_t + pen_c)
+        dev = torch.from_numpy(packed).to(self.device)
+        f = dev[:4 * r].view(torch.float32)
+        o = 4 * r
         pen = {}
-        if pen_o[-1] > 0:
-            pen = dict(pen_tokens=torch.from_numpy(np.concatenate(pen_t)).to(dev),
-                       pen_counts=torch.from_numpy(np.concatenate(pen_c)).to(dev),
-                       pen_offsets=i32(pen_o))
-        self.ops.sample(logits, f32(temp), f32(u), out, top_k=i32(top_k), top_p=f32(top_p),
-                        rep_penalty=f32(rp), **pen)
+        if n_pen > 0:
+            pen = dict(pen_offsets=dev[o + r:o + 2 * r + 1],
+                       pen_tokens=dev[o + 2 * r + 1:o + 2 * r + 1 + n_pen],
+                       pen_counts=dev[o + 2 * r + 1 + n_pen:o + 2 * r + 1 + 2 * n_pen])
+        out = torch.empty(r, dtype=torch.int32, device=self.device)
+        self.ops.sample(logits, f[:r], f[3 * r:4 * r], out, top_k=dev[o:o + r], top_p=f[r:2 * r],
+                        rep_penalty=f[2 * r:3 * r], **pen)
         return out.tolist()
