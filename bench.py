@@ -10,7 +10,8 @@ keys and values; token ids are seeded random). A step is one decode step: one
 new token for every request of the batch through the engine's step function
 (replayed from a captured HIP graph unless --no-graph) and its device sampler. One JSON line is printed: decoded tokens a second as
 `value`; the 2,048-token prefill under "prefill"; the decode step's memory
-roofline under "roofline"; decode at batch 1 and 64 under "points"; and under
+roofline under "roofline" (with the rate of a plain device copy measured beside it, and the
+step's fraction of that); decode at batch 1 and 64 under "points"; and under
 "graph_check" the largest difference between replayed and eager decode steps at
 those batches (untimed; 0.0 when the replays are exact).
 Peaks: HBM 8 TB/s; dense bf16 MFMA 2.5 PFLOP/s (fp32 157.3 TFLOP/s).
@@ -194,6 +195,20 @@ def main() -> int:
         runner._graphs.clear()
         return max(float((a - b).abs().max()) for a, b in zip(*outs))
 
+    def copy_rate() -> float:
+        """Bytes a second that a plain device copy of 2 GiB moves (read + write): what the
+        memory system gives a kernel that does nothing else."""
+        src = torch.empty(1 << 29, dtype=torch.float32, device=runner.device).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(2):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        return 5 * 2 * src.numel() * 4 / (time.perf_counter() - t)
+
     dt, nbytes, n_exp = decode_run(args.batch, args.steps, args.warmup)
     result = {
         "metric": f"decode tok/s at batch {args.batch} ({model_name} shapes, context {ctx})",
@@ -212,6 +227,9 @@ def main() -> int:
                      "frac": round(nbytes / dt / HBM_PEAK, 4),
                      "distinct_experts_per_layer": round(n_exp, 1)},
     }
+    copied = copy_rate()
+    result["roofline"]["measured_copy"] = round(copied / 1e9, 1)
+    result["roofline"]["frac_of_copy"] = round(nbytes / dt / copied, 4)
     if not args.no_prefill:
         pt = min(args.prefill_tokens, ctx)
         pdt, flops = prefill_run(pt, 3)
