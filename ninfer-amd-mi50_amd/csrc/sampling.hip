@@ -71,7 +71,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ top_p, const float* __restrict__ rep_penalty,
     const int* __restrict__ pen_tokens, const int* __restrict__ pen_counts,
     const int* __restrict__ pen_offsets, const float* __restrict__ uniform,
-    int* __restrict__ out) {
+    const int* __restrict__ index_map, int* __restrict__ out) {
   __shared__ unsigned long long hist[256];
   __shared__ unsigned long long sums[kSampleThreads];
   __shared__ float fred[kSampleThreads / 64];
@@ -142,8 +142,10 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
       best_i = ired[i];
     }
   }
+  // (the row may be a list of candidates: index_map gives the token behind each place)
+  const int* map = index_map ? index_map + (int64_t)r * V : nullptr;
   if (!(temp > 0.f)) {
-    if (tid == 0) out[r] = best_i;
+    if (tid == 0) out[r] = map ? map[best_i] : best_i;
     return;
   }
   __syncthreads();
@@ -266,7 +268,119 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   };
   const u64 mine = walk(0, false);
   const u64 before = scan(mine);
-  if (mine > 0 && goal >= before && goal < before + mine) out[r] = (int)walk(before, true);
+  if (mine > 0 && goal >= before && goal < before + mine) {
+    const int pick = (int)walk(before, true);
+    out[r] = map ? map[pick] : pick;
+  }
+}
+
+// Candidates for rows that keep few tokens (greedy, or top-k up to kCandPerSlice): the row is
+// cut into slices of kSlice tokens, one block each, so that the whole GPU reads the logits
+// instead of one CU. A block holds its slice in LDS, applies the repetition penalty to it, and
+// writes out, in index order, its own k best tokens under the order (scaled logit descending,
+// index ascending). Every token of the row's k best is among its slice's k best, so the
+// sampling kernel run on the candidates (sample_kernel with an index map) keeps the same set,
+// sums the same masses and draws the same token as on the whole row.
+constexpr int kSlice = 4096;
+constexpr int kCandPerSlice = 64;
+constexpr int kCandThreads = 256;
+
+__global__ __launch_bounds__(kCandThreads) void sample_candidates_kernel(
+    const float* __restrict__ logits, int ld, int V, const float* __restrict__ temperature,
+    const int* __restrict__ top_k, const float* __restrict__ rep_penalty,
+    const int* __restrict__ pen_tokens, const int* __restrict__ pen_counts,
+    const int* __restrict__ pen_offsets, float* __restrict__ cand_val, int* __restrict__ cand_idx) {
+  __shared__ float vals[kSlice];
+  __shared__ unsigned long long hist[256];
+  __shared__ __align__(8) uint32_t sel[4];
+  __shared__ int wave_tot[kCandThreads / 64];
+  const int r = blockIdx.y, b = blockIdx.x, tid = threadIdx.x;
+  const int s0 = b * kSlice, n = min(kSlice, V - s0);
+  const int C = gridDim.x * kCandPerSlice;
+  const float* row = logits + (int64_t)r * ld;
+  for (int i = tid; i < kSlice; i += kCandThreads) vals[i] = i < n ? row[s0 + i] : -INFINITY;
+  __syncthreads();
+  const float rp = rep_penalty ? rep_penalty[r] : 1.f;
+  if (rp != 1.f && pen_offsets) {
+    for (int e = pen_offsets[r] + tid; e < pen_offsets[r + 1]; e += kCandThreads) {
+      const int tok = pen_tokens[e] - s0;
+      if (tok < 0 || tok >= n) continue;
+      float v = vals[tok];
+      for (int c = 0; c < pen_counts[e]; ++c) v = v > 0.f ? v / rp : v * rp;
+      vals[tok] = v;
+    }
+    __syncthreads();
+  }
+  const float temp = temperature[r];
+  const float inv_t = temp > 0.f ? 1.f / temp : 1.f;
+  int k = temp > 0.f ? top_k[r] : 1;            // greedy is the best one
+  if (k < 1 || k > kCandPerSlice) k = kCandPerSlice;   // (not this entry's rows: kept in bounds)
+  auto key = [&](int i) { return ordered_key(vals[i] * inv_t); };
+  // the slice's k-th largest key, and how many of the tokens tied at it are kept
+  uint32_t thr = 0;
+  int quota = kSlice;
+  if (k < n) {
+    thr = radix_select(n, (unsigned long long)k, hist, sel, key, [](int, uint32_t) { return 1ull; });
+    int above = 0;
+    for (int i = tid; i < n; i += kCandThreads) above += key(i) > thr;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) above += __shfl_xor(above, off, 64);
+    if ((tid & 63) == 0) wave_tot[tid >> 6] = above;
+    __syncthreads();
+    above = 0;
+    for (int i = 0; i < kCandThreads / 64; ++i) above += wave_tot[i];
+    __syncthreads();
+    quota = k - above;
+  }
+  // in index order: a thread owns a run of consecutive tokens
+  constexpr int RUN = kSlice / kCandThreads;
+  auto scan = [&](int mine) -> int {   // sum over the threads before this one
+    const int lane = tid & 63, wv = tid >> 6;
+    int incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int o = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += o;
+    }
+    if (lane == 63) wave_tot[wv] = incl;
+    __syncthreads();
+    int base = 0;
+    for (int i = 0; i < wv; ++i) base += wave_tot[i];
+    __syncthreads();
+    return base + incl - mine;
+  };
+  const int i0 = tid * RUN, i1 = min(n, i0 + RUN);
+  int eq = 0;
+  for (int i = i0; i < i1; ++i) eq += key(i) == thr;
+  int rank = scan(eq);
+  int kept = 0;
+  bool keep[RUN];
+#pragma unroll
+  for (int u = 0; u < RUN; ++u) {
+    const int i = i0 + u;
+    keep[u] = false;
+    if (i < i1) {
+      const uint32_t kk = key(i);
+      keep[u] = kk > thr || (kk == thr && rank++ < quota);
+    }
+    kept += keep[u];
+  }
+  int pos = scan(kept);
+  float* cv = cand_val + (int64_t)r * C + b * kCandPerSlice;
+  int* ci = cand_idx + (int64_t)r * C + b * kCandPerSlice;
+#pragma unroll
+  for (int u = 0; u < RUN; ++u)
+    if (keep[u]) {   // at most min(k, n) <= kCandPerSlice places
+      cv[pos] = vals[i0 + u];
+      ci[pos] = s0 + i0 + u;
+      ++pos;
+    }
+  // the places left over hold nothing: never the largest, no mass
+  const int total = min(k, n);
+  for (int i = total + tid; i < kCandPerSlice; i += kCandThreads) {
+    cv[i] = -INFINITY;
+    ci[i] = 0;
+  }
 }
 
 }  // namespace ninfer
@@ -287,7 +401,39 @@ extern "C" int ninfer_sample(const float* logits, int ld, int V, int R, float* w
   NINFER_REQUIRE(temperature && uniform && work && out, "sample: a required array is null");
   sample_kernel<<<R, kSampleThreads, 0, stream>>>(logits, ld, V, work, temperature, top_k, top_p,
                                                   rep_penalty, pen_tokens, pen_counts, pen_offsets,
-                                                  uniform, out);
+                                                  uniform, nullptr, out);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+// Places per row that ninfer_sample_few needs in each of cand_val, cand_idx and work.
+extern "C" long long ninfer_sample_few_places(int V) {
+  return (long long)((V + kSlice - 1) / kSlice) * kCandPerSlice;
+}
+
+// The same for rows that all keep few tokens: every row greedy (temperature <= 0) or with
+// 1 <= top_k <= 64, which the caller asserts (a row with another top_k would be cut to its 64
+// best per slice). Same result as ninfer_sample, from two launches that use the whole GPU.
+// cand_val, cand_idx, work: [R, ninfer_sample_few_places(V)].
+extern "C" int ninfer_sample_few(const float* logits, int ld, int V, int R, float* cand_val,
+                                 int* cand_idx, float* work, const float* temperature,
+                                 const int* top_k, const float* top_p, const float* rep_penalty,
+                                 const int* pen_tokens, const int* pen_counts,
+                                 const int* pen_offsets, const float* uniform, int* out,
+                                 hipStream_t stream) {
+  NINFER_REQUIRE(R > 0 && V > 0, "sample: R=%d V=%d must be positive", R, V);
+  NINFER_REQUIRE(ld >= V, "sample: row stride %d < vocabulary %d", ld, V);
+  NINFER_REQUIRE(temperature && top_k && uniform && cand_val && cand_idx && work && out,
+                 "sample: a required array is null");
+  const int slices = (V + kSlice - 1) / kSlice, C = slices * kCandPerSlice;
+  NINFER_REQUIRE(R <= 65535, "sample: %d rows are too many", R);
+  sample_candidates_kernel<<<dim3(slices, R), kCandThreads, 0, stream>>>(
+      logits, ld, V, temperature, top_k, rep_penalty, pen_tokens, pen_counts, pen_offsets, cand_val,
+      cand_idx);
+  NINFER_LAUNCH_CHECK();
+  sample_kernel<<<R, kSampleThreads, 0, stream>>>(cand_val, C, C, work, temperature, top_k, top_p,
+                                                  nullptr, nullptr, nullptr, nullptr, uniform,
+                                                  cand_idx, out);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

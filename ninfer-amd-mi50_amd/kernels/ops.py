@@ -102,6 +102,7 @@ class HipOps:
         self.lib = ctypes.CDLL(self.lib_path)
         self.lib.ninfer_last_error.restype = ctypes.c_char_p
         self.lib.ninfer_attention_workspace_floats.restype = ctypes.c_longlong
+        self.lib.ninfer_sample_few_places.restype = ctypes.c_longlong
         self.force_generic = False  # tests: run the plain kernels whatever the shape
         self._held = None           # products held back inside `together()`
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
@@ -506,8 +507,12 @@ class HipOps:
                                                  1 if self.force_generic else 0, self._stream()))
 
     # ---- sampling -------------------------------------------------------------------
+    FEW_TOKENS = 64   # most tokens a row may keep (top_k) for the two-launch sampling path
+
     def sample(self, logits, temperature, uniform, out, top_k=None, top_p=None, rep_penalty=None,
-               pen_tokens=None, pen_counts=None, pen_offsets=None):
+               pen_tokens=None, pen_counts=None, pen_offsets=None, few=False):
+        """One token per row. `few`: the caller asserts that every row is greedy
+        (temperature <= 0) or has 1 <= top_k <= FEW_TOKENS; same result, much faster."""
         _dev(logits, "logits", torch.float32, 2)
         r, v = logits.shape
         _dev(temperature, "temperature", torch.float32, 1)
@@ -525,6 +530,24 @@ class HipOps:
             _dev(pen_tokens, "pen_tokens", torch.int32, 1)
             _dev(pen_counts, "pen_counts", torch.int32, 1)
             _need(pen_offsets.shape[0] == r + 1, "sample: pen_offsets has the wrong size")
+        if few:
+            # every row keeps few tokens (the caller knows its rows' options): candidates from
+            # the whole GPU first, then the same selection and draw on those
+            _need(top_k is not None, "sample: rows that keep few tokens need top_k")
+            places = int(self.lib.ninfer_sample_few_places(v))
+            cand_val = torch.empty((r, places), dtype=torch.float32, device=logits.device)
+            cand_idx = torch.empty((r, places), dtype=torch.int32, device=logits.device)
+            work = torch.empty((r, places), dtype=torch.float32, device=logits.device)
+            self._ok(self.lib.ninfer_sample_few(
+                ctypes.c_void_p(logits.data_ptr()), logits.stride(0), v, r,
+                ctypes.c_void_p(cand_val.data_ptr()), ctypes.c_void_p(cand_idx.data_ptr()),
+                ctypes.c_void_p(work.data_ptr()), ctypes.c_void_p(temperature.data_ptr()),
+                ctypes.c_void_p(top_k.data_ptr()), ctypes.c_void_p(_ptr(top_p)),
+                ctypes.c_void_p(_ptr(rep_penalty)), ctypes.c_void_p(_ptr(pen_tokens)),
+                ctypes.c_void_p(_ptr(pen_counts)), ctypes.c_void_p(_ptr(pen_offsets)),
+                ctypes.c_void_p(uniform.data_ptr()), ctypes.c_void_p(out.data_ptr()),
+                self._stream()))
+            return
         work = torch.empty((r, v), dtype=torch.float32, device=logits.device)
         self._ok(self.lib.ninfer_sample(
             ctypes.c_void_p(logits.data_ptr()), logits.stride(0), v, r,

@@ -136,6 +136,13 @@ class Sampler:
                        pen_tokens=dev[o + 2 * r + 1:o + 2 * r + 1 + n_pen],
                        pen_counts=dev[o + 2 * r + 1 + n_pen:o + 2 * r + 1 + 2 * n_pen])
         out = torch.empty(r, dtype=torch.int32, device=self.device)
+        # rows that are greedy or keep at most a few dozen tokens (the reference's default is
+        # top_k = 50) take the path that reads the logits with the whole GPU
+        most = getattr(self.ops, "FEW_TOKENS", 0)
+        # (rows that are all greedy stay with the one launch: it is short as it is)
+        if most and any(row.params.temperature > 0 for row in rows) and all(
+                row.params.temperature <= 0 or 1 <= row.params.top_k <= most for row in rows):
+            pen["few"] = True
         self.ops.sample(logits, f[:r], f[3 * r:4 * r], out, top_k=dev[o:o + r], top_p=f[r:2 * r],
                         rep_penalty=f[2 * r:3 * r], **pen)
         return out.tolist()

@@ -693,3 +693,36 @@ def test_sample_ties_keep_the_sorted_prefix(ops, seed):
     assert (freq - p).abs().max() < 3.0 / n + 2e-3
     if top_k == 1:
         assert len(set(draws)) == 1
+
+
+@pytest.mark.parametrize("v", [70, 4096, 4097, 20011, 151936])
+def test_sample_rows_that_keep_few_tokens(ops, gen, v):
+    """Rows that are greedy or keep at most 64 tokens have a path of two launches that reads
+    the logits with the whole GPU: the same tokens as the one-block path, row by row, with
+    penalties, ties, a vocabulary that ends inside a slice, and top_k beyond the vocabulary's
+    last slice."""
+    r = 9
+    logits = torch.randn(r, v, generator=gen, device="cuda") * 3
+    logits[1] = (logits[1] * 2).round() / 2                      # ties
+    logits[2, -1] = 40.0                                          # the best one is the last token
+    logits[3] = 1.0                                               # all equal
+    temp = torch.tensor([0.0, 0.7, 1.0, 0.9, 0.3, 0.0, 2.0, 1.0, 0.7], device="cuda")
+    top_k = torch.tensor([0, 50, 1, 64, 7, 5, 33, 2, 64], device="cuda", dtype=torch.int32)
+    top_p = torch.tensor([1.0, 0.95, 1.0, 0.5, 0.9, 1.0, 0.99, 0.01, 1.0], device="cuda")
+    rp = torch.tensor([1.3, 1.05, 1.0, 1.0, 2.0, 1.0, 1.1, 1.0, 1.5], device="cuda")
+    pens = [[0, 5 % v, v - 1], [1, 2, 3], [], [], [int(torch.argmax(logits[4]))], [], [7 % v], [], list(range(0, v, 3))]
+    offs = [0]
+    for p in pens:
+        offs.append(offs[-1] + len(p))
+    i32 = lambda x: torch.tensor(x, device="cuda", dtype=torch.int32)
+    flat = [t for p in pens for t in p]
+    args = dict(top_k=top_k, top_p=top_p, rep_penalty=rp, pen_tokens=i32(flat),
+                pen_counts=i32([1 + i % 3 for i in range(len(flat))]), pen_offsets=i32(offs))
+    a = torch.empty(r, device="cuda", dtype=torch.int32)
+    b = torch.empty_like(a)
+    for u in torch.linspace(0.001, 0.999, 41).tolist():
+        uniform = torch.full((r,), u, device="cuda")
+        ops.sample(logits, temp, uniform, a, **args)
+        ops.sample(logits, temp, uniform, b, few=True, **args)
+        assert torch.equal(a, b), f"u={u}: {a.tolist()} vs {b.tolist()}"
+    assert int(a[2]) == v - 1 or float(temp[2]) > 0
