@@ -36,10 +36,14 @@ constexpr int SM = 16;  // rows of A per tile
 // share the K range at compile time; WAVES == 0 takes them from `waves_arg` (waves of the
 // block beyond that number must not call). `red` holds waves x (2 with SwiGLU, else 1) x 256
 // floats.
-template <int WAVES, bool FULL, bool SWIGLU, typename TC>
+// TWO: the block owns 32 output features, as two sets of 16 W rows that meet the same
+// activations (for products with many small tiles: half the blocks, each activation row
+// read once for twice the weights). Not with SwiGLU, which has its two sets already.
+template <int WAVES, bool FULL, bool SWIGLU, typename TC, bool TWO = false>
 __device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, int waves_arg,
                                              int bx, int by, float* red, int* tile_info) {
-  constexpr int HALVES = SWIGLU ? 2 : 1;
+  static_assert(!(TWO && SWIGLU) && (!TWO || FULL), "two feature sets: whole tiles, no SwiGLU");
+  constexpr int HALVES = (SWIGLU || TWO) ? 2 : 1;
   const int waves = WAVES > 0 ? WAVES : waves_arg;
   int row0, row_end, group = 0;
   if (a.offsets && a.tiles16) {
@@ -64,14 +68,16 @@ __device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, in
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, j = lane >> 4;
   const int rows = FULL ? 16 : rows_arg;   // features per block, at most 16
-  const int n0 = bx * rows;
+  const int n0 = bx * (TWO ? 32 : rows);
   const bool w_valid = FULL || r < rows;   // lanes of the empty rows load nothing
   const int K = a.K;
 
   const bf16* W = (const bf16*)a.W + (int64_t)group * a.w_group_stride;
   const int n = min(n0 + r, a.N - 1);
   const bf16* wrow = W + (int64_t)n * K + 8 * j;
-  const bf16* urow = SWIGLU ? wrow + (int64_t)a.N * K : nullptr;
+  const bf16* urow = SWIGLU ? wrow + (int64_t)a.N * K
+                     : TWO  ? W + (int64_t)min(n0 + 16 + r, a.N - 1) * K + 8 * j
+                            : nullptr;
 
   const int mrow = row0 + r;
   const bool m_valid = mrow < row_end;
@@ -91,21 +97,21 @@ __device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, in
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         w[i] = w_valid ? *(const bf16x8*)(wrow + (s0 + i) * 32) : zero;
-        if (SWIGLU) u[i] = w_valid ? *(const bf16x8*)(urow + (s0 + i) * 32) : zero;
+        if (SWIGLU || TWO) u[i] = w_valid ? *(const bf16x8*)(urow + (s0 + i) * 32) : zero;
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) x[i] = m_valid ? *(const bf16x8*)(xrow + (s0 + i) * 32) : zero;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[i], x[i], acc, 0, 0, 0);
-        if (SWIGLU) accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u[i], x[i], accu, 0, 0, 0);
+        if (SWIGLU || TWO) accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u[i], x[i], accu, 0, 0, 0);
       }
     } else {
       for (int s = s0; s < steps; ++s) {
         bf16x8 w = w_valid ? *(const bf16x8*)(wrow + s * 32) : zero;
         bf16x8 x = m_valid ? *(const bf16x8*)(xrow + s * 32) : zero;
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, x, acc, 0, 0, 0);
-        if (SWIGLU) {
+        if (SWIGLU || TWO) {
           bf16x8 u = w_valid ? *(const bf16x8*)(urow + s * 32) : zero;
           accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u, x, accu, 0, 0, 0);
         }
@@ -118,7 +124,7 @@ __device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, in
   for (int v = 0; v < 4; ++v) {
     int f = 4 * j + v;
     red[(wave * HALVES) * 256 + r * 16 + f] = acc[v];
-    if (SWIGLU) red[(wave * HALVES + 1) * 256 + r * 16 + f] = accu[v];
+    if (SWIGLU || TWO) red[(wave * HALVES + 1) * 256 + r * 16 + f] = accu[v];
   }
   __syncthreads();
   if (threadIdx.x < 256) {
@@ -130,24 +136,27 @@ __device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, in
       for (int w = 0; w < (WAVES > 0 ? WAVES : 16); ++w) {
         if (WAVES == 0 && w >= waves) break;
         v += red[(w * HALVES) * 256 + threadIdx.x];
-        if (SWIGLU) up += red[(w * HALVES + 1) * 256 + threadIdx.x];
+        if (SWIGLU || TWO) up += red[(w * HALVES + 1) * 256 + threadIdx.x];
       }
       if (SWIGLU) {
         v = v / (1.f + __expf(-v)) * up;
       } else if (a.bias) {
         v += a.bias[col];
+        if (TWO && col + 16 < a.N) up += a.bias[col + 16];
       }
       int64_t c_row = a.c_index ? a.c_index[row] : row;
       ((TC*)a.C)[c_row * a.ldc + col] = from_f32<TC>(v);
+      if (TWO && col + 16 < a.N) ((TC*)a.C)[c_row * a.ldc + col + 16] = from_f32<TC>(up);
     }
   }
 }
 
-template <int WAVES, bool FULL, bool SWIGLU, typename TC>
+template <int WAVES, bool FULL, bool SWIGLU, typename TC, bool TWO = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a, int rows_arg) {
-  __shared__ float red[WAVES * (SWIGLU ? 2 : 1) * 256];
+  __shared__ float red[WAVES * ((SWIGLU || TWO) ? 2 : 1) * 256];
   __shared__ int tile_info[3];
-  skinny_block<WAVES, FULL, SWIGLU, TC>(a, rows_arg, WAVES, blockIdx.x, blockIdx.y, red, tile_info);
+  skinny_block<WAVES, FULL, SWIGLU, TC, TWO>(a, rows_arg, WAVES, blockIdx.x, blockIdx.y, red,
+                                            tile_info);
 }
 
 // Two products that do not depend on each other in one launch: the first blocks are the
@@ -158,12 +167,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a, int
 // does not use leave at once.
 struct SkinnyPlan {
   int waves;    // waves that share the K range
-  int rows;     // features per block
+  int rows;     // features per block (32 with `two`)
   int grid_x;
   int grid_y;
+  bool two;     // two sets of 16 features per block
 };
 
-template <bool FULL_A, bool SW_A, typename TC_A, bool FULL_B, bool SW_B, typename TC_B>
+template <bool FULL_A, bool SW_A, typename TC_A, bool FULL_B, bool SW_B, typename TC_B,
+          bool TWO_A = false>
 __global__ __launch_bounds__(1024) void gemm_skinny_pair_kernel(GemmArgs a, SkinnyPlan pa,
                                                                GemmArgs b, SkinnyPlan pb) {
   __shared__ float red[16 * 2 * 256];
@@ -178,17 +189,24 @@ __global__ __launch_bounds__(1024) void gemm_skinny_pair_kernel(GemmArgs a, Skin
   } else {
     id -= blocks_b;
     if (wave >= pa.waves) return;
-    skinny_block<0, FULL_A, SW_A, TC_A>(a, pa.rows, pa.waves, id % pa.grid_x, id / pa.grid_x, red,
-                                        tile_info);
+    skinny_block<0, FULL_A, SW_A, TC_A, TWO_A>(a, pa.rows, pa.waves, id % pa.grid_x,
+                                               id / pa.grid_x, red, tile_info);
   }
 }
 
 template <int WAVES>
-static void launch_skinny(const GemmArgs& a, int rows, hipStream_t stream) {
+static void launch_skinny(const GemmArgs& a, int rows, bool two, hipStream_t stream) {
   int m_tiles = a.offsets ? min((a.M + SM - 1) / SM + a.groups, a.M) : (a.M + SM - 1) / SM;
   dim3 grid((a.N + rows - 1) / rows, m_tiles);   // as plan_skinny counts them
   dim3 block(WAVES * 64);
   bool swiglu = a.epilogue == kEpilogueSwiGLU;
+  if (two) {   // whole tiles, no SwiGLU (plan_skinny)
+    if (a.out_dtype == kF32)
+      gemm_skinny_kernel<WAVES, true, false, float, true><<<grid, block, 0, stream>>>(a, 16);
+    else
+      gemm_skinny_kernel<WAVES, true, false, bf16, true><<<grid, block, 0, stream>>>(a, 16);
+    return;
+  }
 #define NINFER_SKINNY(FULL)                                                                   \
   do {                                                                                        \
     if (a.out_dtype == kF32) {                                                                \
@@ -213,6 +231,9 @@ bool gemm_skinny_takes(const GemmArgs& a) {
          ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0) && a.w_group_stride % 8 == 0;
 }
 
+static int g_skinny_two = 1;   // tests and measurements switch the two-set blocks off
+static long g_skinny_two_min = 4096;
+
 static SkinnyPlan plan_skinny(const GemmArgs& a) {
   SkinnyPlan p;
   // more waves per block when the grid alone would leave CUs idle (grouped: at most one tile
@@ -234,6 +255,11 @@ static SkinnyPlan plan_skinny(const GemmArgs& a) {
     p.rows = (int)(((long)a.N * m_tiles + per_cu * cus - 1) / (per_cu * cus));
   }
   p.waves = (blocks < 512 && chunks >= 16) ? 16 : (blocks < 2048 && chunks >= 8) ? 8 : 4;
+  // a grouped product without SwiGLU whose tiles are many and short (K small): two feature
+  // sets per block, so that blocks are half as many and each does twice the work
+  p.two = g_skinny_two && a.offsets && a.epilogue == kEpilogueNone && p.rows == 16 && p.waves == 4 &&
+          blocks >= g_skinny_two_min && a.N % 32 == 0;
+  if (p.two) p.rows = 32;
   p.grid_x = (a.N + p.rows - 1) / p.rows;
   return p;
 }
@@ -241,11 +267,11 @@ static SkinnyPlan plan_skinny(const GemmArgs& a) {
 int gemm_skinny(const GemmArgs& a, hipStream_t stream) {
   const SkinnyPlan p = plan_skinny(a);
   if (p.waves == 16)
-    launch_skinny<16>(a, p.rows, stream);
+    launch_skinny<16>(a, p.rows, false, stream);
   else if (p.waves == 8)
-    launch_skinny<8>(a, p.rows, stream);
+    launch_skinny<8>(a, p.rows, false, stream);
   else
-    launch_skinny<4>(a, p.rows, stream);
+    launch_skinny<4>(a, p.rows, p.two, stream);
   NINFER_LAUNCH_CHECK();
   return 0;
 }
@@ -267,7 +293,7 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream) {
   SkinnyPlan pa = plan_skinny(a), pb = plan_skinny(b);
   // beside a grouped product with many blocks, which are small, the dense one takes the same
   // few waves: blocks as wide as the larger need would hold up the small blocks' places
-  if (a.offsets) {   // the pair's grouped kernel has whole tiles of 16 features
+  if (a.offsets && !pa.two) {   // the pair's grouped kernel has whole tiles of 16 features
     pa.rows = 16;
     pa.grid_x = (a.N + 15) / 16;
   }
@@ -278,6 +304,9 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream) {
   if (!a.offsets)
     gemm_skinny_pair_kernel<false, false, float, false, true, bf16>
         <<<(unsigned)blocks, threads, 0, stream>>>(a, pa, b, pb);
+  else if (pa.two)
+    gemm_skinny_pair_kernel<true, false, bf16, false, false, bf16, true>
+        <<<(unsigned)blocks, threads, 0, stream>>>(a, pa, b, pb);
   else
     gemm_skinny_pair_kernel<true, false, bf16, false, false, bf16>
         <<<(unsigned)blocks, threads, 0, stream>>>(a, pa, b, pb);
@@ -286,3 +315,8 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream) {
 }
 
 }  // namespace ninfer
+
+extern "C" void ninfer_set_skinny_two(int v, long min_blocks) {
+  ninfer::g_skinny_two = v;
+  if (min_blocks > 0) ninfer::g_skinny_two_min = min_blocks;
+}

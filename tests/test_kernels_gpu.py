@@ -726,3 +726,42 @@ def test_sample_rows_that_keep_few_tokens(ops, gen, v):
         ops.sample(logits, temp, uniform, b, few=True, **args)
         assert torch.equal(a, b), f"u={u}: {a.tolist()} vs {b.tolist()}"
     assert int(a[2]) == v - 1 or float(temp[2]) > 0
+
+
+@pytest.mark.parametrize("t,e,k,h,inner", [(8, 60, 4, 256, 160), (64, 8, 3, 96, 64), (40, 6, 2, 160, 96),
+                                           (3, 130, 6, 64, 32), (17, 5, 2, 320, 1408)])
+def test_grouped_down_with_two_feature_sets_per_block(ops, gen, t, e, k, h, inner):
+    """The few-row grouped product with blocks of 32 features (two sets of 16 that meet the same
+    activations; chosen for products of many short tiles, forced here) gives the bits of the
+    blocks of 16, alone and beside a dense product in one launch; widths that are no multiple
+    of 32 keep the blocks of 16."""
+    from ninfer_amd.parts.moe import Routing
+    logits = torch.randn(t, e, generator=gen, device="cuda")
+    n = t * k
+    i32 = lambda *s: torch.zeros(*s, device="cuda", dtype=torch.int32)
+    r = Routing(i32(t, k), torch.zeros(t, k, device="cuda"), i32(e + 1), i32(n),
+                i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2), big_rows=64)
+    ops.moe_route(logits, e, k, False, r)
+    hh = rnd((n, inner), torch.bfloat16, gen)
+    wd = rnd((e, h, inner), torch.bfloat16, gen, 0.2)
+    x2, w2 = rnd((t, inner), torch.bfloat16, gen), rnd((h, inner), torch.bfloat16, gen, 0.2)
+    outs = []
+    for two in (0, 1):
+        ops.lib.ninfer_set_skinny_two(two, ctypes.c_long(1))
+        try:
+            y = torch.zeros(n, h, device="cuda", dtype=torch.bfloat16)
+            ops.grouped_down(hh, wd, r.offsets, r.order, y, tiles=r)
+            y_pair = torch.zeros_like(y)
+            dense = torch.zeros(t, h, device="cuda", dtype=torch.bfloat16)
+            with ops.together():
+                ops.grouped_down(hh, wd, r.offsets, r.order, y_pair, tiles=r)
+                ops.linear(x2, w2, dense)
+            outs.append((y, y_pair, dense))
+        finally:
+            ops.lib.ninfer_set_skinny_two(1, ctypes.c_long(4096))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    y_ref = torch.zeros(n, h, device="cuda", dtype=torch.bfloat16)
+    PlainOps().grouped_down(hh, wd, r.offsets, r.order, y_ref)
+    close(outs[1][0], y_ref, torch.bfloat16, scale=math.sqrt(inner) * 0.2)
+    assert torch.equal(outs[1][0], outs[1][1])
