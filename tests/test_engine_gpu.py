@@ -293,6 +293,16 @@ def test_long_prompt_on_the_many_row_kernels(wide_case, dtype):
     torch.testing.assert_close(got["c"], ref[600:624], **bound(dtype), msg=lambda m: f"decode c: {m}")
     torch.testing.assert_close(got["d"], ref[333:357], **bound(dtype), msg=lambda m: f"decode d: {m}")
     assert any(e["graph"] is not None for e in runner._graphs.values())
+    # a decoded token of one request beside a long portion of another in one step: the single
+    # row on the split-context kernel, the portion on the prompt kernel
+    runner = load_model(dirs[dtype], EngineOptions(dtype=dtype, max_context=704, prefill_chunk=640,
+                                                   num_sequences=2, page_size=16))
+    steps = [([("e", toks[:500], [])], []),
+             ([("f", toks[:300], [299]), ("e", [toks[500]], [0])], []),
+             ([("e", [toks[501]], [0]), ("f", toks[300:640], list(range(340)))], ["e", "f"])]
+    got = util.run_schedule(runner, steps)
+    torch.testing.assert_close(got["e"], ref[500:502], **bound(dtype), msg=lambda m: f"mixed e: {m}")
+    torch.testing.assert_close(got["f"], ref[299:640], **bound(dtype), msg=lambda m: f"mixed f: {m}")
 
 
 @pytest.mark.parametrize("seed", [0, 10, 16, 28, 35])
