@@ -305,6 +305,78 @@ def test_long_prompt_on_the_many_row_kernels(wide_case, dtype):
     torch.testing.assert_close(got["f"], ref[299:640], **bound(dtype), msg=lambda m: f"mixed f: {m}")
 
 
+@pytest.mark.parametrize("model,layers", [("a2.7b", 2), ("57b-a14b", 1)])
+def test_benchmark_shapes_bf16_stays_near_32bit(model, layers):
+    """A layer or two at the benchmark's layer sizes (hidden 2048, 16 heads of 128, 60 experts
+    top-4 of 1408, shared expert 5632; and hidden 3584, 28 heads over 4 kv heads, 64 experts
+    top-8 of 2560, shared expert 20480; vocabulary 151936), the same bf16-rounded random weights
+    in both precisions: the bf16 engine's steps (a 2,048-token prompt on the 256-row tiles, short
+    prompts, decoding at batch 40, 8 and 1 from replayed graphs, a token beside a long
+    portion) stay near the 32-bit path's, whose kernels are the plain ones. With 60 experts and
+    a random router some rows' routing differs between the precisions (they are left out of
+    the bound on single logits, and the bound is coarse): a kernel that is wrong at these sizes
+    is off by the size of the logits themselves."""
+    from bench import MODELS
+    from ninfer_amd import Chunk, EngineOptions
+    from ninfer_amd.engine.runner import ModelRunner
+    from ninfer_amd.loading import build_spec
+    from ninfer_amd.parts.moe import SparseMoE
+    from ninfer_amd.weights import RandomSource
+    raw = dict(MODELS[model][1], num_hidden_layers=layers)
+    vocab = raw["vocab_size"]
+    runners = {}
+    for dtype in ("float32", "bfloat16"):
+        _, spec = build_spec(raw)
+        source = RandomSource(spec.tensor_specs(), 99, torch.bfloat16, device="cuda")
+        runners[dtype] = ModelRunner(spec, source, EngineOptions(
+            dtype=dtype, max_context=2304, prefill_chunk=2048, num_sequences=41, page_size=16,
+            use_graph=dtype == "bfloat16"))
+    slots = {d: {} for d in runners}
+    same_routing = [0, 0]
+
+    def both(entries, label):
+        out = {}
+        for dtype, r in runners.items():
+            for name, _, _ in entries:
+                if name not in slots[dtype]:
+                    slots[dtype][name] = r.open()
+            logits = r.step([Chunk(slots[dtype][n], t, w) for n, t, w in entries])
+            ids = [b.feed_forward.last_ids.sort(dim=1).values.cpu() for b in r.spec.blocks
+                   if isinstance(b.feed_forward, SparseMoE)]
+            out[dtype] = (logits.float().cpu(), ids)
+        (a, ia), (b, ib) = out["float32"], out["bfloat16"]
+        same = torch.ones(ia[0].shape[0], dtype=torch.bool)
+        for x, y in zip(ia, ib):
+            same &= (x == y).all(dim=1)
+        same_routing[0] += int(same.sum())
+        same_routing[1] += same.numel()
+        # the rows whose logits were asked for, as rows of the step (entries keep their order here)
+        wanted, first = [], 0
+        for _, t, w in entries:
+            wanted += [first + i for i in w]
+            first += len(t)
+        diff = (a - b).abs()
+        alike = same[wanted]
+        assert float(a.abs().max()) > 2.0, f"{label}: the logits are of size 1 and more"
+        assert float(diff.mean()) < 0.06, f"{label}: mean {float(diff.mean()):.4f}"
+        if alike.any():   # a row that routes alike in both is close everywhere
+            assert float(diff[alike].max()) < 0.25, f"{label}: max {float(diff[alike].max()):.4f}"
+
+    toks = util.random_tokens(2048, vocab, 1)
+    both([("a", toks, list(range(2040, 2048)))], "prompt of 2048")
+    short = [util.random_tokens(32, vocab, 10 + i) for i in range(39)]
+    for i in range(0, 39, 13):
+        both([(f"s{j}", short[j], [31]) for j in range(i, i + 13)], "13 prompts of 32")
+    for batch in (40, 40, 8, 8, 8, 1, 1, 1):
+        nxt = util.random_tokens(batch, vocab, 100 + batch + same_routing[1])
+        both([("a", [nxt[0]], [0])] + [(f"s{j}", [nxt[j + 1]], [0]) for j in range(batch - 1)],
+             f"decode at batch {batch}")
+    nxt = util.random_tokens(600, vocab, 400)
+    both([("s0", [nxt[0]], [0]), ("s1", nxt[1:600], [598])], "a token beside a portion of 599")
+    assert same_routing[0] > 0.8 * same_routing[1], "most rows route alike in both precisions"
+    assert any(e["graph"] is not None for e in runners["bfloat16"]._graphs.values())
+
+
 @pytest.mark.parametrize("seed", [0, 10, 16, 28, 35])
 def test_random_configurations(tmp_path, seed):
     """Configurations drawn at random (head sizes that only the plain kernels take, heads in
