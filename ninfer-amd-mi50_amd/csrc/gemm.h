@@ -101,7 +101,7 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream);
 bool gemm_tile_takes(const GemmArgs& a);
 int gemm_tile(const GemmArgs& a, hipStream_t stream);
 int gemm_generic(const GemmArgs& a, hipStream_t stream);
-// Dense products of 33 to 128 rows whose output tiles are too few to fill the GPU: cut
+// Dense products of 33 to 512 rows whose output tiles are too few to fill the GPU: cut
 // along K over more blocks, partial sums in the workspace, then added up in a fixed order.
 int gemm_split_parts(const GemmArgs& a);   // parts the product would be cut into (< 2: not cut)
 int gemm_split(const GemmArgs& a, hipStream_t stream);

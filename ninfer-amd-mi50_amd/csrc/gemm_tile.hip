@@ -280,17 +280,21 @@ __global__ void sum_parts_kernel(const float* __restrict__ ws, int parts, int M,
   store_quad(out + (int64_t)m * ldc + n, v);
 }
 
-// The cut along K pays where 64 x 128 tiles of the output are fewer than the CUs, K is
-// long, and the weights are many enough (48 MB and more) that their stream outweighs the
-// second launch that adds the parts up (measured: 41 against 99 us for the library's product
-// at 64 rows, 3584 x 20480; no gain at 25 MB). Parts so that about two blocks per CU
-// exist, each with at least four k tiles, and no part is empty.
+// The cut along K pays where the tiles of the output (64 x 128, or 128 x 128 beyond 128 rows)
+// are fewer than the CUs, K is long, and the weights are many enough (48 MB and more) that
+// their stream outweighs the second launch that adds the parts up (measured against the
+// library's product at 3584 x 20480: 41 against 99 us at 64 rows, 111 against 226 at 512;
+// no gain at 25 MB; at 8192 x 8192 and 384 rows the library is faster, hence K >= 2 N beyond
+// 128 rows). Parts so that about two blocks per CU exist, each with at least four k tiles,
+// and no part is empty.
 int gemm_split_parts(const GemmArgs& a) {
   if (a.offsets || a.epilogue != kEpilogueNone || !a.workspace || !gemm_tile_takes(a)) return 1;
-  if (a.M <= 32 || a.M > 128 || a.N % 4 || a.ldc % 4 || ((uintptr_t)a.C & 15)) return 1;
+  if (a.M <= 32 || a.M > 512 || a.N % 4 || a.ldc % 4 || ((uintptr_t)a.C & 15)) return 1;
   if ((int64_t)a.N * a.K * 2 < g_split_min_bytes) return 1;
+  if (a.M > 128 && a.K < 2 * a.N) return 1;   // beyond 128 rows only where K is long against N
   const int cus = 256, tk = 64;
-  const int tiles = ((a.M + 63) / 64) * ((a.N + 127) / 128), nk = a.K / tk;
+  const int tm = a.M > 128 ? 128 : 64;
+  const int tiles = ((a.M + tm - 1) / tm) * ((a.N + 127) / 128), nk = a.K / tk;
   if (tiles >= cus) return 1;
   const int64_t fit = a.workspace_floats / ((int64_t)a.M * a.N);
   int parts = (int)min((int64_t)min(min(16, 2 * cus / tiles), nk / 4), fit);
@@ -308,7 +312,8 @@ int gemm_split(const GemmArgs& a, hipStream_t stream) {
   b.out_dtype = kF32;
   b.bias = nullptr;
   b.k_parts = parts;
-  int rc = launch_tile<64, 128, 64, 4, 2, 2>(b, stream);
+  int rc = a.M > 128 ? launch_tile<128, 128, 64, 4, 2, 2>(b, stream)
+                     : launch_tile<64, 128, 64, 4, 2, 2>(b, stream);
   if (rc) return rc;
   const int64_t quads = (int64_t)a.M * (a.N / 4);
   const unsigned blocks = (unsigned)((quads + 255) / 256);

@@ -110,6 +110,7 @@ class HipOps:
         # the activation in its epilogue beats the library's product followed by a kernel for
         # the activation (measured at 33, 64 and 128 rows: 70 against 98 us at 40960 x 3584)
         self.library_min_rows_fused = 128
+        self.split_max_rows = 512   # most rows of a product that may be cut along K (gemm_split)
         self._attn_ws = None
         self._outgrown = []     # workspaces that captured graphs may still point to
         self._split_ws = None   # 32 MB of 32-bit scratch for products cut along K, made at first use
@@ -334,7 +335,7 @@ class HipOps:
             _dev(bias, "bias", torch.float32, 1)
             _need(bias.shape[0] == w.shape[0], "linear: bias has the wrong size")
         if self._use_library(x, out) and bias is None:
-            if x.shape[0] > self.library_min_rows_fused or not self._gemm(
+            if x.shape[0] > self.split_max_rows or not self._gemm(
                     x, w, out, m=x.shape[0], n=w.shape[0], k=x.shape[1], only_if_split=True):
                 torch.matmul(x, w.t(), out=out)
             return

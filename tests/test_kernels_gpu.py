@@ -145,9 +145,10 @@ def test_tile_product_every_tile_height(ops, gen, variant, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(33, 2048, 5632), (64, 3584, 20480), (100, 300, 512),
-                                   (128, 2048, 2048), (64, 136, 4096), (40, 6144, 1024)])
+                                   (128, 2048, 2048), (64, 136, 4096), (40, 6144, 1024),
+                                   (300, 520, 2048), (512, 3584, 20480), (129, 128, 1024)])
 def test_linear_cut_along_k(ops, gen, m, n, k):
-    """Dense bf16 products of 33 to 128 rows whose output tiles would not fill the GPU are cut
+    """Dense bf16 products of 33 to 512 rows whose output tiles would not fill the GPU are cut
     along K over more blocks and summed in a fixed order: against the plain product, the
     same result twice, and (the sizes say so) cut indeed."""
     x, w = rnd((m, k), torch.bfloat16, gen), rnd((n, k), torch.bfloat16, gen)
