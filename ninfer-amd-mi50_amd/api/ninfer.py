@@ -75,7 +75,8 @@ class Ninfer:
     def __init__(self, model_dir: Optional[str] = None, max_context: int = 32768,
                  prefill_chunk: int = 512, num_sequences: int = 1, dtype: str = "bfloat16",
                  page_size: int = 16, num_pages: Optional[int] = None, use_graph: bool = False,
-                 random_config: Optional[dict] = None, random_seed: int = 0):
+                 random_config: Optional[dict] = None, random_seed: int = 0,
+                 random_weights_dtype: Optional[str] = None):
         self.options = EngineOptions(dtype=dtype, max_context=max_context,
                                      prefill_chunk=prefill_chunk, num_sequences=num_sequences,
                                      page_size=page_size, num_pages=num_pages,
@@ -83,7 +84,8 @@ class Ninfer:
         if model_dir is not None:
             self.runner = load_model(model_dir, self.options)
         elif random_config is not None:
-            self.runner = random_model(random_config, random_seed, self.options)
+            self.runner = random_model(random_config, random_seed, self.options,
+                                       weights_dtype=random_weights_dtype)
         else:
             raise ValueError("give a model folder or a configuration for random weights")
         self.sampler = Sampler(self.runner.ops, self.runner.device)

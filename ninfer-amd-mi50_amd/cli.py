@@ -2,7 +2,7 @@
 (src/apps/ninfer.cpp:55-119). Option names and meanings are the reference's
 where it has them: --max-context, --prefill-chunk, --max-new, --temperature
 (0 = greedy), --top-k, --top-p, --repeat-penalty, --seed,
---graph, --log-level. Prompts are token ids (there is no tokenizer here):
+--graph, --verify (here against the 32-bit path), --log-level. Prompts are token ids (there is no tokenizer here):
 --prompt-ids, --prompt-file, --random-prompts. Generated ids go to stdout, one
 line per request; diagnostics go to stderr (src/apps/ninfer.cpp:1-2). An
 unknown option is an error (:114-116). Without a prompt it is the reference's
@@ -37,6 +37,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--repeat-penalty", type=float, default=1.05)
     ap.add_argument("--seed", type=int, default=0, help="sampling seed (0: 1234 for a one-shot run, a fresh one per turn of the loop)")
     ap.add_argument("--graph", action="store_true", help="replay decode steps from a HIP graph")
+    ap.add_argument("--verify", action="store_true",
+                    help="generate again in the 32-bit path and report where the outputs part")
     ap.add_argument("--log-level", choices=["debug", "info", "warn", "error"], default="info")
     ap.add_argument("--dtype", choices=["bf16", "fp32", "bfloat16", "float32"], default="bf16")
     ap.add_argument("--random-weights", type=int, metavar="SEED",
@@ -94,10 +96,40 @@ def main(argv: Optional[List[str]] = None) -> int:
             print(",".join(map(str, o)))
         n = sum(len(o) for o in outs)
         log(f"{n} tokens in {dt:.2f} s ({n / max(dt, 1e-9):.1f} tok/s)")
+        if args.verify:
+            _verify(args, raw, common, prompts, params, stop, outs)
     except Exception as e:  # the reference exits 1 with the message (src/apps/ninfer.cpp:234-237)
         print(f"ninfer: error: {e}", file=sys.stderr)
         return 1
     return 0
+
+
+def _verify(args, raw, common, prompts, params, stop, outs) -> None:
+    """The reference's --verify runs the prompt again on one GPU as the golden output and
+    reports where the two-GPU output parts from it (src/apps/ninfer.cpp:137-176). Here the
+    golden run is the 32-bit path of the same model, with the same sampling seed."""
+    from .api.ninfer import Ninfer
+    if common["dtype"] == "float32":
+        print("[ninfer] verify: the run was in 32-bit already", file=sys.stderr)
+        return
+    golden = dict(common, dtype="float32", use_graph=False)
+    if args.random_weights is not None:   # the same values, rounded as the first run's were
+        eng = Ninfer(random_config=raw, random_seed=args.random_weights,
+                     random_weights_dtype=common["dtype"], **golden)
+    else:
+        eng = Ninfer(args.model_dir, **golden)
+    want = eng.generate(prompts, params, stop)
+    same = True
+    for r, (a, b) in enumerate(zip(outs, want)):
+        if a != b:
+            same = False
+            i = next((j for j, (x, y) in enumerate(zip(a, b)) if x != y), min(len(a), len(b)))
+            print(f"[ninfer] verify: request {r} parts from the 32-bit output at token {i} "
+                  f"({len(a)} / {len(b)} tokens); rounding noise of bfloat16 is expected where "
+                  f"two tokens are nearly as likely", file=sys.stderr)
+    if same:
+        print(f"[ninfer] verify: PASS, the outputs equal the 32-bit path's "
+              f"({sum(len(o) for o in outs)} tokens)", file=sys.stderr)
 
 
 def _interactive(eng, args, stop) -> int:

@@ -151,6 +151,13 @@ def test_command_line(model_dirs):
     answers = [[int(x) for x in l.split(",")] for l in proc.stdout.strip().splitlines()]
     first = plain_model.greedy_generate(w, cfg, prompt, 5)
     assert answers == [first, plain_model.greedy_generate(w, cfg, prompt + first + second, 5)]
+    # --verify: the same prompts again in the 32-bit path, and a line that says how they compare
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "ninfer"), model_dirs["A"]["bfloat16"],
+         "--prompt-ids", ",".join(map(str, prompt)), "--max-new", "4", "--temperature", "0",
+         "--max-context", "64", "--verify"], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "verify:" in proc.stderr
     bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "ninfer"), d, "--no-such-flag"],
                          capture_output=True, text=True, timeout=120)
     assert bad.returncode != 0
