@@ -164,6 +164,12 @@ def test_linear_cut_along_k(ops, gen, m, n, k):
         else:
             ops._gemm(x, w, o3, m=m, n=n, k=k, only_if_split=True)
         assert torch.equal(o1, o3)
+        # with a bias and a 32-bit result (the adding-up kernel's other forms)
+        bias = torch.randn(n, generator=gen, device="cuda")
+        f1, f2 = torch.empty(m, n, device="cuda"), torch.empty(m, n, device="cuda")
+        assert ops._gemm(x, w, f1, m=m, n=n, k=k, bias=bias, only_if_split=True)
+        PlainOps().linear(x, w, f2, bias=bias)
+        close(f1, f2, torch.float32, scale=200 * math.sqrt(k))
     finally:
         ops.lib.ninfer_set_split_min_bytes(ctypes.c_longlong(48 << 20))
     if n * k * 2 < (48 << 20):   # by default only long weight streams are cut
