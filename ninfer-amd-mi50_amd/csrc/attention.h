@@ -35,6 +35,7 @@ struct AttnArgs {
                             // 0 .. single_rows - 1 (0 when the caller does not sort them)
 };
 
+int attention_check(const AttnArgs& a);
 int attention_generic(const void* q, int q_stride, const void* kpool, const void* vpool,
                       const int* block_table, int bt_stride, const int* positions,
                       const int* row_seq, void* out, int T, int Hq, int Hkv, int D, int page_size,
@@ -43,6 +44,7 @@ int attention_generic(const void* q, int q_stride, const void* kpool, const void
 int64_t attention_decode_workspace_floats(int T, int Hq, int D, int max_kv_len);
 bool attention_decode_takes(const AttnArgs& a);
 int attention_decode(const AttnArgs& a, hipStream_t stream);
+void attention_decode_plan(const AttnArgs& a, bool* heads, int* chunk, int* n_chunks);
 bool attention_decode_heads_takes(const AttnArgs& a);
 int attention_decode_heads(const AttnArgs& a, int chunk, int n_chunks, hipStream_t stream);
 bool attention_prefill_takes(const AttnArgs& a);

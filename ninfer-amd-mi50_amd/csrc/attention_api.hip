@@ -3,9 +3,10 @@
 
 using namespace ninfer;
 
-// force_generic != 0 runs the plain one-wave-per-(row, head) kernel whatever
-// the shape (tests compare the fast kernels with it).
-extern "C" int ninfer_paged_attention(const AttnArgs* a, int force_generic, hipStream_t stream) {
+namespace ninfer {
+// What every kernel of the family assumes of the arguments.
+int attention_check(const AttnArgs& args) {
+  const AttnArgs* a = &args;
   NINFER_REQUIRE(a->T > 0 && a->S > 0, "paged_attention: T=%d S=%d must be positive", a->T, a->S);
   NINFER_REQUIRE(a->Hq > 0 && a->Hkv > 0 && a->Hq % a->Hkv == 0,
                  "paged_attention: %d query heads are not a multiple of %d kv heads", a->Hq,
@@ -22,6 +23,14 @@ extern "C" int ninfer_paged_attention(const AttnArgs* a, int force_generic, hipS
   NINFER_REQUIRE(a->max_qlen >= 1 && a->max_kv_len >= 1, "paged_attention: bad size hints");
   NINFER_REQUIRE(a->single_rows >= 0 && a->single_rows <= a->S && a->single_rows <= a->T,
                  "paged_attention: %d single rows of %d requests", a->single_rows, a->S);
+  return 0;
+}
+}  // namespace ninfer
+
+// force_generic != 0 runs the plain one-wave-per-(row, head) kernel whatever
+// the shape (tests compare the fast kernels with it).
+extern "C" int ninfer_paged_attention(const AttnArgs* a, int force_generic, hipStream_t stream) {
+  if (int rc = attention_check(*a)) return rc;
   if (!force_generic && a->max_qlen == 1 && attention_decode_takes(*a))
     return attention_decode(*a, stream);
   if (!force_generic && a->single_rows > 0 && a->single_rows < a->S &&
@@ -53,4 +62,18 @@ extern "C" int ninfer_paged_attention(const AttnArgs* a, int force_generic, hipS
 // 32-bit floats of workspace the split-KV decode kernel needs for this shape.
 extern "C" long long ninfer_attention_workspace_floats(int T, int Hq, int D, int max_kv_len) {
   return attention_decode_workspace_floats(T, Hq, D, max_kv_len);
+}
+
+// How a step of single-token rows would run (nothing is launched): kernel 0 = the plain
+// kernel, 1 = split contexts on scalar FMAs, 2 = split contexts on the matrix cores (grouped
+// heads); the keys per chunk and the number of chunks the merge kernel adds up. Tests name
+// the kernel variant they mean to reach with it.
+extern "C" int ninfer_attention_decode_plan(const AttnArgs* a, int* kernel, int* chunk, int* n_chunks) {
+  *kernel = 0;
+  *chunk = *n_chunks = 0;
+  if (!attention_decode_takes(*a)) return 0;
+  bool heads;
+  attention_decode_plan(*a, &heads, chunk, n_chunks);
+  *kernel = heads ? 2 : 1;
+  return 0;
 }

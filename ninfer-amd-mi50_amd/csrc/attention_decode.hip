@@ -287,25 +287,34 @@ static void launch_decode_chunk(const AttnArgs& a, int chunk, int n_chunks, hipS
     launch_decode<LPK, 256>(a, n_chunks, stream);
 }
 
-int attention_decode(const AttnArgs& a, hipStream_t stream) {
-  int chunk = decode_chunk(a.T, a.Hkv, a.max_kv_len);
-  if (attention_decode_heads_takes(a)) {
+// Which pass-1 kernel a decode step runs and how it cuts the contexts: the matrix-core
+// kernel for grouped heads (`heads`) or the scalar one, chunks of `chunk` keys.
+void attention_decode_plan(const AttnArgs& a, bool* heads, int* chunk, int* n_chunks) {
+  *heads = attention_decode_heads_takes(a);
+  *chunk = decode_chunk(a.T, a.Hkv, a.max_kv_len);
+  if (*heads) {
     // the matrix-core kernel has a start-up of several tiles: the largest chunk that still
     // gives every CU two blocks
-    chunk = 128;
+    *chunk = 128;
     for (int c = 1024; c > 128; c /= 2)
       if ((long)a.T * a.Hkv * ((a.max_kv_len + c - 1) / c) >= 512) {
-        chunk = c;
+        *chunk = c;
         break;
       }
   }
-  const int n_chunks = (a.max_kv_len + chunk - 1) / chunk;
+  *n_chunks = (a.max_kv_len + *chunk - 1) / *chunk;
+}
+
+int attention_decode(const AttnArgs& a, hipStream_t stream) {
+  bool heads;
+  int chunk, n_chunks;
+  attention_decode_plan(a, &heads, &chunk, &n_chunks);
   NINFER_REQUIRE(a.workspace_floats >= attention_decode_workspace_floats(a.T, a.Hq, a.D, a.max_kv_len),
                  "paged_attention: workspace of %lld floats is too small", (long long)a.workspace_floats);
   const size_t merge_lds = (2 * (size_t)n_chunks + kMergeThreads) * sizeof(float);
   NINFER_REQUIRE(merge_lds <= 48 * 1024, "paged_attention: a context of %d keys has too many chunks to merge",
                  a.max_kv_len);
-  if (attention_decode_heads_takes(a)) {
+  if (heads) {
     // three or more query heads per kv head: their products go to the matrix cores
     if (int rc = attention_decode_heads(a, chunk, n_chunks, stream)) return rc;
   } else {

@@ -467,9 +467,11 @@ class HipOps:
 
     # ---- attention ------------------------------------------------------------------
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,
-                        page_size, window, scale, out):
+                        page_size, window, scale, out, plan_only=False):
         """Attention of the rows' query heads (the first n_q * head_dim columns
-        of `qkv`) over their requests' cached keys and values."""
+        of `qkv`) over their requests' cached keys and values. `plan_only`: launch
+        nothing and say how a step of single-token rows of this shape would run
+        (which split-context kernel, keys per chunk, chunks)."""
         _dev(qkv, "qkv", dims=2)
         _dev(k_pool, "k_pool", qkv.dtype, 4)
         _dev(v_pool, "v_pool", qkv.dtype, 4)
@@ -504,6 +506,13 @@ class HipOps:
             ctx.seq_row_start.data_ptr(), ctx.seq_qlen.data_ptr(), ctx.seq_pos0.data_ptr(),
             ws, ws_floats, qkv.shape[1], block_table.shape[1], t, ctx.S, n_q, n_kv, head_dim, page_size,
             int(window or 0), float(scale), _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len, single)
+        if plan_only:
+            kernel, chunk, n_chunks = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+            self._ok(self.lib.ninfer_attention_decode_plan(
+                ctypes.byref(args), ctypes.byref(kernel), ctypes.byref(chunk),
+                ctypes.byref(n_chunks)))
+            return {"kernel": ("plain", "scalar", "heads")[kernel.value], "chunk": chunk.value,
+                    "chunks": n_chunks.value}
         self._ok(self.lib.ninfer_paged_attention(ctypes.byref(args),
                                                  1 if self.force_generic else 0, self._stream()))
 
