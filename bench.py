@@ -108,9 +108,9 @@ def main() -> int:
     runner = random_model(raw, 1234, opt)
     torch.cuda.synchronize()
     print(f"[bench] model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
-    for kp, vp in runner.cache.pools.values():   # a cache full of synthetic keys and values
-        kp.normal_()
-        vp.normal_()
+    for pools in runner.cache.pools.values():   # a cache full of synthetic keys and values
+        for pool in pools.values():
+            pool.normal_()
     sampler = Sampler(runner.ops, runner.device)
     gen = torch.Generator().manual_seed(7)
     greedy = SamplingParams.greedy()

@@ -76,11 +76,13 @@ class Ninfer:
                  prefill_chunk: int = 512, num_sequences: int = 1, dtype: str = "bfloat16",
                  page_size: int = 16, num_pages: Optional[int] = None, use_graph: bool = False,
                  random_config: Optional[dict] = None, random_seed: int = 0,
-                 random_weights_dtype: Optional[str] = None):
+                 random_weights_dtype: Optional[str] = None, kv_bytes: Optional[int] = None,
+                 check_pages: bool = False):
         self.options = EngineOptions(dtype=dtype, max_context=max_context,
                                      prefill_chunk=prefill_chunk, num_sequences=num_sequences,
                                      page_size=page_size, num_pages=num_pages,
-                                     use_graph=use_graph)
+                                     use_graph=use_graph, kv_bytes=kv_bytes,
+                                     check_pages=check_pages)
         if model_dir is not None:
             self.runner = load_model(model_dir, self.options)
         elif random_config is not None:
@@ -116,13 +118,36 @@ class Ninfer:
     @property
     def kv_total_bytes(self) -> int:
         c = self.runner.cache
-        return sum(k.numel() * k.element_size() * 2 for k, _ in c.pools.values())
+        return sum(t.numel() * t.element_size() for pools in c.pools.values()
+                   for t in pools.values())
 
     def kv_pages(self) -> Dict[str, int]:
         c = self.runner.cache
         return {"total": sum(g.allocator.num_pages for g in c.groups),
                 "free": sum(g.allocator.free_pages for g in c.groups),
                 "reused": c.pages_reused()}
+
+    def tensor_names(self) -> List[str]:
+        return self.runner.tensor_names()
+
+    def tensor_read(self, name: str, offset: int = 0, count: Optional[int] = None) -> np.ndarray:
+        """`count` numbers (all by default) from flat index `offset` of the checkpoint tensor
+        `name` as the engine holds it now, as 32-bit floats: what an outside check needs to
+        know of a model whose weights were generated on the device."""
+        flat = self.runner.tensor(name).reshape(-1)
+        end = flat.numel() if count is None else offset + count
+        if not 0 <= offset <= end <= flat.numel():
+            raise ValueError(f"{name}: [{offset}, {end}) is outside its {flat.numel()} numbers")
+        return flat[offset:end].float().cpu().numpy()
+
+    def close(self) -> None:
+        """Give the engine's device memory back (weights, cache, captured graphs)."""
+        import gc
+        import torch
+        self.runner = None
+        self.sampler = None
+        gc.collect()
+        torch.cuda.empty_cache()
 
     # ---- sessions -------------------------------------------------------------------
     def session(self) -> Session:

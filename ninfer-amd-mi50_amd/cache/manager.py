@@ -4,8 +4,9 @@ slots of fixed-size per-request state.
 Layers whose mixers need the same span of the past form a *group*: all keys
 (window None) or the last `window` positions. A group has its own page ids,
 allocator and block tables; every cache instance (one per plan entry that
-writes keys and values) in the group has its own pools, indexed by the
-group's page ids. A request holds one *slot*: its row in every group's block
+writes keys and values) in the group has its own pools (any number, named,
+each with a per-token shape and dtype of its own), indexed by the group's
+page ids. A request holds one *slot*: its row in every group's block
 table and its row of the state tensor.
 
 Pages are given back when a request is released and, in a window group, as
@@ -70,7 +71,7 @@ class CacheManager:
             g.rows = np.full((max_seqs, self.max_pages_per_request), -1, dtype=np.int32)
         self._free_slots: List[int] = list(range(max_seqs - 1, -1, -1))
         self._length: Dict[int, int] = {}
-        self.pools: Dict[int, Tuple[object, object]] = {}
+        self.pools: Dict[int, Dict[str, object]] = {}   # cache instance -> pool name -> tensor
         self.state = None
         # debugging: pages given back are filled with NaN in every pool of their group, so
         # that a read of a page that is no longer held (or of a slot not yet written in a page
@@ -78,15 +79,27 @@ class CacheManager:
         self.poison_freed = False
 
     # ---- device memory -----------------------------------------------------
-    def allocate_pools(self, device, dtype) -> None:
+    def allocate_pools(self, device, dtype, ops=None) -> None:
+        """Device memory of every pool, [pages, *outer, page_size, *inner] in the pool's own
+        dtype (the activation dtype `dtype` where it names none), and the state tensor.
+        `ops` (the kernel library) fills freed pages with NaN when poisoning is on."""
         import torch
+        self._ops = ops
+        named = {"float32": torch.float32, "bfloat16": torch.bfloat16}
         for i, need in enumerate(self.needs):
             if need is None:
                 continue
             n = self.groups[self.group_of_instance[i]].allocator.num_pages
-            shape = (n, need.kv_heads, self.page_size, need.head_dim)
-            self.pools[i] = (torch.zeros(shape, dtype=dtype, device=device),
-                             torch.zeros(shape, dtype=dtype, device=device))
+            self.pools[i] = {}
+            for spec in need.pools:
+                if spec.name in self.pools[i]:
+                    raise ValueError(f"a mixer names two pools {spec.name!r}")
+                if spec.dtype is not None and spec.dtype not in named:
+                    raise ValueError(f"pool {spec.name!r}: dtype {spec.dtype!r} is not one of "
+                                     f"{sorted(named)}")
+                shape = (n, *spec.outer, self.page_size, *spec.inner)
+                self.pools[i][spec.name] = torch.zeros(
+                    shape, dtype=named[spec.dtype] if spec.dtype else dtype, device=device)
         self.state = torch.zeros((self.max_seqs, max(self.state_floats, 1)),
                                  dtype=torch.float32, device=device)
 
@@ -125,10 +138,12 @@ class CacheManager:
         if self.poison_freed and pages and self.pools:
             import torch
             for i in g.instances:
-                k_pool, v_pool = self.pools[i]
-                idx = torch.tensor(pages, dtype=torch.int64, device=k_pool.device)
-                k_pool.index_fill_(0, idx, float("nan"))
-                v_pool.index_fill_(0, idx, float("nan"))
+                for pool in self.pools[i].values():
+                    idx = torch.tensor(pages, dtype=torch.int32, device=pool.device)
+                    if getattr(self, "_ops", None) is not None:
+                        self._ops.fill_nan_pages(pool, idx)
+                    else:   # no kernel library (host tests)
+                        pool.index_fill_(0, idx.long(), float("nan"))
 
     def length(self, slot: int) -> int:
         return self._length[slot]
@@ -209,8 +224,11 @@ class CacheManager:
 
     # ---- introspection -------------------------------------------------------
     def kv_bytes_per_token(self, bytes_per_element: int) -> int:
-        return sum(2 * n.kv_heads * n.head_dim * bytes_per_element
-                   for n in self.needs if n is not None)
+        """Bytes of paged cache one token takes over all cache instances; pools without a
+        dtype of their own count `bytes_per_element` per number."""
+        own = {"float32": 4, "bfloat16": 2}
+        return sum(p.elements_per_token() * (own[p.dtype] if p.dtype else bytes_per_element)
+                   for n in self.needs if n is not None for p in n.pools)
 
     def pages_total(self, group: int = 0) -> int:
         return self.groups[group].allocator.num_pages

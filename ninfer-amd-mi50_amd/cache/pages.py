@@ -61,6 +61,9 @@ class PageAllocator:
             self._free.append(p)
         self.freed += len(pages)
 
+    def is_held(self, page: int) -> bool:
+        return 0 <= page < self.num_pages and self._held[page]
+
     def check(self) -> None:
         """Every page is either free or held, never both, never twice."""
         assert len(set(self._free)) == len(self._free), "a page is on the free list twice"

@@ -22,7 +22,7 @@ from typing import List, Optional
 
 
 def build_parser() -> argparse.ArgumentParser:
-    ap = argparse.ArgumentParser(prog="ninfer", description="Qwen2-MoE generation on one MI355X")
+    ap = argparse.ArgumentParser(prog="ninfer", description="generation with a model folder's architecture on one MI355X")
     ap.add_argument("model_dir", help="folder with config.json (and model.safetensors)")
     ap.add_argument("--prompt-ids", action="append", default=[],
                     help="a prompt as comma-separated token ids (may be given several times)")
@@ -45,6 +45,8 @@ def build_parser() -> argparse.ArgumentParser:
                     help="fill the model with seeded random weights (needs only config.json)")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--kv-pages", type=int, help="pages per cache group")
+    ap.add_argument("--kv-gib", type=float, help="size of the paged cache over all layers, in GiB "
+                    "(instead of --kv-pages; default: room for --max-seqs requests of --max-context)")
     ap.add_argument("--max-seqs", type=int, default=8, help="most live requests")
     ap.add_argument("--eos-id", type=int, help="stop token (default: config.json eos_token_id)")
     return ap
@@ -69,19 +71,23 @@ def main(argv: Optional[List[str]] = None) -> int:
     if args.prompt_file:
         with open(args.prompt_file) as f:
             prompts += [list(map(int, p)) for p in json.load(f)]
-    if args.random_prompts:
-        rng = random.Random(args.seed or 1234)
-        for n in args.random_prompts.split(","):
-            prompts.append([rng.randrange(raw["vocab_size"]) for _ in range(int(n))])
+    if args.kv_pages is not None and args.kv_gib is not None:
+        print("ninfer: error: give --kv-pages or --kv-gib, not both", file=sys.stderr)
+        return 1
     t0 = time.time()
     common = dict(max_context=args.max_context, prefill_chunk=args.prefill_chunk,
                   num_sequences=args.max_seqs, dtype=dtype, page_size=args.page_size,
-                  num_pages=args.kv_pages, use_graph=args.graph)
+                  num_pages=args.kv_pages, use_graph=args.graph,
+                  kv_bytes=int(args.kv_gib * (1 << 30)) if args.kv_gib is not None else None)
     try:
         if args.random_weights is not None:
             eng = Ninfer(random_config=raw, random_seed=args.random_weights, **common)
         else:
             eng = Ninfer(args.model_dir, **common)
+        if args.random_prompts:   # the vocabulary is the bound model's, whatever its config calls it
+            rng = random.Random(args.seed or 1234)
+            for n in args.random_prompts.split(","):
+                prompts.append([rng.randrange(eng.vocab) for _ in range(int(n))])
         log(f"engine ready in {time.time() - t0:.1f} s: vocab={eng.vocab} ctx={args.max_context} "
             f"chunk={args.prefill_chunk} seqs={args.max_seqs} dtype={dtype}")
         stop = [args.eos_id] if args.eos_id is not None else None
@@ -97,6 +103,8 @@ def main(argv: Optional[List[str]] = None) -> int:
         n = sum(len(o) for o in outs)
         log(f"{n} tokens in {dt:.2f} s ({n / max(dt, 1e-9):.1f} tok/s)")
         if args.verify:
+            eng.close()   # the golden engine takes the first one's place: never both at once
+            del eng
             _verify(args, raw, common, prompts, params, stop, outs)
     except Exception as e:  # the reference exits 1 with the message (src/apps/ninfer.cpp:234-237)
         print(f"ninfer: error: {e}", file=sys.stderr)
@@ -113,6 +121,11 @@ def _verify(args, raw, common, prompts, params, stop, outs) -> None:
         print("[ninfer] verify: the run was in 32-bit already", file=sys.stderr)
         return
     golden = dict(common, dtype="float32", use_graph=False)
+    if golden.get("num_pages") is None and golden.get("kv_bytes") is None:
+        # the 32-bit cache takes twice the bytes per token: room for these prompts is enough
+        per = max(len(p) for p in prompts) + params.max_new_tokens
+        golden["num_pages"] = (-(-per // golden["page_size"]) + 1) * min(len(prompts),
+                                                                        golden["num_sequences"])
     if args.random_weights is not None:   # the same values, rounded as the first run's were
         eng = Ninfer(random_config=raw, random_seed=args.random_weights,
                      random_weights_dtype=common["dtype"], **golden)

@@ -17,9 +17,11 @@ class EngineOptions:
     prefill_chunk: int = 512       # token budget of one step (reference --prefill-chunk)
     num_sequences: int = 8         # most live requests (reference num_sequences)
     page_size: int = 16            # tokens per cache page
-    num_pages: Optional[int] = None  # pages per cache group; None: enough for every request at max_context
+    num_pages: Optional[int] = None  # pages per cache group; None: from kv_bytes, else enough for every request at max_context
+    kv_bytes: Optional[int] = None   # bytes of paged cache over all layers (the reference sizes its slabs in bytes, src/api/ninfer_c_api.cpp:105-108)
     use_graph: bool = False        # replay decode-only steps from a captured HIP graph
     poison_freed_pages: bool = False  # debugging: fill pages that are given back with NaN
+    check_pages: bool = False      # debugging: before every step, check on the host that every page the step reads or writes is held by its request and by no other
     device: str = "cuda:0"
 
     def validate(self) -> None:
@@ -30,11 +32,23 @@ class EngineOptions:
                 raise ValueError(f"{name} must be >= 1, got {getattr(self, name)}")
         if self.num_pages is not None and self.num_pages < 1:
             raise ValueError(f"num_pages must be >= 1, got {self.num_pages}")
+        if self.kv_bytes is not None and self.kv_bytes < 1:
+            raise ValueError(f"kv_bytes must be >= 1, got {self.kv_bytes}")
+        if self.kv_bytes is not None and self.num_pages is not None:
+            raise ValueError("give num_pages or kv_bytes, not both")
 
     def pages_per_request(self) -> int:
         return -(-self.max_context // self.page_size)
 
-    def pool_pages(self) -> int:
+    def pool_pages(self, bytes_per_token: int = 0) -> int:
+        """Pages of every cache group. `bytes_per_token`: what one token takes in the paged
+        cache over all layers (needed only with kv_bytes)."""
         if self.num_pages is not None:
             return self.num_pages
+        if self.kv_bytes is not None:
+            pages = self.kv_bytes // max(1, bytes_per_token * self.page_size)
+            if pages < 1:
+                raise ValueError(f"kv_bytes {self.kv_bytes} holds no page of {self.page_size} "
+                                 f"tokens ({bytes_per_token} bytes a token)")
+            return int(pages)
         return self.pages_per_request() * self.num_sequences

@@ -29,10 +29,11 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kDecWaves = 4;
 
-// Keys per block: 256, or 128 when that many blocks would leave the GPU idle.
+// Keys per block: 256, or 128 when that many blocks (fewer than four a CU) would leave the
+// GPU idle.
 static int decode_chunk(int T, int Hkv, int max_kv_len) {
   long blocks = (long)T * Hkv * ((max_kv_len + 255) / 256);
-  return blocks < 1024 ? 128 : 256;
+  return blocks < 4L * device_cu_count() ? 128 : 256;
 }
 
 __device__ __forceinline__ void cvt8(const bf16x8& v, float* f) {
@@ -297,7 +298,7 @@ void attention_decode_plan(const AttnArgs& a, bool* heads, int* chunk, int* n_ch
     // gives every CU two blocks
     *chunk = 128;
     for (int c = 1024; c > 128; c /= 2)
-      if ((long)a.T * a.Hkv * ((a.max_kv_len + c - 1) / c) >= 512) {
+      if ((long)a.T * a.Hkv * ((a.max_kv_len + c - 1) / c) >= 2L * device_cu_count()) {
         *chunk = c;
         break;
       }

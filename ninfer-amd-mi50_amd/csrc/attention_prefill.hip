@@ -91,8 +91,8 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
     // see the most keys, come first.
     const int total = gridDim.x * gridDim.y;
     const int id = blockIdx.x + gridDim.x * blockIdx.y;
-    const int x = id % 8, q = total / 8, rem8 = total % 8;
-    const int w = x * q + min(x, rem8) + id / 8;   // a bijection: x < rem8 own one id more
+    const int x = id % kXcds, q = total / kXcds, rem8 = total % kXcds;
+    const int w = x * q + min(x, rem8) + id / kXcds;   // a bijection: x < rem8 own one id more
     h = w / gridDim.x;
     const int tile = gridDim.x - 1 - w % gridDim.x;
     if (!find_tile(a.seq_row_start, a.S, PQ, tile, tile_info)) return;

@@ -22,6 +22,10 @@ template <> __device__ __forceinline__ float from_f32<float>(float v) { return v
 template <> __device__ __forceinline__ bf16 from_f32<bf16>(float v) { return __float2bfloat16(v); }
 
 constexpr int kWave = 64;
+// gfx950 (the one target) has 8 XCDs, each with an L2 of its own; the hardware deals
+// workgroups to them in turn (block id mod 8). Kernels that share operands through L2 map
+// block ids to work with this number.
+constexpr int kXcds = 8;
 
 // Butterfly reductions over the 64 lanes of a wave: offsets 32 -> 1.
 __device__ __forceinline__ float wave_sum(float v) {
@@ -57,6 +61,10 @@ __device__ __forceinline__ void lds_barrier() {
 }
 
 int set_error(int code, const char* fmt, ...);
+
+// Compute units of the current device (asked once per device; 256 if the runtime cannot
+// say). Launch heuristics count blocks against it.
+int device_cu_count();
 
 #define NINFER_REQUIRE(cond, ...)                         \
   do {                                                    \

@@ -165,7 +165,8 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delt
 // One block per row of the fused q|k|v activations. Adds the bias, rotates q
 // heads in place and k heads on their way into the page; v heads are copied.
 // Pairs are (i, i + rot/2) within the first `rot` dims of a head (reference
-// src/ops/kernels.hip:86-91, full rotation there); dims >= rot pass through.
+// src/ops/kernels.hip:86-91, full rotation there), or neighbours (2i, 2i + 1)
+// when `interleaved`; pair i turns by pos * inv_freq[i]; dims >= rot pass through.
 // A work item is one rotating pair or one pass-through element, read and
 // written by one thread, so q can be rewritten in place without a barrier.
 // Page lookup: logical page pos / page_size of the row's request.
@@ -176,7 +177,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
                                      const float* __restrict__ inv_freq, int rot, int Hq, int Hkv,
                                      int D, T* __restrict__ kpool, T* __restrict__ vpool,
                                      const int* __restrict__ block_table, int bt_stride,
-                                     int page_size, int write_kv) {
+                                     int page_size, int write_kv, int interleaved) {
   const int t = blockIdx.x;
   const int half = rot >> 1;
   const int per_head = half + (D - rot);          // items of a rotated head
@@ -194,8 +195,8 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
     int d0, d1 = -1;                               // element(s) of this item
     float v0, v1 = 0.f;
     if (i < half) {
-      d0 = i;
-      d1 = i + half;
+      d0 = interleaved ? 2 * i : i;
+      d1 = interleaved ? 2 * i + 1 : i + half;
       v0 = to_f32(row[base + d0]) + (bias ? bias[base + d0] : 0.f);
       v1 = to_f32(row[base + d1]) + (bias ? bias[base + d1] : 0.f);
       if (is_q || is_k) {
@@ -422,7 +423,8 @@ extern "C" int ninfer_rope_kv_write(void* qkv, const float* bias, const int* pos
                                     const int* row_seq, const float* inv_freq, int rot_dim, int Hq,
                                     int Hkv, int D, void* kpool, void* vpool,
                                     const int* block_table, int bt_stride, int page_size,
-                                    int write_kv, int T, int dtype, hipStream_t stream) {
+                                    int write_kv, int interleaved, int T, int dtype,
+                                    hipStream_t stream) {
   NINFER_REQUIRE(T > 0, "rope_kv_write: T=%d must be positive", T);
   NINFER_REQUIRE(D > 0 && D <= 1024, "rope_kv_write: head size %d not in [1,1024]", D);
   NINFER_REQUIRE(rot_dim >= 0 && rot_dim <= D && rot_dim % 2 == 0,
@@ -431,7 +433,8 @@ extern "C" int ninfer_rope_kv_write(void* qkv, const float* bias, const int* pos
   NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "rope_kv_write: unknown dtype %d", dtype);
   NINFER_REQUIRE(page_size > 0 && bt_stride > 0, "rope_kv_write: bad page size or table width");
   // many rows of a shape that takes 8-element accesses: one block per row, vectorised
-  const bool vec_ok = (rot_dim / 2) % 8 == 0 && (D - rot_dim) % 8 == 0 && D % 8 == 0 &&
+  // (half-split pairs only: neighbouring pairs stay on the kernel of single items)
+  const bool vec_ok = !interleaved && (rot_dim / 2) % 8 == 0 && (D - rot_dim) % 8 == 0 && D % 8 == 0 &&
                       ((uintptr_t)qkv % 32 == 0) && ((uintptr_t)kpool % 32 == 0) &&
                       ((uintptr_t)vpool % 32 == 0);
   if (T >= 256 && vec_ok) {
@@ -455,11 +458,11 @@ extern "C" int ninfer_rope_kv_write(void* qkv, const float* bias, const int* pos
   if (dtype == kF32)
     rope_kv_write_kernel<float><<<grid, block, 0, stream>>>(
         (float*)qkv, bias, positions, row_seq, inv_freq, rot_dim, Hq, Hkv, D, (float*)kpool,
-        (float*)vpool, block_table, bt_stride, page_size, write_kv);
+        (float*)vpool, block_table, bt_stride, page_size, write_kv, interleaved);
   else
     rope_kv_write_kernel<bf16><<<grid, block, 0, stream>>>(
         (bf16*)qkv, bias, positions, row_seq, inv_freq, rot_dim, Hq, Hkv, D, (bf16*)kpool,
-        (bf16*)vpool, block_table, bt_stride, page_size, write_kv);
+        (bf16*)vpool, block_table, bt_stride, page_size, write_kv, interleaved);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

@@ -13,6 +13,19 @@ int set_error(int code, const char* fmt, ...) {
   va_end(ap);
   return code;
 }
+
+int device_cu_count() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
 }  // namespace ninfer
 
 extern "C" const char* ninfer_last_error() { return ninfer::g_error; }

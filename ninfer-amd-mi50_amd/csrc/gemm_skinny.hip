@@ -255,7 +255,7 @@ static SkinnyPlan plan_skinny(const GemmArgs& a) {
   // features per block: 16, or for a dense product with few tiles the count that makes the
   // blocks a whole multiple of the CUs
   p.rows = 16;
-  const int cus = 256;
+  const int cus = device_cu_count();
   if (!a.offsets && m_tiles == 1 && blocks < 8 * cus) {
     const int per_cu = (a.N + 16 * cus - 1) / (16 * cus);          // blocks each CU gets
     p.rows = (a.N + per_cu * cus - 1) / (per_cu * cus);
@@ -264,7 +264,7 @@ static SkinnyPlan plan_skinny(const GemmArgs& a) {
     const long per_cu = ((long)a.N * m_tiles + 16 * cus - 1) / (16 * cus);
     p.rows = (int)(((long)a.N * m_tiles + per_cu * cus - 1) / (per_cu * cus));
   }
-  p.waves = (blocks < 512 && chunks >= 16) ? 16 : (blocks < 2048 && chunks >= 8) ? 8 : 4;
+  p.waves = (blocks < 2 * cus && chunks >= 16) ? 16 : (blocks < 8 * cus && chunks >= 8) ? 8 : 4;
   // a grouped product without SwiGLU whose tiles are many and short (K small): two feature
   // sets per block, so that blocks are half as many and each does twice the work
   p.two = g_skinny_two && a.offsets && a.epilogue == kEpilogueNone && p.rows == 16 && p.waves == 4 &&

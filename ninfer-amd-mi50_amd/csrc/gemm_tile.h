@@ -28,8 +28,8 @@ __device__ inline void block_to_tile(bool grouped, int& bx, int& by) {
   const int total = gridDim.x * gridDim.y;
   const int id = blockIdx.x + gridDim.x * blockIdx.y;
   // ids congruent to x mod 8 number total / 8 (one more for x < total % 8): a bijection
-  const int x = id % 8, q = total / 8, rem8 = total % 8;
-  const int w = x * q + min(x, rem8) + id / 8;
+  const int x = id % kXcds, q = total / kXcds, rem8 = total % kXcds;
+  const int w = x * q + min(x, rem8) + id / kXcds;
   const int nt = gridDim.y, mt = gridDim.x;
   const int chunk = w / (4 * nt), rem = w % (4 * nt);
   const int full = mt / 4;   // chunks of four row tiles; the rest is walked one by one

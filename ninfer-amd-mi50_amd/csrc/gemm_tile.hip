@@ -250,7 +250,7 @@ int gemm_tile(const GemmArgs& a, hipStream_t stream) {
   } else {
     const int n_units = a.epilogue == kEpilogueSwiGLU ? 2 * a.N : a.N;   // W rows
     auto blocks = [&](int tm, int tn) { return ((a.M + tm - 1) / tm) * ((n_units + tn - 1) / tn); };
-    const int cus = 256;
+    const int cus = device_cu_count();
     rows = blocks(256, 256) >= cus ? 256 : blocks(128, 128) >= cus ? 128 : 64;
     if (a.M <= 64) rows = 64;           // and no taller than the rows there are
     else if (a.M <= 128 && rows > 128) rows = 128;
@@ -292,7 +292,7 @@ int gemm_split_parts(const GemmArgs& a) {
   if (a.M <= 32 || a.M > 512 || a.N % 4 || a.ldc % 4 || ((uintptr_t)a.C & 15)) return 1;
   if ((int64_t)a.N * a.K * 2 < g_split_min_bytes) return 1;
   if (a.M > 128 && a.K < 2 * a.N) return 1;   // beyond 128 rows only where K is long against N
-  const int cus = 256, tk = 64;
+  const int cus = device_cu_count(), tk = 64;
   const int tm = a.M > 128 ? 128 : 64;
   const int tiles = ((a.M + tm - 1) / tm) * ((a.N + 127) / 128), nk = a.K / tk;
   if (tiles >= cus) return 1;

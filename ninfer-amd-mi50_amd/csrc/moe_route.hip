@@ -48,10 +48,14 @@ __device__ __forceinline__ int route_row(const float* __restrict__ row, int E, i
     sum += p[i];
   }
   sum = wave_sum(sum);
+  // A row with a NaN or an infinite logit has no softmax. The choice stays total all the
+  // same (every probability counts as 0, so the first k experts are taken: ids are always
+  // valid indices) and the weights come out NaN, so the fault stays visible downstream.
+  const bool bad = !(sum > 0.f && sum < INFINITY);
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
     int e = lane + i * 64;
-    p[i] = e < E ? p[i] / sum : -1.f;  // -1 marks "not a candidate"
+    p[i] = e < E ? (bad ? 0.f : p[i] / sum) : -1.f;  // -1 marks "not a candidate"
   }
   float chosen_sum = 0.f, my_w = 0.f;
   int my_id = 0;
@@ -86,7 +90,7 @@ __device__ __forceinline__ int route_row(const float* __restrict__ row, int E, i
   }
   if (lane < k) {
     ids[lane] = my_id;
-    wts[lane] = renorm ? my_w / chosen_sum : my_w;
+    wts[lane] = bad ? __builtin_nanf("") : (renorm ? my_w / chosen_sum : my_w);
   }
   return my_id;
 }
@@ -103,7 +107,8 @@ __device__ void align_block(const int* ids, int n, int E, int* __restrict__ offs
                             int* __restrict__ tiles64, int* __restrict__ tile_counts, int big, int* cnt) {
   for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
   __syncthreads();
-  for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cnt[ids[i]], 1);
+  // ids from outside this file are clamped into [0, E): never an index out of bounds
+  for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cnt[min(max(ids[i], 0), E - 1)], 1);
   __syncthreads();
   if (threadIdx.x < 64) {
     // the first wave scans 64 experts at a time: rows, 16-row tiles, 64-row tiles
@@ -146,7 +151,8 @@ __device__ void align_block(const int* ids, int n, int E, int* __restrict__ offs
     }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < n; i += blockDim.x) order[atomicAdd(&cnt[ids[i]], 1)] = i;
+  for (int i = threadIdx.x; i < n; i += blockDim.x)
+    order[atomicAdd(&cnt[min(max(ids[i], 0), E - 1)], 1)] = i;
 }
 
 __global__ void moe_align_kernel(const int* __restrict__ ids, int n, int E,

@@ -160,9 +160,10 @@ extern "C" int ninfer_qkv_rope(const QkvRopeArgs* args, hipStream_t stream) {
   NINFER_REQUIRE(blocks < (1L << 31), "qkv_rope: %ld blocks are too many", blocks);
   dim3 grid((unsigned)blocks, m_tiles);
   const int chunks = a.K / 128;
-  if (blocks * m_tiles < 256 && chunks >= 16)
+  const int cus = device_cu_count();
+  if (blocks * m_tiles < cus && chunks >= 16)
     qkv_rope_kernel<16><<<grid, 16 * 64, 0, stream>>>(a, pairs);
-  else if (blocks * m_tiles < 2048 && chunks >= 8)
+  else if (blocks * m_tiles < 8 * cus && chunks >= 8)
     qkv_rope_kernel<8><<<grid, 8 * 64, 0, stream>>>(a, pairs);
   else
     qkv_rope_kernel<4><<<grid, 4 * 64, 0, stream>>>(a, pairs);

@@ -51,7 +51,9 @@ class ModelRunner:
             ops = load_ops()
         self.ops = ops
         check_tensors(source.shapes(), spec.tensor_specs(), where, spec.unused_tensor_specs())
-        spec.bind(WeightBinder(source, self.device, self.act_dtype))
+        binder = WeightBinder(source, self.device, self.act_dtype)
+        spec.bind(binder)
+        self._held = binder.held
 
         # one cache instance per plan entry that writes keys and values
         needs = []
@@ -63,14 +65,30 @@ class ModelRunner:
             n = mixer.state_floats()
             self._state_range.append(slice(floats, floats + n) if n else None)
             floats += n
-        self.cache = CacheManager(needs, options.page_size, options.pool_pages(),
+        own = {"float32": 4, "bfloat16": 2}
+        per_token = sum(p.elements_per_token() * own[p.dtype or options.dtype]
+                        for n in needs if n is not None for p in n.pools)
+        self.cache = CacheManager(needs, options.page_size, options.pool_pages(per_token),
                                   options.num_sequences, options.max_context, floats)
-        self.cache.allocate_pools(self.device, self.act_dtype)
+        self.cache.allocate_pools(self.device, self.act_dtype, ops=self.ops)
         self.cache.poison_freed = options.poison_freed_pages
         self.vocab_size = spec.vocab_size
         self.steps_run = 0
         self._graphs: Dict[tuple, dict] = {}
         self.graph_context_step = 1024   # a graph serves contexts up to the next multiple
+
+    # ---- read-back -------------------------------------------------------------
+    def tensor_names(self) -> List[str]:
+        return sorted(self._held)
+
+    def tensor(self, name: str) -> torch.Tensor:
+        """The checkpoint tensor `name` as the engine holds it now: a view of the
+        device memory its kernels read (a slice of a fused or stacked tensor
+        where parts fuse), in the dtype it is kept in. For tests and tools that
+        have to know what a model generated on the device holds."""
+        if name not in self._held:
+            raise KeyError(f"the model holds no tensor named {name!r}")
+        return self._held[name]
 
     # ---- requests --------------------------------------------------------------
     def open(self) -> int:
@@ -140,6 +158,8 @@ class ModelRunner:
             max_kv_len = min(-(-max_kv_len // self.graph_context_step) * self.graph_context_step,
                              cache.max_pages_per_request * cache.page_size)
         tables = [cache.block_table(g, slots, width) for g in range(len(cache.groups))]
+        if self.options.check_pages:
+            self._check_pages(chunks, pos0, tables)
         parts = [tokens, positions, row_seq, np.asarray(slots, np.int32), row_start, qlen,
                  np.asarray(pos0, np.int32), np.asarray(want_rows, np.int32)]
         parts += [t.reshape(-1) for t in tables]
@@ -158,6 +178,35 @@ class ModelRunner:
             cache.commit(c.slot, p + len(c.tokens))
         self.steps_run += 1
         return logits
+
+    def _check_pages(self, chunks: Sequence[Chunk], pos0: List[int], tables) -> None:
+        """Debugging: what the kernels assume of the step's block tables, checked on the host
+        before anything is launched. Every entry is -1 or a page of the pool; every position
+        the step writes, and every earlier one its rows can see, lies in a page that the
+        allocator counts as held; no page stands in two requests' rows. (The reference's
+        analogue is the overflow throw of its slab, src/runtime/kv_cache.cpp:35-37.)"""
+        ps = self.cache.page_size
+        for g, table in zip(self.cache.groups, tables):
+            owner: Dict[int, int] = {}
+            for i, (c, p) in enumerate(zip(chunks, pos0)):
+                row = table[i]
+                if ((row < -1) | (row >= g.allocator.num_pages)).any():
+                    raise RuntimeError(f"slot {c.slot}: block table holds a page outside "
+                                       f"[0, {g.allocator.num_pages}): {row.tolist()}")
+                lo = 0 if g.window is None else max(0, p - g.window + 1)
+                last = p + len(c.tokens) - 1
+                if last // ps >= row.shape[0]:
+                    raise RuntimeError(f"slot {c.slot}: position {last} is beyond the block "
+                                       f"table's {row.shape[0]} pages")
+                for lp in range(lo // ps, last // ps + 1):
+                    page = int(row[lp])
+                    if page < 0 or not g.allocator.is_held(page):
+                        raise RuntimeError(f"slot {c.slot}: positions {lp * ps}.. are read or "
+                                           f"written, but page {page} is not held")
+                for page in row[row >= 0].tolist():
+                    if owner.setdefault(page, c.slot) != c.slot:
+                        raise RuntimeError(f"page {page} stands in the block tables of slots "
+                                           f"{owner[page]} and {c.slot}")
 
     def _forward(self, dev: torch.Tensor, shape: dict) -> Optional[torch.Tensor]:
         """Run the model on the step described by the packed index buffer `dev`
@@ -222,8 +271,7 @@ class ModelRunner:
             view = None
             if owner in cache.pools:
                 g = cache.group_of_instance[owner]
-                k_pool, v_pool = cache.pools[owner]
-                view = CacheView(k_pool, v_pool, d_tables[g], cache.page_size,
+                view = CacheView(cache.pools[owner], d_tables[g], cache.page_size,
                                  cache.groups[g].window)
             rng = self._state_range[i]
             state = cache.state[:, rng] if rng is not None else None

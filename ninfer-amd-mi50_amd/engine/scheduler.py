@@ -18,8 +18,12 @@ Logits are asked for decode rows and for the portion that ends a prompt.
 When pages run out: a decode token or portion that cannot get its pages
 preempts the most recently admitted running request (its pages and slot are
 given back, it returns to the front of the waiting queue and later recomputes
-prompt + generated tokens); the oldest request is never preempted for a newer
-one. A request that could not fit even alone is finished with an error.
+prompt + generated tokens). Only requests that arrived after the one in need
+are preempted for it: an older request is never given back for a newer one,
+which waits instead (it brings no tokens to this step). A request that could
+not fit even alone is finished with an error; in a group of windowed layers
+"fit" means the window plus one step's portion, since older pages are given
+back as the window passes them.
 """
 from __future__ import annotations
 
@@ -123,6 +127,20 @@ class Scheduler:
     def _pages_for(self, req: Request, n: int) -> List[int]:
         return self.cache.pages_needed(req.slot, req.cached + n)
 
+    def _fits_alone(self, total: int) -> bool:
+        """Could a request of `total` tokens run with every page to itself? A group that
+        keeps all keys must hold them all; a windowed group never holds more than the window
+        and the portion of one step (pages the window has passed are given back after every
+        step), plus the two pages that the ends of that span may share with their neighbours."""
+        ps = self.cache.page_size
+        for g in self.cache.groups:
+            most = -(-total // ps)
+            if g.window is not None:
+                most = min(most, -(-(g.window + self.max_batch_tokens) // ps) + 2)
+            if most > g.allocator.num_pages:
+                return False
+        return True
+
     def plan(self) -> PlannedStep:
         """Decide the next step. Acquires slots for admitted requests and
         releases preempted ones; touches no pages."""
@@ -142,11 +160,11 @@ class Scheduler:
             return True
 
         def preempt_newest(keep: Request) -> bool:
-            """Give back the newest running request other than `keep` that is
-            not yet part of this step; false if there is none."""
+            """Give back the newest running request that arrived after `keep`
+            and is not yet part of this step; false if there is none."""
             planned = {id(c[0]) for c in chunks}
-            for victim in reversed(self.running):
-                if victim is keep or id(victim) in planned:
+            for victim in sorted(self.running, key=lambda r: -r.order):
+                if victim is keep or id(victim) in planned or victim.order < keep.order:
                     continue
                 for i, g in enumerate(cache.groups):
                     free[i] += sum(1 for p in g.tables[victim.slot] if p >= 0)
@@ -190,8 +208,7 @@ class Scheduler:
                 and cache.free_slots > 0 and not preempted:
             req = self.waiting[0]
             total = len(req.tokens)
-            if total > cache.max_context or -(-total // cache.page_size) > min(
-                    [g.allocator.num_pages for g in cache.groups] or [1 << 30]):
+            if total > cache.max_context or not self._fits_alone(total):
                 self.waiting.popleft()
                 req.status, req.error = "failed", "the request does not fit in the cache"
                 failed.append(req)

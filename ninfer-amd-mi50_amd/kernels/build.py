@@ -52,9 +52,26 @@ def _build_dirs() -> List[str]:
             os.path.join(tempfile.gettempdir(), f"ninfer_hip_build_{uid}")]
 
 
+def _trusted(d: str) -> bool:
+    """The in-tree folder is trusted as the sources beside it are. The fallback folder lies
+    in a place anyone can write to: it counts only if it is this user's own and nobody else
+    can write into it, so that no other user's library is ever loaded."""
+    if d == os.path.join(CSRC, "_build"):
+        return True
+    try:
+        st = os.lstat(d)
+    except OSError:
+        return False
+    import stat
+    return (stat.S_ISDIR(st.st_mode) and st.st_uid == os.getuid()
+            and not st.st_mode & (stat.S_IWGRP | stat.S_IWOTH))
+
+
 def _matching_library() -> Optional[str]:
     want = _fingerprint()
     for d in _build_dirs():
+        if not _trusted(d):
+            continue
         lib, stamp = os.path.join(d, LIB_NAME), os.path.join(d, "fingerprint")
         if os.path.isfile(lib) and os.path.isfile(stamp):
             with open(stamp) as f:
@@ -86,7 +103,9 @@ def build(force: bool = True, jobs: int = 8) -> str:
     out_dir = None
     for d in _build_dirs():
         try:
-            os.makedirs(d, exist_ok=True)
+            os.makedirs(d, mode=0o700, exist_ok=True)
+            if not _trusted(d):
+                continue
             with open(os.path.join(d, ".probe"), "w"):
                 pass
             os.remove(os.path.join(d, ".probe"))

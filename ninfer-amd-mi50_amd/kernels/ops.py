@@ -129,6 +129,29 @@ class HipOps:
         self._ok(self.lib.ninfer_device_info(ctypes.byref(cu), ctypes.byref(lds), arch, 128))
         return {"cu_count": cu.value, "lds_bytes": lds.value, "arch": arch.value.decode()}
 
+    # ---- fills --------------------------------------------------------------------
+    def fill_nan_pages(self, pool, pages):
+        """NaN into every number of the given pages of a pool [pages, ...] (debugging:
+        pages that were given back)."""
+        _dev(pool, "pool")
+        _dev(pages, "pages", torch.int32, 1)
+        _need(pool.dtype in _DT, f"fill_nan_pages: pool of {pool.dtype}")
+        per_page = pool.numel() // pool.shape[0]
+        self._ok(self.lib.ninfer_fill_nan_pages(
+            ctypes.c_void_p(pool.data_ptr()), ctypes.c_void_p(pages.data_ptr()), pages.shape[0],
+            pool.shape[0], ctypes.c_longlong(per_page), _DT[pool.dtype], self._stream()))
+
+    def fill_random(self, out, key, std, mean=0.0):
+        """out[i] = mean + std * z(key, i), z an approximately normal number that is a pure
+        function of the 64-bit key and the flat index (see weights/counter_random.py, which
+        computes the same bits on the host)."""
+        _dev(out, "out")
+        _need(out.dtype in _DT, f"fill_random: tensor of {out.dtype}")
+        self._ok(self.lib.ninfer_fill_random(
+            ctypes.c_void_p(out.data_ptr()), ctypes.c_longlong(out.numel()),
+            ctypes.c_ulonglong(key & ((1 << 64) - 1)), ctypes.c_float(std), ctypes.c_float(mean),
+            _DT[out.dtype], self._stream()))
+
     # ---- row-wise ---------------------------------------------------------------
     def embed(self, tokens, table, out):
         _dev(tokens, "tokens", torch.int32, 1)
@@ -185,7 +208,10 @@ class HipOps:
         return k, stride
 
     def rope_kv_write(self, qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv, head_dim,
-                      k_pool, v_pool, block_table, page_size, write_kv=True):
+                      k_pool, v_pool, block_table, page_size, write_kv=True, interleaved=False):
+        """Bias, rotation of q and k, and the write of k and v into pages. Pair i of the
+        first `rot_dim` dims of a head turns by pos * inv_freq[i]; the pairs are
+        (i, i + rot_dim / 2), or the neighbours (2i, 2i + 1) when `interleaved`."""
         _dev(qkv, "qkv", dims=2)
         t = qkv.shape[0]
         width = (n_q + 2 * n_kv) * head_dim
@@ -211,20 +237,23 @@ class HipOps:
             ctypes.c_void_p(_ptr(inv_freq) if rot_dim else None), rot_dim, n_q, n_kv, head_dim,
             ctypes.c_void_p(k_pool.data_ptr()), ctypes.c_void_p(v_pool.data_ptr()),
             ctypes.c_void_p(block_table.data_ptr()), block_table.shape[1], page_size,
-            1 if write_kv else 0, t, _DT[qkv.dtype], self._stream()))
+            1 if write_kv else 0, 1 if interleaved else 0, t, _DT[qkv.dtype], self._stream()))
 
     def qkv_rope(self, x, w_qkv, bias, qkv, positions, row_seq, inv_freq, rot_dim, n_q, n_kv,
-                 head_dim, k_pool, v_pool, block_table, page_size, write_kv=True):
+                 head_dim, k_pool, v_pool, block_table, page_size, write_kv=True,
+                 interleaved=False):
         """qkv = x w_qkv^T, then what `rope_kv_write` does. Few bf16 rows with a full
-        rotation run as one kernel; everything else as the product and the rotation
-        kernel one after the other."""
+        rotation in half-split pairs run as one kernel; everything else as the product
+        and the rotation kernel one after the other."""
         t = x.shape[0]
-        fused = (not self.force_generic and x.dtype == torch.bfloat16 and x.dim() == 2
+        fused = (not self.force_generic and not interleaved and x.dtype == torch.bfloat16
+                 and x.dim() == 2
                  and self.lib.ninfer_qkv_rope_takes(t, x.shape[1], x.shape[1], head_dim, rot_dim))
         if not fused:
             self.linear(x, w_qkv, qkv)
             self.rope_kv_write(qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv,
-                               head_dim, k_pool, v_pool, block_table, page_size, write_kv)
+                               head_dim, k_pool, v_pool, block_table, page_size, write_kv,
+                               interleaved)
             return
         width = (n_q + 2 * n_kv) * head_dim
         _dev(x, "x", torch.bfloat16, 2)

@@ -47,15 +47,17 @@ def load_model(model_dir: str, options: Optional[EngineOptions] = None, ops=None
 
 
 def random_model(raw_config: Dict[str, Any], seed: int, options: Optional[EngineOptions] = None,
-                 ops=None, weights_dtype: Optional[str] = None) -> ModelRunner:
+                 ops=None, weights_dtype: Optional[str] = None, std: float = 0.02) -> ModelRunner:
     """A runner with seeded random weights generated on the engine's device
     (for models too large to write to disk). `weights_dtype`: the precision the values are
     rounded to before the engine takes them (default: the engine's own), so that a 32-bit
-    engine can hold exactly the weights of a bfloat16 one."""
+    engine can hold exactly the weights of a bfloat16 one. The values are those that
+    `write_random_model` would store for the same configuration, seed and std, bit for bit;
+    `runner.tensor(name)` reads them back."""
     options = options or EngineOptions()
     cfg, spec = build_spec(raw_config)
     source = RandomSource(spec.tensor_specs(), seed, _DTYPES[weights_dtype or options.dtype],
-                          device=options.device)
+                          std=std, device=options.device, ops=ops)
     runner = ModelRunner(spec, source, options, ops=ops, where="random weights")
     runner.config = cfg
     return runner

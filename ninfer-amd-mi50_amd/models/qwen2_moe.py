@@ -9,37 +9,41 @@ Layer loop and tensor names: reference src/models/model.hip:509-583,
 """
 from __future__ import annotations
 
+from .. import parts  # noqa: F401  (registers the part factories by kind and name)
 from ..config.qwen2_moe import Qwen2MoeConfig
-from ..parts.attention import Attention
-from ..parts.block import PreNormBlock
 from ..parts.embedding import LMHead, TokenEmbedding
-from ..parts.mlp import SwiGLU
-from ..parts.moe import SparseMoE
-from ..parts.norm import RMSNorm
-from ..parts.rotary import Rotary
-from ..registry import register_architecture
+from ..registry import make_part, register_architecture
 from .spec import ModelSpec
 
 
 def build_qwen2_moe(cfg: Qwen2MoeConfig) -> ModelSpec:
+    """Every part of a layer is made by kind and name through the part registry, so a
+    builder of another architecture chooses other names (its own, registered from outside
+    the package, or these) layer by layer in the same way."""
     h = cfg.hidden_size
-    rotary = Rotary(cfg.head_dim, cfg.rope_theta)
+    rotary = make_part("position", "rotary", rot_dim=cfg.head_dim, theta=cfg.rope_theta)
     embedding = TokenEmbedding("model.embed_tokens.", cfg.vocab_size, h)
     blocks = []
     for l in range(cfg.num_hidden_layers):
         p = f"model.layers.{l}."
-        mixer = Attention(p + "self_attn.", h, cfg.num_attention_heads, cfg.num_key_value_heads,
-                          cfg.head_dim, rotary, qkv_bias=cfg.qkv_bias, window=cfg.layer_window(l))
+        mixer = make_part("mixer", "attention", prefix=p + "self_attn.", hidden=h,
+                          heads=cfg.num_attention_heads, kv_heads=cfg.num_key_value_heads,
+                          head_dim=cfg.head_dim, position=rotary, qkv_bias=cfg.qkv_bias,
+                          window=cfg.layer_window(l))
         if cfg.layer_is_sparse(l):
-            ff = SparseMoE(p + "mlp.", h, cfg.num_experts, cfg.num_experts_per_tok,
-                           cfg.moe_intermediate_size, cfg.norm_topk_prob,
-                           cfg.shared_expert_intermediate_size)
+            ff = make_part("feed_forward", "sparse_moe", prefix=p + "mlp.", hidden=h,
+                           experts=cfg.num_experts, top_k=cfg.num_experts_per_tok,
+                           inner=cfg.moe_intermediate_size, renorm=cfg.norm_topk_prob,
+                           shared_inner=cfg.shared_expert_intermediate_size)
         else:
-            ff = SwiGLU(p + "mlp.", h, cfg.intermediate_size)
-        blocks.append(PreNormBlock(RMSNorm(p + "input_layernorm.", h, cfg.rms_norm_eps), mixer,
-                                   RMSNorm(p + "post_attention_layernorm.", h, cfg.rms_norm_eps),
-                                   ff))
-    final_norm = RMSNorm("model.norm.", h, cfg.rms_norm_eps)
+            ff = make_part("feed_forward", "swiglu", prefix=p + "mlp.", hidden=h,
+                           inner=cfg.intermediate_size)
+        norm = lambda name: make_part("norm", "rmsnorm", prefix=p + name, size=h,
+                                      eps=cfg.rms_norm_eps)
+        blocks.append(make_part("block", "pre_norm", mixer_norm=norm("input_layernorm."),
+                                mixer=mixer, ff_norm=norm("post_attention_layernorm."),
+                                feed_forward=ff))
+    final_norm = make_part("norm", "rmsnorm", prefix="model.norm.", size=h, eps=cfg.rms_norm_eps)
     head = LMHead("lm_head.", cfg.vocab_size, h,
                   tied_to=embedding if cfg.tie_word_embeddings else None)
     return ModelSpec(embedding, blocks, final_norm, head, eos_token_id=cfg.eos_token_id)

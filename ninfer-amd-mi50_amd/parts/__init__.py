@@ -1,6 +1,6 @@
 from .attention import Attention
 from .base import (Block, CacheNeed, CacheView, CallInfo, FeedForward, Mixer, Norm, Part,
-                   PendingRows, PositionEncoding, StepContext, WeightBinder, settle)
+                   PendingRows, PoolSpec, PositionEncoding, StepContext, WeightBinder, settle)
 from .block import PreNormBlock
 from .embedding import LMHead, TokenEmbedding
 from .mlp import SwiGLU
@@ -9,6 +9,6 @@ from .norm import RMSNorm
 from .rotary import NoPosition, Rotary
 
 __all__ = ["Attention", "Block", "CacheNeed", "CacheView", "CallInfo", "FeedForward", "Mixer",
-           "Norm", "Part", "PendingRows", "settle", "PositionEncoding", "StepContext", "WeightBinder", "PreNormBlock",
+           "Norm", "Part", "PendingRows", "PoolSpec", "settle", "PositionEncoding", "StepContext", "WeightBinder", "PreNormBlock",
            "LMHead", "TokenEmbedding", "SwiGLU", "RoutedExperts", "SoftmaxTopKRouter",
            "SparseMoE", "RMSNorm", "NoPosition", "Rotary"]

@@ -45,7 +45,7 @@ class Attention(Mixer):
         return (self.heads + 2 * self.kv_heads) * self.head_dim
 
     def cache_need(self) -> Optional[CacheNeed]:
-        return CacheNeed(self.kv_heads, self.head_dim, self.window)
+        return CacheNeed.keys_values(self.kv_heads, self.head_dim, self.window)
 
     def children(self) -> List[Part]:
         return [self.position]
@@ -80,6 +80,9 @@ class Attention(Mixer):
         if self.qkv_bias:
             self.b_qkv = torch.cat([w.float32(p + "q_proj.bias"), w.float32(p + "k_proj.bias"),
                                     w.float32(p + "v_proj.bias")])
+            w.hold(p + "q_proj.bias", self.b_qkv[:nq])
+            w.hold(p + "k_proj.bias", self.b_qkv[nq:nq + nk])
+            w.hold(p + "v_proj.bias", self.b_qkv[nq + nk:])
         self.w_o = w.matrix(p + "o_proj.weight")
 
     def forward(self, ctx: StepContext, x, residual, call: CallInfo):
@@ -89,10 +92,11 @@ class Attention(Mixer):
         # the product, then bias, rotation of q and k, and the write of k, v into pages
         ops.qkv_rope(x, self.w_qkv, self.b_qkv, qkv, ctx.positions, ctx.row_seq,
                      self.position.table(), self.position.rot_dim, self.heads, self.kv_heads,
-                     self.head_dim, cache.k_pool, cache.v_pool, cache.block_table,
-                     cache.page_size, write_kv=call.writes_cache)
+                     self.head_dim, cache["k"], cache["v"], cache.block_table,
+                     cache.page_size, write_kv=call.writes_cache,
+                     interleaved=self.position.pairing == "interleaved")
         attn = ctx.empty((ctx.T, self.heads * self.head_dim))
-        ops.paged_attention(qkv, cache.k_pool, cache.v_pool, cache.block_table, ctx,
+        ops.paged_attention(qkv, cache["k"], cache["v"], cache.block_table, ctx,
                             self.heads, self.kv_heads, self.head_dim,
                             cache.page_size, self.window, self.scale, attn)
         out = ctx.empty((ctx.T, self.hidden))

@@ -10,7 +10,7 @@ which model it is in: it sees its own parameters, a name prefix, and a
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, List, Optional, Tuple
 
 import torch
 
@@ -18,25 +18,56 @@ from ..weights.source import TensorSpec
 
 
 @dataclass(frozen=True)
+class PoolSpec:
+    """One paged pool of a mixer: what it keeps per token under `name`.
+
+    The pool's tensor is [pages, *outer, page_size, *inner]: `outer` are the
+    dimensions a page is split by before its token slots (heads, for keys and
+    values), `inner` what one token holds in one of them (a head's numbers).
+    `dtype` None means the engine's activation dtype; 'float32' or 'bfloat16'
+    fix it."""
+    name: str
+    outer: Tuple[int, ...]
+    inner: Tuple[int, ...]
+    dtype: Optional[str] = None
+
+    def elements_per_token(self) -> int:
+        n = 1
+        for d in self.outer + self.inner:
+            n *= d
+        return n
+
+
+@dataclass(frozen=True)
 class CacheNeed:
-    """What a mixer needs of the paged cache for each token it has seen: keys
-    and values of `kv_heads` heads of `head_dim`, all of them (window None) or
-    only the last `window` positions."""
-    kv_heads: int
-    head_dim: int
+    """What a mixer needs of the paged cache for each token it has seen: any
+    number of named pools, each with a per-token shape and dtype of its own,
+    for all positions (window None) or only the last `window` of them. Mixers
+    with the same window share page numbers and block tables; each has pools
+    of its own."""
+    pools: Tuple[PoolSpec, ...]
     window: Optional[int] = None
+
+    @staticmethod
+    def keys_values(kv_heads: int, head_dim: int, window: Optional[int] = None) -> "CacheNeed":
+        """Keys and values of `kv_heads` heads of `head_dim`: pools 'k' and 'v',
+        each [pages, kv_heads, page_size, head_dim]."""
+        return CacheNeed((PoolSpec("k", (kv_heads,), (head_dim,)),
+                          PoolSpec("v", (kv_heads,), (head_dim,))), window)
 
 
 @dataclass
 class CacheView:
-    """One cache instance as a step sees it: the layer's page pools
-    [pages, kv_heads, page_size, head_dim] and the block table of the step's
+    """One cache instance as a step sees it: the mixer's pools by name (each
+    [pages, *outer, page_size, *inner]) and the block table of the step's
     requests [S, max_pages] (int32, -1 where a page was given back)."""
-    k_pool: torch.Tensor
-    v_pool: torch.Tensor
+    pools: Dict[str, torch.Tensor]
     block_table: torch.Tensor
     page_size: int
     window: Optional[int]
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        return self.pools[name]
 
 
 @dataclass
@@ -106,22 +137,35 @@ def settle(ctx: "StepContext", residual: torch.Tensor, pending) -> Optional[torc
 
 class WeightBinder:
     """Reads tensors by name from a weight source and places them on the
-    device: matrices in the compute dtype, gains and biases in 32-bit."""
+    device: matrices in the compute dtype, gains and biases in 32-bit. It keeps
+    a record name -> the device tensor (or the slice of a fused or stacked one)
+    that now holds that checkpoint tensor, so that what the engine holds can be
+    read back by checkpoint name."""
 
     def __init__(self, source: Any, device: torch.device, act_dtype: torch.dtype):
         self.source = source
         self.device = device
         self.act_dtype = act_dtype
+        self.held: Dict[str, torch.Tensor] = {}
+
+    def hold(self, name: str, where: torch.Tensor) -> None:
+        """Record (or correct, after a part has moved it) where a tensor lives."""
+        self.held[name] = where
 
     def matrix(self, name: str) -> torch.Tensor:
-        return self.source.read(name).to(device=self.device, dtype=self.act_dtype).contiguous()
+        t = self.source.read(name).to(device=self.device, dtype=self.act_dtype).contiguous()
+        self.held[name] = t
+        return t
 
     def float32(self, name: str) -> torch.Tensor:
-        return self.source.read(name).to(device=self.device, dtype=torch.float32).contiguous()
+        t = self.source.read(name).to(device=self.device, dtype=torch.float32).contiguous()
+        self.held[name] = t
+        return t
 
     def matrix_into(self, name: str, out: torch.Tensor) -> None:
         """Copy a matrix into a slice of a larger (fused or stacked) tensor."""
         out.copy_(self.source.read(name).to(device=self.device), non_blocking=False)
+        self.held[name] = out
 
 
 class Part:
@@ -181,9 +225,15 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    """A position encoding applied to queries and keys inside a mixer."""
+    """A position encoding applied to queries and keys inside a mixer: a
+    rotation of the first `rot_dim` dims of every head, pair i by the angle
+    pos * table()[i]. `pairing` says which dims form pair i: 'half' pairs
+    (i, i + rot_dim / 2), 'interleaved' the neighbours (2i, 2i + 1). The table
+    holds any frequencies (scaled per dimension or not); rot_dim 0 is no
+    rotation."""
 
     rot_dim: int = 0
+    pairing: str = "half"
 
     def table(self) -> Optional[torch.Tensor]:
         raise NotImplementedError
@@ -192,7 +242,8 @@ class PositionEncoding(Part):
 class Mixer(Part):
     """Mixes information between the positions of a request.
 
-    `cache_need()` says what it keeps per token in pages (None: nothing),
+    `cache_need()` says what it keeps per token in pages (None: nothing; else
+    named pools, each with its own per-token shape and dtype),
     `state_floats()` how many 32-bit numbers of fixed-size state it keeps per
     request (0: none). `forward` takes the normed rows [T, hidden] and returns
     rows [T, hidden] that the block adds to the residual.

@@ -168,6 +168,8 @@ class SparseMoE(FeedForward):
             self.router_and_gate = torch.cat([self.router.weight, self.shared_gate])
             self.router.weight = self.router_and_gate[:e]
             self.shared_gate = self.router_and_gate[e:]
+            w.hold(self.router.prefix + "weight", self.router.weight)
+            w.hold(self.prefix + "shared_expert_gate.weight", self.shared_gate)
 
     def forward(self, ctx: StepContext, x, residual):
         if self.shared is None:

@@ -1,4 +1,5 @@
-"""Rotary position encoding, half-split pairing (i, i + rot_dim/2).
+"""Rotary position encoding; half-split pairing (i, i + rot_dim/2) unless told
+`pairing="interleaved"` (neighbours 2i, 2i + 1).
 
 f_i = theta^(-2i/rot_dim), evaluated in double and rounded once to 32-bit
 (reference src/models/model.hip:635-642 builds the same table with std::pow);
@@ -18,10 +19,13 @@ from .base import PositionEncoding, WeightBinder
 
 
 class Rotary(PositionEncoding):
-    def __init__(self, rot_dim: int, theta: float):
+    def __init__(self, rot_dim: int, theta: float, pairing: str = "half"):
         if rot_dim % 2:
             raise ValueError(f"rotary dimension must be even, got {rot_dim}")
+        if pairing not in ("half", "interleaved"):
+            raise ValueError(f"pairing must be 'half' or 'interleaved', got {pairing!r}")
         self.rot_dim = rot_dim
+        self.pairing = pairing
         self.theta = float(theta)
         self._table: Optional[torch.Tensor] = None
 

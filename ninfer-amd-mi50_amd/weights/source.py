@@ -7,7 +7,6 @@ of `model.safetensors.index.json`'s `weight_map` if that file exists, else
 """
 from __future__ import annotations
 
-import hashlib
 import json
 import os
 from dataclasses import dataclass
@@ -73,37 +72,43 @@ class CheckpointSource:
 class RandomSource:
     """Seeded random tensors for a set of expected tensors.
 
-    Every tensor is drawn from its own generator, seeded by (seed, name), so a
-    tensor's values do not depend on which other tensors exist or on the order
-    they are asked for. Matrices and biases: N(0, std); gains: 1 + N(0, std).
-    On 'cpu' the values are those `write_random_model` stores; on a GPU device
-    the generator is the device's (other values, same distribution), which is
-    how models too large to write to disk are filled.
+    Every element is a pure function of (seed, tensor name, flat index): a
+    counter hash turned into an approximately normal number (the sum of twelve
+    uniform ones, see counter_random.py). Matrices and biases: std * z; gains:
+    1 + std * z. A tensor's values do not depend on which other tensors exist,
+    on the order they are asked for, or on where they are made: on 'cpu' the
+    host computes them, on a GPU device the library's fill kernel does, and
+    both give the same bits. That is how models too large to write to disk are
+    filled, and how a test can know what such a model holds.
     """
 
     def __init__(self, specs: Dict[str, TensorSpec], seed: int, dtype: torch.dtype,
-                 std: float = 0.02, device: str = "cpu"):
+                 std: float = 0.02, device: str = "cpu", ops=None):
         self.specs = specs
         self.seed = int(seed)
         self.dtype = dtype
         self.std = std
         self.device = device
+        self._ops = ops
 
     def shapes(self) -> Dict[str, Tuple[int, ...]]:
         return {n: s.shape for n, s in self.specs.items()}
 
     def read(self, name: str) -> torch.Tensor:
+        from . import counter_random
         if name not in self.specs:
             raise WeightError(f"missing tensor in checkpoint: {name}")
         spec = self.specs[name]
-        digest = hashlib.sha256(f"{self.seed}:{name}".encode("utf-8")).digest()
-        gen = torch.Generator(device=self.device)
-        gen.manual_seed(int.from_bytes(digest[:8], "little") & ((1 << 63) - 1))
-        t = torch.empty(spec.shape, dtype=torch.float32, device=self.device)
-        t.normal_(0.0, self.std, generator=gen)
-        if spec.role == "gain":
-            t += 1.0
-        return t.to(self.dtype)
+        key = counter_random.tensor_key(self.seed, name)
+        mean = 1.0 if spec.role == "gain" else 0.0
+        if torch.device(self.device).type == "cpu":
+            return counter_random.fill(spec.shape, key, self.std, mean).to(self.dtype)
+        if self._ops is None:
+            from ..kernels import load_ops
+            self._ops = load_ops()
+        t = torch.empty(spec.shape, dtype=self.dtype, device=self.device)
+        self._ops.fill_random(t, key, self.std, mean)
+        return t
 
     def close(self) -> None:
         pass

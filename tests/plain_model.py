@@ -149,16 +149,18 @@ def router(x: Tensor, wr: Tensor, top_k: int, renorm: bool) -> Tuple[Tensor, Ten
     t, e = p.shape
     ids = torch.empty(t, top_k, dtype=torch.long)
     wts = torch.empty(t, top_k, dtype=torch.float32)
-    for i in range(t):
-        row = p[i].clone()
-        for j in range(top_k):
-            best = 0
-            for c in range(1, e):
-                if row[c] > row[best]:
-                    best = c
-            ids[i, j] = best
-            wts[i, j] = row[best]
-            row[best] = -1.0
+    rows = torch.arange(t)
+    work = p.clone()
+    for j in range(top_k):
+        # a linear scan for the maximum, all rows at once; strictly greater replaces, so among
+        # equal probabilities the lowest index stays
+        best = torch.zeros(t, dtype=torch.long)
+        for c in range(1, e):
+            better = work[:, c] > work[rows, best]
+            best = torch.where(better, torch.full_like(best, c), best)
+        ids[:, j] = best
+        wts[:, j] = work[rows, best]
+        work[rows, best] = -1.0
     if renorm:
         wts = wts / wts.sum(dim=-1, keepdim=True)
     return ids, wts

@@ -26,6 +26,9 @@ class PlainOps:
         """Independent products: nothing to gain here, they run as they are called."""
         return contextlib.nullcontext()
 
+    def fill_nan_pages(self, pool, pages):
+        pool.index_fill_(0, pages.long(), float("nan"))
+
     def embed(self, tokens, table, out):
         out.copy_(_f(table[tokens.long()]))
 
@@ -49,13 +52,14 @@ class PlainOps:
         out.copy_((v * torch.rsqrt(ms + eps) * gain).to(out.dtype))
 
     def qkv_rope(self, x, w_qkv, bias, qkv, positions, row_seq, inv_freq, rot_dim, n_q, n_kv,
-                 head_dim, k_pool, v_pool, block_table, page_size, write_kv=True):
+                 head_dim, k_pool, v_pool, block_table, page_size, write_kv=True,
+                 interleaved=False):
         self.linear(x, w_qkv, qkv)
         self.rope_kv_write(qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv, head_dim,
-                           k_pool, v_pool, block_table, page_size, write_kv)
+                           k_pool, v_pool, block_table, page_size, write_kv, interleaved)
 
     def rope_kv_write(self, qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv, head_dim,
-                      k_pool, v_pool, block_table, page_size, write_kv=True):
+                      k_pool, v_pool, block_table, page_size, write_kv=True, interleaved=False):
         t = qkv.shape[0]
         x = _f(qkv)
         if bias is not None:
@@ -66,9 +70,14 @@ class PlainOps:
             phi = positions.to(torch.float32)[:, None] * inv_freq[None, :]
             c, s = torch.cos(phi)[:, None, :], torch.sin(phi)[:, None, :]
             qk = x[:, :n_q + n_kv, :]
-            x1, x2 = qk[..., :half].clone(), qk[..., half:rot_dim].clone()
-            qk[..., :half] = x1 * c - x2 * s
-            qk[..., half:rot_dim] = x1 * s + x2 * c
+            if interleaved:   # pair i is dims (2i, 2i + 1)
+                x1, x2 = qk[..., 0:rot_dim:2].clone(), qk[..., 1:rot_dim:2].clone()
+                qk[..., 0:rot_dim:2] = x1 * c - x2 * s
+                qk[..., 1:rot_dim:2] = x1 * s + x2 * c
+            else:             # pair i is dims (i, i + rot_dim / 2)
+                x1, x2 = qk[..., :half].clone(), qk[..., half:rot_dim].clone()
+                qk[..., :half] = x1 * c - x2 * s
+                qk[..., half:rot_dim] = x1 * s + x2 * c
         qkv.view(t, n_q + 2 * n_kv, head_dim)[:, :n_q] = x[:, :n_q].to(qkv.dtype)
         if not write_kv:
             return

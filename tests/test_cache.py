@@ -28,7 +28,7 @@ def test_allocator_is_lifo_and_counts_reuse():
 
 
 def manager(num_pages=16, window=None, page_size=4, seqs=4, max_context=64):
-    needs = [CacheNeed(2, 8, None), CacheNeed(2, 8, window)]
+    needs = [CacheNeed.keys_values(2, 8, None), CacheNeed.keys_values(2, 8, window)]
     return CacheManager(needs, page_size, num_pages, seqs, max_context, state_floats=0)
 
 
@@ -36,7 +36,7 @@ def test_groups_by_window():
     m = manager(window=8)
     assert [g.window for g in m.groups] == [None, 8]
     assert m.group_of_instance == {0: 0, 1: 1}
-    same = CacheManager([CacheNeed(2, 8), CacheNeed(4, 16), None], 4, 8, 2, 32)
+    same = CacheManager([CacheNeed.keys_values(2, 8), CacheNeed.keys_values(4, 16), None], 4, 8, 2, 32)
     assert len(same.groups) == 1 and same.groups[0].instances == [0, 1]
     assert same.kv_bytes_per_token(2) == 2 * (2 * 8 + 4 * 16) * 2
 

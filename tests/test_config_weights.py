@@ -286,3 +286,27 @@ def test_load_model_refuses_without_gpu_or_reports_bad_folder(model_dirs, tmp_pa
     if not torch.cuda.is_available():
         with pytest.raises(RuntimeError, match="no CPU path"):
             ninfer_amd.load_model(model_dirs["A"]["float32"])
+
+
+def test_random_weights_are_a_function_of_seed_name_and_index():
+    """Every element depends on (seed, tensor name, flat index) alone: a slice of a tensor
+    can be computed without the rest, another name or seed gives other numbers, and the
+    numbers have the moments of a normal distribution (they are sums of twelve uniform ones)."""
+    from ninfer_amd.weights import RandomSource, TensorSpec, counter_random
+    specs = {"a.weight": TensorSpec((300, 70)), "b.weight": TensorSpec((300, 70)),
+             "n.weight": TensorSpec((64,), "gain")}
+    src = RandomSource(specs, 7, torch.float32, std=0.5)
+    a = src.read("a.weight")
+    assert torch.equal(a, RandomSource({"a.weight": specs["a.weight"]}, 7, torch.float32, std=0.5).read("a.weight"))
+    key = counter_random.tensor_key(7, "a.weight")
+    part = counter_random.counter_normal(key, 1000, 50)
+    assert torch.equal(a.reshape(-1)[1000:1050], torch.from_numpy(part) * 0.5)
+    assert not torch.equal(a, src.read("b.weight"))
+    assert not torch.equal(a, RandomSource(specs, 8, torch.float32, std=0.5).read("a.weight"))
+    z = a / 0.5
+    assert abs(float(z.mean())) < 0.02 and abs(float(z.std()) - 1) < 0.02
+    assert abs(float((z ** 4).mean()) - 2.9) < 0.15 and float(z.abs().max()) <= 6.0
+    gain = src.read("n.weight")
+    assert abs(float(gain.mean()) - 1) < 0.3
+    bf = RandomSource(specs, 7, torch.bfloat16, std=0.5).read("a.weight")
+    assert torch.equal(bf, a.to(torch.bfloat16))

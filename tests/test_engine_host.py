@@ -157,3 +157,106 @@ def test_toy_routed_feed_forward_and_another_position_encoding(tmp_path):
     got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=4, max_live=3))
     for k in reqs:
         torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+
+
+def test_toy_interleaved_pairs(tmp_path):
+    """The second toy with neighbouring dims as rotation pairs: the pairing is a property of
+    the position encoding that attention hands to the rotation, nothing else changes."""
+    import ninfer_amd
+    toy.register_routed()
+    cfg = dict(toy.TOY_ROUTED_CONFIG, pairing="interleaved", rot_dim=12)
+    d = str(tmp_path / "toy_interleaved")
+    ninfer_amd.write_random_model(d, cfg, 10, std=0.3)
+    _, w = util.read_folder(d)
+    runner = runner_for(d, seqs=3)
+    reqs = {f"r{i}": util.random_tokens(n, 83, 50 + i) for i, n in enumerate([7, 26, 15])}
+    ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
+    half = toy.plain_forward_routed(w, dict(cfg, pairing="half"), reqs["r1"])
+    assert (half - ref["r1"]).abs().max() > 1e-3, "the pairing must matter"
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=6, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+
+
+def test_toy_mixer_with_pools_of_its_own(tmp_path):
+    """A mixer whose paged cache is two pools of different widths and dtypes (a 32-bit latent
+    that is key and value at once, a short rotated key in the activation dtype), one layer
+    with a window: the cache manager allocates, groups, frees and reuses its pages as it
+    does attention's, and nothing of the framework is changed for it."""
+    import ninfer_amd
+    toy.register_latent()
+    cfg = toy.TOY_LATENT_CONFIG
+    d = str(tmp_path / "toy_latent")
+    ninfer_amd.write_random_model(d, cfg, 12, std=0.3)
+    _, w = util.read_folder(d)
+    runner = runner_for(d, page_size=4, num_pages=26, seqs=3)
+    pools = runner.cache.pools
+    assert sorted(pools[0]) == ["latent", "pos_key"] and pools[0]["latent"].shape == (26, 4, 12)
+    assert pools[1]["pos_key"].shape == (26, 4, 6)
+    assert [g.window for g in runner.cache.groups] == [None, 9]
+    assert runner.cache.kv_bytes_per_token(4) == 2 * (12 * 4 + 6 * 4)
+    assert runner.cache.kv_bytes_per_token(2) == 2 * (12 * 4 + 6 * 2)   # the latent stays 32-bit
+    reqs = {f"l{i}": util.random_tokens(n, 61, 70 + i) for i, n in enumerate([9, 30, 17, 41, 5])}
+    ref = {k: toy.plain_forward_latent(w, cfg, v) for k, v in reqs.items()}
+    for k, v in reqs.items():
+        for sched in (util.schedule_whole(k, v), util.schedule_tail(k, v, 5),
+                      util.schedule_portions(k, v, 1)):
+            torch.testing.assert_close(util.run_schedule(runner, sched)[k], ref[k],
+                                       atol=3e-5, rtol=1e-4)
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=8, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+    runner.cache.check()
+    assert runner.cache.pages_reused() > 0 and runner.cache.groups[1].window_freed > 0
+
+
+def test_page_checks_name_a_table_that_the_kernels_could_not_trust(model_dirs):
+    """The debugging option checks every step's block tables on the host before anything is
+    launched: a page number outside the pool, a position without a held page, a page in two
+    requests' tables."""
+    from ninfer_amd import Chunk, EngineOptions, load_model
+    opt = EngineOptions(dtype="float32", max_context=64, num_sequences=3, page_size=4,
+                        num_pages=12, device="cpu", check_pages=True)
+    runner = load_model(model_dirs["B"]["float32"], opt, ops=PlainOps())
+    a, b = runner.open(), runner.open()
+    runner.step([Chunk(a, list(range(9)), []), Chunk(b, list(range(5)), [])])
+    g = runner.cache.groups[0]
+    keep = g.rows[a, 1]
+    g.rows[a, 1] = 99
+    with pytest.raises(RuntimeError, match="outside"):
+        runner.step([Chunk(a, [1], [0])])
+    g.rows[a, 1] = -1
+    with pytest.raises(RuntimeError, match="not held"):
+        runner.step([Chunk(a, [1], [0])])
+    g.rows[a, 1] = g.rows[b, 0]
+    with pytest.raises(RuntimeError, match="slots"):
+        runner.step([Chunk(a, [1], []), Chunk(b, [1], [])])
+    g.rows[a, 1] = keep
+    assert runner.step([Chunk(a, [1], [0]), Chunk(b, [2], [0])]).shape[0] == 2
+
+
+def test_cache_sized_in_bytes(model_dirs):
+    from ninfer_amd import EngineOptions, load_model
+    # A: two layers of 2 kv heads x 16, keys and values, 32-bit: 2 * 2 * 2 * 16 * 4 = 512 bytes a token
+    opt = EngineOptions(dtype="float32", max_context=64, num_sequences=2, page_size=8,
+                        kv_bytes=512 * 8 * 10 + 100, device="cpu")
+    runner = load_model(model_dirs["A"]["float32"], opt, ops=PlainOps())
+    assert runner.cache.kv_bytes_per_token(4) == 512 and runner.cache.pages_total(0) == 10
+    with pytest.raises(ValueError, match="not both"):
+        EngineOptions(num_pages=4, kv_bytes=1 << 20).validate()
+    with pytest.raises(ValueError, match="holds no page"):
+        load_model(model_dirs["A"]["float32"],
+                   EngineOptions(dtype="float32", kv_bytes=100, device="cpu"), ops=PlainOps())
+
+
+def test_weights_can_be_read_back_by_name(model_dirs):
+    """What the engine holds under a checkpoint name, fused and stacked tensors included,
+    is what the folder holds."""
+    d = model_dirs["B"]["float32"]
+    _, w = util.read_folder(d)
+    runner = runner_for(d)
+    assert set(runner.tensor_names()) == set(w) 
+    for name, t in w.items():
+        assert torch.equal(runner.tensor(name).float().cpu().reshape(t.shape), t), name
+    with pytest.raises(KeyError):
+        runner.tensor("no.such.weight")

@@ -69,7 +69,7 @@ def test_a_crowd_under_a_tight_pool_generates_what_each_request_does_alone(model
     runner = load_model(d, EngineOptions(dtype="float32", max_context=96, num_sequences=3,
                                          page_size=page, num_pages=pages,
                                          prefill_chunk=rng.choice([8, 16, 64]),
-                                         poison_freed_pages=True, use_graph=seed % 3 == 0))
+                                         poison_freed_pages=True, check_pages=True, use_graph=seed % 3 == 0))
     sched = Scheduler(runner, Sampler(runner.ops, runner.device))
     crowd = requests()
     for r in crowd:
@@ -134,7 +134,8 @@ def test_command_line(model_dirs):
     proc = subprocess.run(
         [sys.executable, os.path.join(ROOT, "bin", "ninfer"), d, "--prompt-ids",
          ",".join(map(str, prompt)), "--random-prompts", "5,9", "--max-new", "6", "--temperature",
-         "0", "--dtype", "fp32", "--max-context", "64", "--prefill-chunk", "8", "--seed", "3"],
+         "0", "--dtype", "fp32", "--max-context", "64", "--prefill-chunk", "8", "--seed", "3",
+         "--repeat-penalty", "1"],
         capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stderr[-2000:]
     lines = proc.stdout.strip().splitlines()
@@ -155,12 +156,50 @@ def test_command_line(model_dirs):
     proc = subprocess.run(
         [sys.executable, os.path.join(ROOT, "bin", "ninfer"), model_dirs["A"]["bfloat16"],
          "--prompt-ids", ",".join(map(str, prompt)), "--max-new", "4", "--temperature", "0",
-         "--max-context", "64", "--verify"], capture_output=True, text=True, timeout=300)
+         "--max-context", "64", "--repeat-penalty", "1", "--kv-gib", "0.001", "--verify"],
+        capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stderr[-2000:]
-    assert "verify:" in proc.stderr
+    # what --verify has to say follows from the run's own output and the plain model on the
+    # same (bfloat16-rounded) weights, which is what the 32-bit path computes
+    _, w16 = util.read_folder(model_dirs["A"]["bfloat16"])
+    out = [int(x) for x in proc.stdout.strip().splitlines()[0].split(",")]
+    want = plain_model.greedy_generate(w16, cfg, prompt, 4)
+    report = [l for l in proc.stderr.splitlines() if "verify:" in l]
+    assert len(report) == 1
+    if out == want:
+        assert "PASS" in report[0] and "(4 tokens)" in report[0]
+    else:
+        first = next(i for i, (a, b) in enumerate(zip(out, want)) if a != b)
+        assert f"request 0 parts from the 32-bit output at token {first} " in report[0]
     bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "ninfer"), d, "--no-such-flag"],
                          capture_output=True, text=True, timeout=120)
     assert bad.returncode != 0
+
+
+def test_verify_names_the_first_token_that_differs(model_dirs, capsys):
+    """--verify's report on a case with a known answer: outputs that were made to differ from
+    the 32-bit path's at chosen places."""
+    from ninfer_amd import SamplingParams, cli
+    d = model_dirs["A"]["bfloat16"]
+    cfg, w16 = util.read_folder(d)
+    prompts = [util.random_tokens(n, cfg["vocab_size"], 8 + n) for n in (6, 9, 4)]
+    golden = [plain_model.greedy_generate(w16, cfg, p, 5) for p in prompts]
+    args = cli.build_parser().parse_args([d])
+    common = dict(max_context=64, prefill_chunk=16, num_sequences=4, dtype="bfloat16",
+                  page_size=16, num_pages=None, use_graph=False, kv_bytes=None)
+    params = SamplingParams.greedy(5)
+    cli._verify(args, cfg, common, prompts, params, None, [list(g) for g in golden])
+    err = capsys.readouterr().err
+    assert "verify: PASS" in err and "(15 tokens)" in err
+    outs = [list(g) for g in golden]
+    outs[1][3] = (outs[1][3] + 1) % cfg["vocab_size"]
+    outs[2] = outs[2][:2]
+    cli._verify(args, cfg, common, prompts, params, None, outs)
+    err = capsys.readouterr().err
+    assert "PASS" not in err
+    assert "request 1 parts from the 32-bit output at token 3 (5 / 5 tokens)" in err
+    assert "request 2 parts from the 32-bit output at token 2 (2 / 5 tokens)" in err
+    assert "request 0" not in err
 
 
 def test_toy_mixer_on_the_gpu(tmp_path):
@@ -198,6 +237,71 @@ def test_toy_routed_feed_forward_and_position_on_the_gpu(tmp_path):
     torch.testing.assert_close(
         util.run_schedule(runner, util.schedule_tail(k0, reqs[k0], 6))[k0], ref[k0],
         atol=3e-5, rtol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_interleaved_pairs_on_the_gpu(tmp_path, dtype):
+    """Neighbouring dims as rotation pairs (a partial rotation of 12 of 16 dims), chosen by
+    the position encoding alone: the rotation kernel takes the pairing as a parameter."""
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, load_model
+    toy.register_routed()
+    cfg = dict(toy.TOY_ROUTED_CONFIG, pairing="interleaved", rot_dim=12)
+    d = str(tmp_path / "toy_interleaved")
+    ninfer_amd.write_random_model(d, cfg, 10, dtype=dtype, std=0.3)
+    _, w = util.read_folder(d)
+    runner = load_model(d, EngineOptions(dtype=dtype, max_context=64, num_sequences=3, page_size=4,
+                                         check_pages=True))
+    reqs = {f"r{i}": util.random_tokens(n, 83, 50 + i) for i, n in enumerate([7, 26, 15, 33])}
+    ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
+    half = toy.plain_forward_routed(w, dict(cfg, pairing="half"), reqs["r1"])
+    assert (half - ref["r1"]).abs().max() > 1e-3, "the pairing must matter"
+    if dtype == "float32":
+        got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=6, max_live=3))
+        for k in reqs:
+            torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+    else:
+        # One expert per token: a row whose two best experts are nearly tied may go either way
+        # in bfloat16, so single rows have no bound. What is asked: the typical row lies far
+        # closer to the plain model with these pairs than to the one with the other pairs.
+        got = util.run_schedule(runner, util.schedule_portions("r3", reqs["r3"], 2))["r3"]
+        other = toy.plain_forward_routed(w, dict(cfg, pairing="half"), reqs["r3"])
+        err = (got - ref["r3"]).abs().max(-1).values
+        wrong = (got - other).abs().max(-1).values
+        assert float(err.median()) < float(wrong.median()) / 3
+        assert float(err.median()) < 0.03 * float(ref["r3"].abs().max())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_mixer_with_pools_of_its_own_on_the_gpu(tmp_path, dtype):
+    """The third toy: a mixer with two paged pools of different widths and dtypes (the latent
+    is 32-bit also in the bfloat16 engine), a window on one layer, freed pages poisoned."""
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, load_model
+    toy.register_latent()
+    cfg = toy.TOY_LATENT_CONFIG
+    d = str(tmp_path / "toy_latent")
+    ninfer_amd.write_random_model(d, cfg, 12, dtype=dtype, std=0.2)
+    _, w = util.read_folder(d)
+    runner = load_model(d, EngineOptions(dtype=dtype, max_context=64, num_sequences=3, page_size=4,
+                                         num_pages=26, poison_freed_pages=True, check_pages=True))
+    pools = runner.cache.pools[0]
+    assert pools["latent"].dtype == torch.float32 and pools["latent"].shape == (26, 4, 12)
+    assert pools["pos_key"].dtype == runner.act_dtype and pools["pos_key"].shape == (26, 4, 6)
+    reqs = {f"l{i}": util.random_tokens(n, 61, 70 + i) for i, n in enumerate([9, 30, 17, 41, 5])}
+    ref = {k: toy.plain_forward_latent(w, cfg, v) for k, v in reqs.items()}
+    # bfloat16 keeps three digits: the bound follows the size of the logits
+    size = max(float(r.abs().max()) for r in ref.values())
+    bound = dict(atol=3e-5, rtol=1e-4) if dtype == "float32" else dict(atol=0.03 * size, rtol=0.05)
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=8, max_live=3))
+    for k in reqs:
+        assert torch.isfinite(got[k]).all()
+        torch.testing.assert_close(got[k], ref[k], **bound)
+    torch.testing.assert_close(
+        util.run_schedule(runner, util.schedule_tail("l3", reqs["l3"], 7))["l3"], ref["l3"], **bound)
+    runner.cache.check()
+    assert runner.cache.pages_reused() > 0 and runner.cache.groups[1].window_freed > 0
+    assert torch.isnan(pools["latent"]).any() and torch.isnan(pools["pos_key"]).any()
 
 
 @pytest.mark.parametrize("plan", [[(0, None), (1, 0), (2, None)],

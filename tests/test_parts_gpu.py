@@ -67,7 +67,7 @@ def test_attention_part(ops, dtype, heads, kv, d, window):
     outs = []
     for first, rows in ((0, 33), (33, 17)):
         ctx = util.make_context(ops, dtype, [(first, rows)])
-        call = CallInfo(cache=CacheView(pools[0], pools[1], table.contiguous(), ps, window))
+        call = CallInfo(cache=CacheView({"k": pools[0], "v": pools[1]}, table.contiguous(), ps, window))
         outs.append(att.forward(ctx, x[first:first + rows].cuda(), None, call))
     got = torch.cat(outs).float().cpu()
     torch.testing.assert_close(got, ref, **BOUND[dtype])
@@ -138,7 +138,7 @@ def test_block_arrangement(ops):
     pools = [torch.zeros(6, 2, ps, d, device="cuda") for _ in range(2)]
     table = torch.arange(5, dtype=torch.int32, device="cuda")[None]
     residual = x.cuda().clone()
-    pending = block.forward(ctx, residual, None, CallInfo(cache=CacheView(pools[0], pools[1], table,
-                                                                          ps, None)))
+    pending = block.forward(ctx, residual, None, CallInfo(cache=CacheView({"k": pools[0], "v": pools[1]},
+                                                                          table, ps, None)))
     torch.testing.assert_close((residual + pending).cpu(), ref, atol=3e-5, rtol=1e-4)
     torch.testing.assert_close(residual.cpu(), h1, atol=3e-5, rtol=1e-4)

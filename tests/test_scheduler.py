@@ -190,3 +190,61 @@ def test_history_counts_like_a_counter():
         assert dict(zip(a.tolist(), n.tolist())) == dict(Counter(toks))
         assert len(h) == len(set(toks)) and h.count(toks[0]) == Counter(toks)[toks[0]]
         assert h.count(100000) == 0
+
+
+def test_an_older_request_is_never_given_back_for_a_newer_one(setup):
+    """An old request with a long prompt is still being fed in portions when a newer, short
+    one is already decoding and the pool runs dry: the newer one waits or is preempted, the
+    older one keeps its pages (it would have to recompute all its portions)."""
+    _, cfg, w = setup
+    runner, sched = make(setup, num_pages=14, chunk=8, max_context=96)   # 56 tokens of cache
+    old, new = requests(cfg, [44, 6], 6, temperature=0.0, repetition_penalty=1.0)
+    sched.add(old)
+    sched.add(new)
+    steps = 0
+    while sched.has_work():
+        sched.step()
+        steps += 1
+        assert old.preemptions == 0
+        assert steps < 200
+    assert old.status == "finished" and new.status == "finished"
+    assert old.output == plain_model.greedy_generate(w, cfg, old.prompt, 6)
+    assert new.output == plain_model.greedy_generate(w, cfg, new.prompt, 6)
+    assert new.preemptions > 0, "the pool was meant to run dry while the old prompt was fed"
+    runner.cache.check()
+    assert all(g.allocator.in_use == 0 for g in runner.cache.groups)
+
+
+def test_a_windowed_group_admits_what_its_window_can_serve(model_dirs):
+    """All layers of this model see a window of 8 keys. Eleven pages of 4 tokens cannot hold
+    the 60 tokens of the request, but they hold the window and one step's portion, and pages
+    the window has passed come back after every step: the request runs, and its tokens are
+    those of the plain model."""
+    import json
+    import os
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, Request, SamplingParams, Sampler, Scheduler, load_model
+    cfg = dict(TINY["B"][0], max_window_layers=0, sliding_window=8)
+    d = os.path.join(os.path.dirname(model_dirs["B"]["float32"]), "windows_only")
+    ninfer_amd.write_random_model(d, cfg, 5, std=0.1)
+    raw, w = util.read_folder(d)
+    opt = EngineOptions(dtype="float32", max_context=96, prefill_chunk=16, num_sequences=2,
+                        page_size=4, num_pages=11, device="cpu", check_pages=True)
+    runner = load_model(d, opt, ops=PlainOps())
+    assert [g.window for g in runner.cache.groups] == [8]
+    sched = Scheduler(runner, Sampler(PlainOps(), runner.device))
+    req = Request("long", util.random_tokens(52, cfg["vocab_size"], 3),
+                  SamplingParams.greedy(8))
+    sched.add(req)
+    sched.run()
+    assert req.status == "finished", req.error
+    assert req.output == plain_model.greedy_generate(w, raw, req.prompt, 8)
+    assert runner.cache.groups[0].window_freed > 0
+    # a pool smaller than the window and a portion still refuses it at admission
+    opt.num_pages = 5
+    runner = load_model(d, opt, ops=PlainOps())
+    sched = Scheduler(runner, Sampler(PlainOps(), runner.device))
+    req2 = Request("long", list(req.prompt), SamplingParams.greedy(8))
+    sched.add(req2)
+    sched.run()
+    assert req2.status == "failed" and "fit" in req2.error

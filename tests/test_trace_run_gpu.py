@@ -58,3 +58,11 @@ def test_trace_replay_all_ways(model_dirs, tmp_path, name, dtype):
     for k in reqs:
         torch.testing.assert_close(got[k], ref[k], **bound,
                                    msg=lambda m: f"{name} {dtype} {k} mixed: {m}")
+    import json
+    with open(str(tmp_path / "mixed" / "stats.json")) as f:
+        stats = json.load(f)
+    assert stats["steps"] == len(steps) and len(stats["groups"]) == (1 if name == "A" else 2)
+    for g in stats["groups"]:
+        assert g["reused"] > 0 and g["in_use"] == 0 and g["allocated"] == g["freed"]
+        assert 0 < g["peak_in_use"] <= g["pages"] == 16
+        assert (g["window_freed"] > 0) == (g["window"] is not None)

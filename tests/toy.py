@@ -15,8 +15,9 @@ from typing import Dict, List
 import torch
 
 from ninfer_amd.models.spec import ModelSpec
-from ninfer_amd.parts import (Attention, FeedForward, LMHead, Mixer, PendingRows, PositionEncoding,
-                              PreNormBlock, RMSNorm, RoutedExperts, SwiGLU, TokenEmbedding)
+from ninfer_amd.parts import (Attention, CacheNeed, FeedForward, LMHead, Mixer, PendingRows,
+                              PoolSpec, PositionEncoding, PreNormBlock, RMSNorm, RoutedExperts,
+                              SwiGLU, TokenEmbedding)
 from ninfer_amd.parts.moe import Routing
 from ninfer_amd.registry import register_architecture, register_part
 from ninfer_amd.weights import TensorSpec
@@ -110,10 +111,11 @@ def plain_forward(w: Dict[str, torch.Tensor], cfg: dict, tokens: List[int]) -> t
 
 class HarmonicPosition(PositionEncoding):
     """Rotation by the angles pos * slope / (1 + i), i < rot_dim / 2: no geometric
-    series, and only the first rot_dim dims of a head turn."""
+    series, and only the first rot_dim dims of a head turn; pair i is dims
+    (i, i + rot_dim / 2) or, with pairing "interleaved", (2i, 2i + 1)."""
 
-    def __init__(self, rot_dim: int, slope: float):
-        self.rot_dim, self.slope = rot_dim, slope
+    def __init__(self, rot_dim: int, slope: float, pairing: str = "half"):
+        self.rot_dim, self.slope, self.pairing = rot_dim, slope, pairing
         self._table = None
 
     def inv_freq(self) -> torch.Tensor:
@@ -175,7 +177,8 @@ def build_toy_routed(cfg: ToyRoutedConfig) -> ModelSpec:
     for l in range(c["num_hidden_layers"]):
         p = f"layers.{l}."
         attn = Attention(p + "attn.", h, c["heads"], c["kv_heads"], c["head_dim"],
-                         HarmonicPosition(c["rot_dim"], c["slope"]), qkv_bias=False,
+                         HarmonicPosition(c["rot_dim"], c["slope"], c.get("pairing", "half")),
+                         qkv_bias=False,
                          window=c["window"])
         blocks.append(PreNormBlock(RMSNorm(p + "norm1.", h, c["rms_norm_eps"]), attn,
                                    RMSNorm(p + "norm2.", h, c["rms_norm_eps"]),
@@ -205,7 +208,13 @@ def plain_forward_routed(w: Dict[str, torch.Tensor], c: dict, tokens: List[int])
     phi = pos.float()[:, None] * f[None, :]
     cos, sin = torch.cos(phi)[:, None, :], torch.sin(phi)[:, None, :]
 
-    def turn(v):   # [T, heads, D]: the first rot dims in half-split pairs, the rest as they are
+    def turn(v):   # [T, heads, D]: the first rot dims in pairs, the rest as they are
+        if c.get("pairing", "half") == "interleaved":   # pair i = dims (2i, 2i + 1)
+            out = v.clone()
+            a, b = v[..., 0:rot:2], v[..., 1:rot:2]
+            out[..., 0:rot:2] = a * cos - b * sin
+            out[..., 1:rot:2] = a * sin + b * cos
+            return out
         a, b, rest = v[..., :rot // 2], v[..., rot // 2:rot], v[..., rot:]
         return torch.cat([a * cos - b * sin, a * sin + b * cos, rest], dim=-1)
 
@@ -228,4 +237,125 @@ def plain_forward_routed(w: Dict[str, torch.Tensor], c: dict, tokens: List[int])
             y[r] = prob[r, e] * pm.swiglu_mlp(m[r:r + 1], w[pe + "gate_proj.weight"],
                                               w[pe + "up_proj.weight"], w[pe + "down_proj.weight"])[0]
         x = x + y
+    return pm.rms_norm(x, w["norm.weight"], c["rms_norm_eps"]) @ w["head.weight"].float().T
+
+
+# ---- a third toy: a mixer whose paged cache is not "keys and values of one shape" ----
+
+class LatentMixer(Mixer):
+    """Keeps two pools per token that differ in width and in dtype: a latent vector c_t =
+    x_t Wc^T of `latent` numbers, always 32-bit, which serves as key and as value, and a short
+    position key r_t = x_t Wr^T of `pos_dim` numbers in the activation dtype, turned by the
+    angle t * slope in neighbouring pairs. Row t scores key j <= t (within the window) by
+    (x_t Wq^T . c_j + turn(x_t Wp^T) . r_j) / sqrt(latent + pos_dim) and returns
+    (sum_j p_j c_j) Wo^T. Written with torch operations on the engine's pools and block
+    table: what it shows is that the cache manager hands any named pools to a mixer."""
+
+    def __init__(self, prefix: str, hidden: int, latent: int, pos_dim: int, slope: float,
+                 window=None):
+        self.prefix, self.hidden, self.latent, self.pos_dim = prefix, hidden, latent, pos_dim
+        self.slope, self.window = slope, window
+        self.w = {}
+
+    def cache_need(self):
+        return CacheNeed((PoolSpec("latent", (), (self.latent,), "float32"),
+                          PoolSpec("pos_key", (), (self.pos_dim,))), self.window)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        p, h = self.prefix, self.hidden
+        return {p + "c.weight": TensorSpec((self.latent, h)), p + "r.weight": TensorSpec((self.pos_dim, h)),
+                p + "q.weight": TensorSpec((self.latent, h)), p + "p.weight": TensorSpec((self.pos_dim, h)),
+                p + "o.weight": TensorSpec((h, self.latent))}
+
+    def bind(self, w) -> None:
+        self.w = {n: w.matrix(self.prefix + n + ".weight").float() for n in "crqpo"}
+
+    def turn(self, v: torch.Tensor, pos: torch.Tensor) -> torch.Tensor:
+        phi = pos.float()[:, None] * self.slope
+        out = v.clone()
+        a, b = v[:, 0::2], v[:, 1::2]
+        out[:, 0::2] = a * torch.cos(phi) - b * torch.sin(phi)
+        out[:, 1::2] = a * torch.sin(phi) + b * torch.cos(phi)
+        return out
+
+    def forward(self, ctx, x, residual, call):
+        cache, ps = call.cache, call.cache.page_size
+        latent, pos_key = cache["latent"], cache["pos_key"]
+        assert latent.dtype == torch.float32 and pos_key.dtype == x.dtype
+        assert latent.shape[1:] == (ps, self.latent) and pos_key.shape[1:] == (ps, self.pos_dim)
+        xf, pos = x.float(), ctx.positions.long()
+        table = cache.block_table.long()[ctx.row_seq.long()]          # [T, pages]
+        page = table.gather(1, (pos // ps)[:, None])[:, 0]
+        assert (page >= 0).all()
+        c = xf @ self.w["c"].T
+        latent[page, pos % ps] = c
+        pos_key[page, pos % ps] = self.turn(xf @ self.w["r"].T, pos).to(pos_key.dtype)
+        q, qp = xf @ self.w["q"].T, self.turn(xf @ self.w["p"].T, pos)
+        out = torch.empty_like(c)
+        for t in range(x.shape[0]):
+            lo = max(0, int(pos[t]) - self.window + 1) if self.window else 0
+            js = torch.arange(lo, int(pos[t]) + 1, device=x.device)
+            pages = table[t, js // ps]
+            assert (pages >= 0).all(), "read of a page that is not held"
+            cj, rj = latent[pages, js % ps], pos_key[pages, js % ps].float()
+            s = (cj @ q[t] + rj @ qp[t]) / (self.latent + self.pos_dim) ** 0.5
+            out[t] = torch.softmax(s, 0) @ cj
+        return (out @ self.w["o"].T).to(x.dtype)
+
+
+def build_toy_latent(cfg: ToyRoutedConfig) -> ModelSpec:
+    c = cfg.raw
+    h = c["hidden_size"]
+    blocks = []
+    for l in range(c["num_hidden_layers"]):
+        p = f"layers.{l}."
+        blocks.append(PreNormBlock(RMSNorm(p + "norm1.", h, c["rms_norm_eps"]),
+                                   LatentMixer(p + "mix.", h, c["latent"], c["pos_dim"], c["slope"],
+                                               c["windows"][l]),
+                                   RMSNorm(p + "norm2.", h, c["rms_norm_eps"]),
+                                   SwiGLU(p + "mlp.", h, c["inner"])))
+    return ModelSpec(TokenEmbedding("embed.", c["vocab_size"], h), blocks,
+                     RMSNorm("norm.", h, c["rms_norm_eps"]), LMHead("head.", c["vocab_size"], h))
+
+
+def register_latent() -> None:
+    register_part("mixer", "latent", LatentMixer)
+    register_architecture("ToyLatentForCausalLM", ToyRoutedConfig.from_dict, build_toy_latent)
+
+
+TOY_LATENT_CONFIG = {"architectures": ["ToyLatentForCausalLM"], "vocab_size": 61, "hidden_size": 40,
+                     "num_hidden_layers": 2, "latent": 12, "pos_dim": 6, "slope": 0.4,
+                     "windows": [None, 9], "inner": 48, "rms_norm_eps": 1e-5}
+
+
+def plain_forward_latent(w: Dict[str, torch.Tensor], c: dict, tokens: List[int]) -> torch.Tensor:
+    """Whole-sequence reference of the third toy (32-bit, no cache)."""
+    import plain_model as pm
+    t = len(tokens)
+    pos = torch.arange(t)
+    phi = pos.float()[:, None] * c["slope"]
+
+    def turn(v):
+        out = v.clone()
+        a, b = v[:, 0::2], v[:, 1::2]
+        out[:, 0::2] = a * torch.cos(phi) - b * torch.sin(phi)
+        out[:, 1::2] = a * torch.sin(phi) + b * torch.cos(phi)
+        return out
+
+    x = w["embed.weight"][torch.tensor(tokens)].float()
+    for l in range(c["num_hidden_layers"]):
+        p = f"layers.{l}."
+        a = pm.rms_norm(x, w[p + "norm1.weight"], c["rms_norm_eps"])
+        lat, key = a @ w[p + "mix.c.weight"].T, turn(a @ w[p + "mix.r.weight"].T)
+        q, qp = a @ w[p + "mix.q.weight"].T, turn(a @ w[p + "mix.p.weight"].T)
+        s = (q @ lat.T + qp @ key.T) / (c["latent"] + c["pos_dim"]) ** 0.5
+        dist = pos[:, None] - pos[None, :]
+        seen = dist >= 0
+        if c["windows"][l]:
+            seen &= dist < c["windows"][l]
+        s = s.masked_fill(~seen, float("-inf"))
+        x = x + (torch.softmax(s, -1) @ lat) @ w[p + "mix.o.weight"].T
+        m = pm.rms_norm(x, w[p + "norm2.weight"], c["rms_norm_eps"])
+        x = x + pm.swiglu_mlp(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
+                              w[p + "mlp.down_proj.weight"])
     return pm.rms_norm(x, w["norm.weight"], c["rms_norm_eps"]) @ w["head.weight"].float().T

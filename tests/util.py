@@ -46,20 +46,30 @@ def routing_margins(w, cfg, tokens) -> torch.Tensor:
     return worst
 
 
-def safe_prompt(w, cfg, n: int, seed: int, rel_margin: float = 0.06) -> List[int]:
+def safe_prompt(w, cfg, n: int, seed: int, rel_margin: float = 0.06,
+                max_forwards: int = 0) -> List[int]:
     """Seeded random token ids, redrawn where the plain model's routing would
     be nearly tied: top-k routing is discontinuous, so a row whose k-th and
     (k+1)-th experts are within rounding noise of each other may legitimately
     pick either in reduced precision, and no bound on logits could hold there.
-    A row's routing depends only on its prefix, so rows are fixed left to right."""
+    A row's routing depends only on its prefix, so the prompt grows token by
+    token, each drawn again until its own row routes clearly. With
+    `max_forwards` the search stops after that many runs of the plain model and
+    the prompt found so far (at least two tokens) is returned: with dozens of
+    experts in several layers most rows are nearly tied somewhere."""
     rng = random.Random(seed)
-    toks = [rng.randrange(cfg["vocab_size"]) for _ in range(n)]
-    for _ in range(20 * n):
-        bad = torch.nonzero(routing_margins(w, cfg, toks) < rel_margin).flatten()
-        if bad.numel() == 0:
-            return toks
-        toks[int(bad[0])] = rng.randrange(cfg["vocab_size"])
-    raise RuntimeError("no prompt with clear routing found")
+    toks: List[int] = []
+    forwards = 0
+    while len(toks) < n:
+        cand = rng.randrange(cfg["vocab_size"])
+        forwards += 1
+        if float(routing_margins(w, cfg, toks + [cand])[-1]) >= rel_margin:
+            toks.append(cand)
+        elif max_forwards and forwards >= max_forwards and len(toks) >= 2:
+            break
+        elif forwards > 60 * n + 200:
+            raise RuntimeError("no prompt with clear routing found")
+    return toks
 
 
 # A schedule is a list of steps; a step is (entries, end) with entries
