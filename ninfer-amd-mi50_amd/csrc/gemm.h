@@ -36,6 +36,12 @@ struct GemmArgs {
                          // gemm_split, not by callers
   float* workspace;      // 32-bit scratch for a product cut along K, or null
   int64_t workspace_floats;
+  // What tests and measurements ask of one call (all 0: the library chooses). Per call, not
+  // state of the library: a caller that forgets to reset it changes nothing for the next.
+  int64_t split_min_bytes;  // least bytes of weights for a cut along K (0: 48 MB)
+  int force_kernel;      // many-row kernel: 1, 2, 3 = tiles of 64, 128, 256 rows
+  int skinny_two;        // few-row grouped products with two feature sets per block: 1 = whenever
+                         // the shape allows, -1 = never
 };
 
 // Which rows does tile `ti` of the grouped enumeration cover? Tiles of

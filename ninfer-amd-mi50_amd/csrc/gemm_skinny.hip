@@ -241,8 +241,7 @@ bool gemm_skinny_takes(const GemmArgs& a) {
          ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0) && a.w_group_stride % 8 == 0;
 }
 
-static int g_skinny_two = 1;   // tests and measurements switch the two-set blocks off
-static long g_skinny_two_min = 4096;
+constexpr long kSkinnyTwoMinBlocks = 4096;   // GemmArgs::skinny_two overrides the choice for tests
 
 static SkinnyPlan plan_skinny(const GemmArgs& a) {
   SkinnyPlan p;
@@ -267,8 +266,8 @@ static SkinnyPlan plan_skinny(const GemmArgs& a) {
   p.waves = (blocks < 2 * cus && chunks >= 16) ? 16 : (blocks < 8 * cus && chunks >= 8) ? 8 : 4;
   // a grouped product without SwiGLU whose tiles are many and short (K small): two feature
   // sets per block, so that blocks are half as many and each does twice the work
-  p.two = g_skinny_two && a.offsets && a.epilogue == kEpilogueNone && p.rows == 16 && p.waves == 4 &&
-          blocks >= g_skinny_two_min && a.N % 32 == 0;
+  p.two = a.skinny_two >= 0 && a.offsets && a.epilogue == kEpilogueNone && p.rows == 16 &&
+          p.waves == 4 && blocks >= (a.skinny_two > 0 ? 1 : kSkinnyTwoMinBlocks) && a.N % 32 == 0;
   if (p.two) p.rows = 32;
   p.grid_x = (a.N + p.rows - 1) / p.rows;
   return p;
@@ -326,8 +325,4 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream) {
 
 }  // namespace ninfer
 
-extern "C" void ninfer_set_skinny_two(int v, long min_blocks) {
-  ninfer::g_skinny_two = v;
-  if (min_blocks > 0) ninfer::g_skinny_two_min = min_blocks;
-}
 

@@ -85,9 +85,16 @@ __global__ __launch_bounds__(NW * 64, OCC) void gemm_tile_kernel(GemmArgs a) {
     int v = tid + i * NT, r = v / VPR, kv = v % VPR;
     wsrc[i] = W + (int64_t)staged_w_row<TN, WGM, SWIGLU>(r, out0, N) * K + 8 * kv + kt_first * TK;
   }
+  // Every block walks its k tiles in a circle from a start of its own: blocks that start
+  // together would otherwise read the same columns of rows that lie a power of two apart at
+  // the same time, which fall on few memory channels.
+  const int phase = (int)((blockIdx.x * 5u + blockIdx.y * 3u) % (unsigned)nk);
   // P register stages: the loads of k tile t + P are issued while tile t is multiplied
   bf16x8 xreg[P][XV], wreg[P][WV];
-  auto load_tile = [&](int st, int k0) {
+  auto load_tile = [&](int st, int k_lin) {   // k_lin: the tile's place in this block's walk, times TK
+    int kt = k_lin / TK + phase;
+    kt = kt >= nk ? kt - nk : kt;
+    const int k0 = kt * TK;
 #pragma unroll
     for (int i = 0; i < XV; ++i) xreg[st][i] = *(const bf16x8*)(xsrc[i] + k0);
 #pragma unroll
@@ -206,8 +213,7 @@ bool gemm_tile_takes(const GemmArgs& a) {
          ((uintptr_t)a.W % 16 == 0) && a.w_group_stride % 8 == 0;
 }
 
-static int g_tile_variant = 0;   // tests: 0 = choose by shape
-static int64_t g_split_min_bytes = 48 << 20;   // tests lower it to cut small products too
+constexpr int64_t kSplitMinBytes = 48 << 20;   // GemmArgs::split_min_bytes lowers it for tests
 
 template <int TM, int TN, int TK, int NW, int WGM, int P, int OCC = 2>
 static int launch_tile(const GemmArgs& a, hipStream_t stream) {
@@ -241,12 +247,12 @@ static int launch_tile(const GemmArgs& a, hipStream_t stream) {
 int gemm_tile(const GemmArgs& a, hipStream_t stream) {
   // Tile height. Grouped: as the tile lists were made. Dense: the tallest tile that still
   // gives every CU a block (taller tiles read less per product, but fewer of them fill the
-  // chip). g_tile_variant (tests) forces 64, 128 or 256 rows on dense products.
+  // chip). force_kernel (tests) forces 64, 128 or 256 rows on dense products.
   int rows;
   if (a.offsets) {
     rows = a.big_rows ? a.big_rows : 64;
-  } else if (g_tile_variant >= 1 && g_tile_variant <= 3) {
-    rows = 32 << g_tile_variant;
+  } else if (a.force_kernel >= 1 && a.force_kernel <= 3) {
+    rows = 32 << a.force_kernel;
   } else {
     const int n_units = a.epilogue == kEpilogueSwiGLU ? 2 * a.N : a.N;   // W rows
     auto blocks = [&](int tm, int tn) { return ((a.M + tm - 1) / tm) * ((n_units + tn - 1) / tn); };
@@ -290,7 +296,7 @@ __global__ void sum_parts_kernel(const float* __restrict__ ws, int parts, int M,
 int gemm_split_parts(const GemmArgs& a) {
   if (a.offsets || a.epilogue != kEpilogueNone || !a.workspace || !gemm_tile_takes(a)) return 1;
   if (a.M <= 32 || a.M > 512 || a.N % 4 || a.ldc % 4 || ((uintptr_t)a.C & 15)) return 1;
-  if ((int64_t)a.N * a.K * 2 < g_split_min_bytes) return 1;
+  if ((int64_t)a.N * a.K * 2 < (a.split_min_bytes > 0 ? a.split_min_bytes : kSplitMinBytes)) return 1;
   if (a.M > 128 && a.K < 2 * a.N) return 1;   // beyond 128 rows only where K is long against N
   const int cus = device_cu_count(), tk = 64;
   const int tm = a.M > 128 ? 128 : 64;
@@ -329,5 +335,3 @@ int gemm_split(const GemmArgs& a, hipStream_t stream) {
 
 }  // namespace ninfer
 
-extern "C" void ninfer_set_tile_variant(int v) { ninfer::g_tile_variant = v; }
-extern "C" void ninfer_set_split_min_bytes(long long v) { ninfer::g_split_min_bytes = v; }

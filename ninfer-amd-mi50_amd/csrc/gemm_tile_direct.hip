@@ -104,14 +104,21 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   typedef __attribute__((address_space(3))) void* lptr;
   // Every lane of every load takes part: with some lanes switched off, a load into LDS did
   // not leave the other lanes' bytes where this layout expects them (products came out wrong).
-  auto issue = [&](int t) {   // k tile t into buffer t % NBUF
+  // Every block walks the k tiles in a circle from a start of its own: blocks that start
+  // together would otherwise read the same columns of rows that lie a power of two apart at
+  // the same time, which fall on few memory channels.
+  const int nk_all = K / TK;
+  const int phase = (int)((blockIdx.x * 5u + blockIdx.y * 3u) % (unsigned)nk_all);
+  auto issue = [&](int t) {   // the t-th k tile of this block's walk into buffer t % NBUF
     unsigned char* buf = smem + (t % NBUF) * BUF_BYTES + wave * 1024;
+    int kt = t + phase;
+    kt = kt >= nk_all ? kt - nk_all : kt;
 #pragma unroll
     for (int i = 0; i < NL; ++i)
-      __builtin_amdgcn_global_load_lds((gptr)(xsrc[i] + t * TK), (lptr)(buf + i * 4096), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr)(xsrc[i] + kt * TK), (lptr)(buf + i * 4096), 16, 0, 0);
 #pragma unroll
     for (int i = 0; i < NL; ++i)
-      __builtin_amdgcn_global_load_lds((gptr)(wsrc[i] + t * TK), (lptr)(buf + X_BYTES + i * 4096), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr)(wsrc[i] + kt * TK), (lptr)(buf + X_BYTES + i * 4096), 16, 0, 0);
   };
 
   f32x16 acc[FI][FJ];

@@ -33,7 +33,8 @@ class _GemmArgs(ctypes.Structure):
                 ("a_div", ctypes.c_int), ("in_dtype", ctypes.c_int), ("out_dtype", ctypes.c_int),
                 ("epilogue", ctypes.c_int), ("big_rows", ctypes.c_int),
                 ("k_parts", ctypes.c_int), ("workspace", ctypes.c_void_p),
-                ("workspace_floats", ctypes.c_int64)]
+                ("workspace_floats", ctypes.c_int64), ("split_min_bytes", ctypes.c_int64),
+                ("force_kernel", ctypes.c_int), ("skinny_two", ctypes.c_int)]
 
 
 class _AttnArgs(ctypes.Structure):
@@ -96,6 +97,20 @@ class _Together:
         return False
 
 
+class _Tuned:
+    def __init__(self, ops, values):
+        self.ops, self.values = ops, values
+
+    def __enter__(self):
+        self.saved = dict(self.ops._tune)
+        self.ops._tune.update(self.values)
+        return self.ops
+
+    def __exit__(self, *exc):
+        self.ops._tune = self.saved
+        return False
+
+
 class HipOps:
     def __init__(self, lib_path: Optional[str] = None):
         self.lib_path = lib_path or ensure_built()
@@ -114,6 +129,20 @@ class HipOps:
         self._attn_ws = None
         self._outgrown = []     # workspaces that captured graphs may still point to
         self._split_ws = None   # 32 MB of 32-bit scratch for products cut along K, made at first use
+        # what tests and measurements ask of the product kernels (see `tuned`); all 0: the
+        # library chooses
+        self._tune = {"force_kernel": 0, "split_min_bytes": 0, "skinny_two": 0}
+
+    def tuned(self, **values):
+        """Context manager for tests and measurements: inside it every product call carries
+        these choices (force_kernel: 1, 2, 3 = many-row tiles of 64, 128, 256 rows;
+        split_min_bytes: least bytes of weights for a cut along K;
+        skinny_two: 1 / -1 = two feature sets per block whenever possible / never). They
+        travel with each call; the library keeps no such state."""
+        unknown = set(values) - set(self._tune)
+        if unknown:
+            raise KernelError(f"tuned(): unknown choices {sorted(unknown)}")
+        return _Tuned(self, values)
 
     # ---- helpers ----------------------------------------------------------------
     def _stream(self) -> ctypes.c_void_p:
@@ -314,6 +343,9 @@ class HipOps:
                          _ptr(a_index), _ptr(c_index), t16, t64, tc, w_group_stride, m, n, k,
                          a.shape[1],
                          c.shape[1], groups, a_div, _DT[a.dtype], _DT[c.dtype], epilogue, big)
+        args.force_kernel = self._tune["force_kernel"]
+        args.split_min_bytes = self._tune["split_min_bytes"]
+        args.skinny_two = self._tune["skinny_two"]
         if only_if_split:
             # a dense product of few dozen rows: the library's unless the kernels here cut it
             # along K (its output tiles alone would not fill the GPU)

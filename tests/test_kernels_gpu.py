@@ -117,14 +117,12 @@ def test_swiglu_linear(ops_mode, gen, dtype, m, inner, k):
 
 @pytest.mark.parametrize("variant", [1, 2, 3])
 @pytest.mark.parametrize("m,n,k", [(333, 700, 256), (70, 130, 384), (129, 1000, 512), (600, 520, 320),
-                                   (257, 264, 64), (40, 36, 128)])
+                                   (257, 264, 64), (40, 36, 128), (1, 8, 1408), (170, 1408, 2048)])
 def test_tile_product_every_tile_height(ops, gen, variant, m, n, k):
-    """The many-row kernels with 64-row, 128-row and 256-row tiles (tile counts
-    that are no multiple of the 8 XCDs, rows that end inside a tile, one to five
-    k tiles of the 256-row kernel's pipeline, widths that are and are not a
-    multiple of 8: both epilogues)."""
-    ops.lib.ninfer_set_tile_variant(variant)
-    try:
+    """The many-row kernels with 64-row, 128-row and 256-row tiles (tile counts that are no
+    multiple of the 8 XCDs, rows that end inside a tile and inside a block of 32, one to 32
+    k tiles of the pipelines, widths that are and are not a multiple of 8: both epilogues)."""
+    with ops.tuned(force_kernel=variant):
         x, w = rnd((m, k), torch.bfloat16, gen), rnd((n, k), torch.bfloat16, gen)
         bias = torch.randn(n, generator=gen, device="cuda")
         o1 = torch.empty(m, n, device="cuda")
@@ -140,8 +138,6 @@ def test_tile_product_every_tile_height(ops, gen, variant, m, n, k):
         ops.library_min_rows = saved
         PlainOps().swiglu_linear(x, wgu, h2)
         close(h1, h2, torch.bfloat16, scale=k * 0.2)
-    finally:
-        ops.lib.ninfer_set_tile_variant(0)
 
 
 @pytest.mark.parametrize("m,n,k", [(33, 2048, 5632), (64, 3584, 20480), (100, 300, 512),
@@ -154,8 +150,7 @@ def test_linear_cut_along_k(ops, gen, m, n, k):
     x, w = rnd((m, k), torch.bfloat16, gen), rnd((n, k), torch.bfloat16, gen)
     o1 = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
     o2, o3 = torch.empty_like(o1), torch.empty_like(o1)
-    ops.lib.ninfer_set_split_min_bytes(ctypes.c_longlong(0))   # products of any size
-    try:
+    with ops.tuned(split_min_bytes=1):   # products of any size
         assert ops._gemm(x, w, o1, m=m, n=n, k=k, only_if_split=True), "not cut along K"
         PlainOps().linear(x, w, o2)
         close(o1, o2, torch.bfloat16, scale=math.sqrt(k))
@@ -170,8 +165,6 @@ def test_linear_cut_along_k(ops, gen, m, n, k):
         assert ops._gemm(x, w, f1, m=m, n=n, k=k, bias=bias, only_if_split=True)
         PlainOps().linear(x, w, f2, bias=bias)
         close(f1, f2, torch.float32, scale=200 * math.sqrt(k))
-    finally:
-        ops.lib.ninfer_set_split_min_bytes(ctypes.c_longlong(48 << 20))
     if n * k * 2 < (48 << 20):   # by default only long weight streams are cut
         assert not ops._gemm(x, w, o3, m=m, n=n, k=k, only_if_split=True)
 
@@ -765,9 +758,8 @@ def test_grouped_down_with_two_feature_sets_per_block(ops, gen, t, e, k, h, inne
     wd = rnd((e, h, inner), torch.bfloat16, gen, 0.2)
     x2, w2 = rnd((t, inner), torch.bfloat16, gen), rnd((h, inner), torch.bfloat16, gen, 0.2)
     outs = []
-    for two in (0, 1):
-        ops.lib.ninfer_set_skinny_two(two, ctypes.c_long(1))
-        try:
+    for two in (-1, 1):
+        with ops.tuned(skinny_two=two):
             y = torch.zeros(n, h, device="cuda", dtype=torch.bfloat16)
             ops.grouped_down(hh, wd, r.offsets, r.order, y, tiles=r)
             y_pair = torch.zeros_like(y)
@@ -776,8 +768,6 @@ def test_grouped_down_with_two_feature_sets_per_block(ops, gen, t, e, k, h, inne
                 ops.grouped_down(hh, wd, r.offsets, r.order, y_pair, tiles=r)
                 ops.linear(x2, w2, dense)
             outs.append((y, y_pair, dense))
-        finally:
-            ops.lib.ninfer_set_skinny_two(1, ctypes.c_long(4096))
     for a, b in zip(*outs):
         assert torch.equal(a, b)
     y_ref = torch.zeros(n, h, device="cuda", dtype=torch.bfloat16)
