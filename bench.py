@@ -70,6 +70,10 @@ def main() -> int:
                     help="every decode step launched kernel by kernel")
     ap.add_argument("--model", default="a2.7b", choices=sorted(MODELS),
                     help="layer sizes: a2.7b (the default and the headline) or 57b-a14b")
+    ap.add_argument("--profile", action="store_true",
+                    help="also time every kind of kernel call of one eager decode step and one "
+                         "prefill with device events (untimed runs of their own; the table goes "
+                         "to stderr and under \"profile\")")
     ap.add_argument("--scenario", default="decode", choices=["decode", "long"])
     ap.add_argument("--requests", type=int, default=8, help="--scenario long: concurrent requests")
     ap.add_argument("--prompt", type=int, default=32768, help="--scenario long: prompt tokens")
@@ -195,6 +199,65 @@ def main() -> int:
         runner._graphs.clear()
         return max(float((a - b).abs().max()) for a, b in zip(*outs))
 
+    def profile_calls(label: str, chunks) -> dict:
+        """Microseconds by kind of kernel call for one eager step: every call of the kernel
+        library is bracketed by device events (calls inside `together()` are launched when
+        it ends and are timed there, as one kind). The reference prints such a table per
+        phase (src/models/model.hip:1066-1081)."""
+        ops = runner.ops
+        spans = []
+
+        def kind(name, a):
+            if name in ("linear", "swiglu_linear"):
+                return f"{name} {a[0].shape[0]}x{a[1].shape[1]}->{a[2].shape[1]}"
+            if name in ("grouped_swiglu", "grouped_down"):
+                return f"{name} {a[0].shape[0]} rows"
+            return name
+
+        names = ["embed", "rmsnorm", "qkv_rope", "rope_kv_write", "paged_attention", "linear",
+                 "swiglu_linear", "silu_mul", "grouped_swiglu", "grouped_down", "moe_route",
+                 "moe_combine", "_launch_held"]
+        saved = {n: getattr(ops, n) for n in names}
+
+        depth = [0]
+
+        def wrap(n):
+            def call(*a, **kw):
+                if (ops._held is not None and n != "_launch_held") or depth[0]:
+                    return saved[n](*a, **kw)       # held back (timed when launched), or part of a call that is timed
+                s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s.record()
+                depth[0] += 1
+                try:
+                    out = saved[n](*a, **kw)
+                finally:
+                    depth[0] -= 1
+                e.record()
+                spans.append(("products launched together" if n == "_launch_held" else kind(n, a), s, e))
+                return out
+            return call
+
+        use_graph, runner.options.use_graph = runner.options.use_graph, False
+        try:
+            for n in names:
+                setattr(ops, n, wrap(n))
+            runner.step(chunks)
+            torch.cuda.synchronize()
+        finally:
+            for n in names:
+                setattr(ops, n, saved[n])
+            runner.options.use_graph = use_graph
+        table = {}
+        for k_, s, e in spans:
+            calls, us = table.get(k_, (0, 0.0))
+            table[k_] = (calls + 1, us + s.elapsed_time(e) * 1e3)
+        total = sum(us for _, us in table.values())
+        print(f"[bench] {label}: {total:.0f} us in kernel calls (eager, with event overhead)",
+              file=sys.stderr)
+        for k_, (calls, us) in sorted(table.items(), key=lambda kv: -kv[1][1]):
+            print(f"[bench]   {us:9.1f} us {100 * us / total:5.1f}%  {calls:4d} x {k_}", file=sys.stderr)
+        return {k_: round(us, 1) for k_, (_, us) in table.items()}
+
     def copy_rate() -> float:
         """Bytes a second that a plain device copy of 2 GiB moves (read + write): what the
         memory system gives a kernel that does nothing else."""
@@ -237,12 +300,32 @@ def main() -> int:
                              "ms": round(pdt * 1e3, 3),
                              "frac": round(flops / pdt / FLOP_PEAK[args.dtype], 4)}
     if not args.no_points:
-        points = {}
+        points, fracs = {}, {}
         for b in (1, 64):
             steps = max(8, args.steps // (4 if b == 64 else 1))
-            d, _, _ = decode_run(b, steps, max(2, args.warmup // 2))
+            d, nb, _ = decode_run(b, steps, max(2, args.warmup // 2))
             points[f"decode_b{b}"] = round(b / d, 2)
+            fracs[f"decode_b{b}"] = round(nb / d / HBM_PEAK, 4)
         result["points"] = points
+        result["points_hbm_frac"] = fracs   # the same roofline as the default step's, per point
+    if args.profile:
+        slots = [runner.open() for _ in range(args.batch)]
+        for sl in slots:
+            runner.cache.reserve(sl, ctx - 2)
+            runner.cache.commit(sl, ctx - 2)
+        toks = torch.randint(0, V, (args.batch,), generator=gen).tolist()
+        step = [Chunk(sl, [t], [0]) for sl, t in zip(slots, toks)]
+        profile_calls("warm-up", step)
+        result["profile"] = {"decode": profile_calls(f"decode step, batch {args.batch}", step)}
+        for sl in slots:
+            runner.close(sl)
+        pt = min(args.prefill_tokens, ctx)
+        ptoks = torch.randint(0, V, (pt,), generator=gen).tolist()
+        for label in ("warm-up", f"prefill of {pt} tokens"):
+            sl = runner.open()
+            table = profile_calls(label, [Chunk(sl, ptoks, [pt - 1])])
+            runner.close(sl)
+        result["profile"]["prefill"] = table
     if args.graph and not args.no_check:
         batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
         worst = max(graph_check(b) for b in batches)
