@@ -149,7 +149,11 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
   // V: thread loads a 4-key x 8-dim block and stores it transposed.
   constexpr int K_VECS = PK * D / 8;                  // 16-byte vectors in a K tile
   constexpr int K_PER_THREAD = (K_VECS + NT - 1) / NT;
-  constexpr int V_BLOCKS = (PK / 4) * (D / 8);        // 4 x 8 blocks in a V tile
+  // V: blocks of 4 keys x VD dims; 8 dims (16-byte loads) unless that leaves threads without
+  // a block, then 4 (8-byte loads, every thread busy)
+  constexpr int VD = (PK / 4) * (D / 8) < NT ? 4 : 8;
+  typedef __bf16 vvec __attribute__((ext_vector_type(VD)));
+  constexpr int V_BLOCKS = (PK / 4) * (D / VD);       // 4 x VD blocks in a V tile
   constexpr int V_PER_THREAD = (V_BLOCKS + NT - 1) / NT;
   static_assert(K_VECS % NT == 0, "tile does not divide over the block");
 
@@ -158,9 +162,12 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
   // the other buffer, the loads of tile i + 1 + NS are issued into those registers,
   // and the page numbers of tile i + 1 + 2 NS are fetched: no load waits for another
   // inside the loop.
-  bf16x8 kreg[NS][K_PER_THREAD], vreg[NS][V_PER_THREAD][4];
+  bf16x8 kreg[NS][K_PER_THREAD];
+  vvec vreg[NS][V_PER_THREAD][4];
   int kpage[NS][K_PER_THREAD], vpage[NS][V_PER_THREAD];
-  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  vvec zero_v;
+#pragma unroll
+  for (int d = 0; d < VD; ++d) zero_v[d] = 0;
   // Every load below is unconditional (a select replaces what is not there by zeros): a
   // load under a condition would have to be waited for where the condition ends.
   auto load_pages = [&](int st, int t0) {
@@ -188,7 +195,7 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
 #pragma unroll
   for (int i = 0; i < V_PER_THREAD; ++i) {
     const int blk = (tid + i * NT) % V_BLOCKS;
-    v_in_page[i] = (((int64_t)g << ps_shift) + ((4 * (blk % (PK / 4))) & ps_mask)) * D + 8 * (blk / (PK / 4));
+    v_in_page[i] = (((int64_t)g << ps_shift) + ((4 * (blk % (PK / 4))) & ps_mask)) * D + VD * (blk / (PK / 4));
   }
   auto load_regs = [&](int st, int t0) {
 #pragma unroll
@@ -207,8 +214,8 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
       // a value that is not there must be zero: its probability is, but 0 x anything is not
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const bf16x8 got = *(const bf16x8*)(vsrc + r * D);
-        vreg[st][i][r] = (page >= 0 && kp0 + r <= pos_last) ? got : zero8;
+        const vvec got = *(const vvec*)(vsrc + r * D);
+        vreg[st][i][r] = (page >= 0 && kp0 + r <= pos_last) ? got : zero_v;
       }
     }
   };
@@ -226,9 +233,9 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
       if (blk < V_BLOCKS) {
         int kg = blk % (PK / 4), dv = blk / (PK / 4);
 #pragma unroll
-        for (int d = 0; d < 8; ++d) {
+        for (int d = 0; d < VD; ++d) {
           bf16x4 col = {vreg[st][i][0][d], vreg[st][i][1][d], vreg[st][i][2][d], vreg[st][i][3][d]};
-          *(bf16x4*)(vt_s + (8 * dv + d) * VPAD + 4 * kg) = col;
+          *(bf16x4*)(vt_s + (VD * dv + d) * VPAD + 4 * kg) = col;
         }
       }
     }
@@ -275,29 +282,35 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
     }
     mx *= scale2;   // the scale is positive: the largest score stays the largest
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, mx);
-    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+    // The reference point m of a row's exponents follows its maximum only in jumps: while the
+    // maximum stays within 2^8 of it, probabilities are formed against the old m (they may
+    // exceed 1, by up to 2^8: nothing for 32-bit sums or for bf16, which rounds relative to
+    // size) and neither the sum nor the 64 output registers are rescaled. The result is the
+    // same quotient; at the end the two halves and the chunks are merged by their own m.
+    const bool moved = __any(mx > m + 8.f);
     float psum = 0.f;
+    if (moved) {
+      asm volatile("" ::: "memory");   // a real branch: as selects the products would always run
+      const float m_new = fmaxf(m, mx);
+      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+      l *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) o[db] *= alpha;
+      m = m_new;
+    }
     // pf[kb][h]: the 16-key step h of key block kb; slot i of lane j is key 16 h + 8 (i / 4) + 4 j + i % 4
     bf16x8 pf[NKB][2];
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        float p = __builtin_amdgcn_exp2f(fmaf(s[kb][v], scale2, -m_new));
+        float p = __builtin_amdgcn_exp2f(fmaf(s[kb][v], scale2, -m));
         psum += p;
         pf[kb][v >> 3][v & 7] = (__bf16)p;
       }
-    l = l * alpha + psum;
-    // the output needs rescaling only when some row's maximum has moved
-    const bool moved = __any(m_new > m);
-    m = m_new;
+    l += psum;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      if (moved) {
-        asm volatile("" ::: "memory");   // a real branch: as selects the products would always run
-        o[db] *= alpha;
-      }
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll

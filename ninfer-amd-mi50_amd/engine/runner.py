@@ -171,13 +171,36 @@ class ModelRunner:
         if graph:
             logits = self._step_graph(host, shape)
         else:
-            if self.device.type == "cuda":
-                host = host.pin_memory()
-            logits = self._forward(host.to(self.device, non_blocking=True), shape)
+            logits = self._forward(self._to_device(host), shape)
         for c, p in zip(chunks, pos0):
             cache.commit(c.slot, p + len(c.tokens))
         self.steps_run += 1
         return logits
+
+    def _to_device(self, host: torch.Tensor) -> torch.Tensor:
+        """The step's packed index buffer on the device, copied through one of a few pinned
+        staging buffers that are kept and used in turn (allocating pinned memory every step
+        costs more than the copy). A buffer is reused only after the copy out of it has run."""
+        if self.device.type != "cuda":
+            return host
+        n = host.numel()
+        if not hasattr(self, "_staging"):
+            self._staging, self._staging_next = [], 0
+        if len(self._staging) < 4:
+            self._staging.append([torch.empty(max(n, 4096), dtype=torch.int32).pin_memory(),
+                                  torch.cuda.Event()])
+            slot = self._staging[-1]
+        else:
+            slot = self._staging[self._staging_next]
+            self._staging_next = (self._staging_next + 1) % len(self._staging)
+            slot[1].synchronize()
+            if slot[0].numel() < n:
+                slot[0] = torch.empty(2 * n, dtype=torch.int32).pin_memory()
+        slot[0][:n].copy_(host)
+        dev = torch.empty(n, dtype=torch.int32, device=self.device)
+        dev.copy_(slot[0][:n], non_blocking=True)
+        slot[1].record()
+        return dev
 
     def _check_pages(self, chunks: Sequence[Chunk], pos0: List[int], tables) -> None:
         """Debugging: what the kernels assume of the step's block tables, checked on the host
