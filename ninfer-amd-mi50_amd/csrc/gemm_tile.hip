@@ -88,7 +88,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void gemm_tile_kernel(GemmArgs a) {
   // Every block walks its k tiles in a circle from a start of its own: blocks that start
   // together would otherwise read the same columns of rows that lie a power of two apart at
   // the same time, which fall on few memory channels.
-  const int phase = (int)((blockIdx.x * 5u + blockIdx.y * 3u) % (unsigned)nk);
+  const int phase = (int)((bx * 5u + by * 3u) % (unsigned)nk);
   // P register stages: the loads of k tile t + P are issued while tile t is multiplied
   bf16x8 xreg[P][XV], wreg[P][WV];
   auto load_tile = [&](int st, int k_lin) {   // k_lin: the tile's place in this block's walk, times TK
@@ -220,7 +220,8 @@ static int launch_tile(const GemmArgs& a, hipStream_t stream) {
   if (a.offsets && a.tiles64 && TM != (a.big_rows ? a.big_rows : 64))
     return set_error(-1, "gemm: the grouped tile lists are made for %d rows, not %d", a.big_rows, TM);
   const bool swiglu = a.epilogue == kEpilogueSwiGLU;
-  const int m_tiles = (a.M + TM - 1) / TM + (a.offsets ? a.groups : 0);
+  int m_tiles = (a.M + TM - 1) / TM + (a.offsets ? a.groups : 0);
+  if (a.offsets) m_tiles = (m_tiles + kXcds - 1) / kXcds * kXcds;   // block_to_tile's bijection
   const int per_block = swiglu ? TN / 2 : TN;
   const dim3 grid(m_tiles, (a.N + per_block - 1) / per_block, a.k_parts > 1 ? a.k_parts : 1);
   const size_t lds = 2 * (TM + TN) * (TK + 8) * sizeof(bf16);

@@ -1,7 +1,9 @@
 // C = A W^T for very many rows per weight matrix (bf16): 256 x 256 tiles, loaded
 // from global memory straight into LDS (global_load_lds_dwordx4), so that no
 // registers stage the tiles, in k tiles of 64 (whole 128-byte lines of every
-// row) and two buffers. Dense or grouped by expert, bias or SwiGLU epilogue, as
+// row): two buffers for the rows of A, which neighbours share through L2, and
+// three for the rows of W, which come from HBM and are the bytes that have to
+// be on their way (all 160 KB of a CU's LDS). Dense or grouped by expert, bias or SwiGLU epilogue, as
 // the staged kernel beside it; the reference sends these products to rocBLAS
 // (src/ops/linear.hip:21-35, src/models/model.hip:406-425).
 //
@@ -17,8 +19,8 @@
 //
 // One barrier per k tile, before its last quarter: when a wave passes the
 // barrier of tile t, tile t + 1 has landed for every wave and every wave holds
-// the last fragments of tile t in registers, so the loads of tile t + 2 may
-// overwrite tile t. The fragments of every quarter are read while the products
+// the last fragments of tile t in registers, so the loads of A's tile t + 2 and
+// of W's tile t + 3 may overwrite tile t. The fragments of every quarter are read while the products
 // of the quarter before run, across the barrier too.
 #include "gemm_tile.h"
 #include <type_traits>
@@ -41,22 +43,24 @@ template <int N> __device__ __forceinline__ void wait_loads_and_lds() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(N) : "memory");
 }
 
-template <int TK, int NBUF, bool SWIGLU, typename TC>
+template <int TK, bool SWIGLU, typename TC>
 __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   using namespace direct;
   constexpr int KK = TK / 16;                // parts of a k tile: one MFMA depth each
   constexpr int ROW_BYTES = TK * 2;
   constexpr int CPR = ROW_BYTES / 16;        // 16-byte chunks of a staged row
   constexpr int RPP = 64 / CPR;              // rows of a 1 KB piece
-  constexpr int X_BYTES = TM * ROW_BYTES;
-  constexpr int BUF_BYTES = (TM + TN) * ROW_BYTES;
+  constexpr int X_BYTES = TM * ROW_BYTES, W_BYTES = TN * ROW_BYTES;
+  constexpr int NBX = 2, NBW = 3;            // buffers of A rows, of W rows
+  constexpr int W_BASE = NBX * X_BYTES;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  __shared__ int tile_info[3];
 
   int bx, by;
   block_to_tile(a.offsets != nullptr, bx, by);
   int row0, row_end, group;
-  if (!tile_rows<TM>(a, bx, tile_info, row0, row_end, group)) return;
+  // the search's three ints lie in the buffers: no load may land before every wave has them
+  if (!tile_rows<TM>(a, bx, (int*)smem, row0, row_end, group)) return;
+  __syncthreads();
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave % WGM, wn = wave / WGM;
@@ -108,18 +112,26 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   // together would otherwise read the same columns of rows that lie a power of two apart at
   // the same time, which fall on few memory channels.
   const int nk_all = K / TK;
-  const int phase = (int)((blockIdx.x * 5u + blockIdx.y * 3u) % (unsigned)nk_all);
-  auto issue = [&](int t) {   // the t-th k tile of this block's walk into buffer t % NBUF
-    unsigned char* buf = smem + (t % NBUF) * BUF_BYTES + wave * 1024;
+  const int phase = (int)((bx * 5u + by * 3u) % (unsigned)nk_all);
+  // the t-th k tile of this block's walk: A rows into their buffer t % NBX, W rows into
+  // theirs at byte w_off (the caller's count of t % NBW)
+  auto issue_x = [&](int t) {
+    unsigned char* buf = smem + (t % NBX) * X_BYTES + wave * 1024;
     int kt = t + phase;
     kt = kt >= nk_all ? kt - nk_all : kt;
 #pragma unroll
     for (int i = 0; i < NL; ++i)
       __builtin_amdgcn_global_load_lds((gptr)(xsrc[i] + kt * TK), (lptr)(buf + i * 4096), 16, 0, 0);
+  };
+  auto issue_w = [&](int t, int w_off) {
+    unsigned char* buf = smem + W_BASE + w_off + wave * 1024;
+    int kt = t + phase;
+    kt = kt >= nk_all ? kt - nk_all : kt;
 #pragma unroll
     for (int i = 0; i < NL; ++i)
-      __builtin_amdgcn_global_load_lds((gptr)(wsrc[i] + kt * TK), (lptr)(buf + X_BYTES + i * 4096), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr)(wsrc[i] + kt * TK), (lptr)(buf + i * 4096), 16, 0, 0);
   };
+  auto next_w = [](int w_off) { return w_off == (NBW - 1) * W_BYTES ? 0 : w_off + W_BYTES; };
 
   f32x16 acc[FI][FJ];
 #pragma unroll
@@ -139,7 +151,7 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   const int lr = lane & 31, lk = lane >> 5;
   const int sw = (lr / (16 / CPR)) % CPR;
   const int x_lane = (tok0 + lr) * ROW_BYTES;
-  const int w_lane = X_BYTES + (wm * (TN / WGM) + lr) * ROW_BYTES;
+  const int w_lane = W_BASE + (wm * (TN / WGM) + lr) * ROW_BYTES;
   int c_part[KK];
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk) c_part[kk] = 16 * ((2 * kk + lk) ^ sw);
@@ -149,13 +161,15 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
     constexpr int NJ = decltype(nj_tag)::value;
     constexpr int NX = NJ > 0 ? NJ : 1;
     bf16x8 wf[2][FI], xf[2][NX];
-    auto read_part = [&](int set, int t, int kk) {
+    // fragments of k part kk of the tile in A's buffer t % NBX and W's buffer at w_off
+    auto read_part = [&](int set, int t, int w_off, int kk) {
       if constexpr (NJ == 0) return;
-      const unsigned char* buf = smem + (t % NBUF) * BUF_BYTES + c_part[kk];
+      const unsigned char* xb = smem + (t % NBX) * X_BYTES + c_part[kk];
+      const unsigned char* wb = smem + w_off + c_part[kk];
 #pragma unroll
-      for (int i = 0; i < FI; ++i) wf[set][i] = *(const bf16x8*)(buf + w_lane + i * 32 * ROW_BYTES);
+      for (int i = 0; i < FI; ++i) wf[set][i] = *(const bf16x8*)(wb + w_lane + i * 32 * ROW_BYTES);
 #pragma unroll
-      for (int jj = 0; jj < NJ; ++jj) xf[set][jj] = *(const bf16x8*)(buf + x_lane + jj * 32 * ROW_BYTES);
+      for (int jj = 0; jj < NJ; ++jj) xf[set][jj] = *(const bf16x8*)(xb + x_lane + jj * 32 * ROW_BYTES);
     };
     auto multiply = [&](int set) {
 #pragma unroll
@@ -174,57 +188,54 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
       }
       __builtin_amdgcn_sched_group_barrier(0x008, FI * NJ > FI + NJ ? FI * NJ - FI - NJ : 0, 0);
     };
-    // Waiting for tile t + 1 leaves the tiles after it under way: `later` of them.
-    auto wait_tile = [&](int later) {
-      switch (later) {
-        case 0: wait_loads_and_lds<0>(); break;
-        case 1: wait_loads_and_lds<NLT>(); break;
-        case 2: wait_loads_and_lds<2 * NLT>(); break;
-        default: wait_loads_and_lds<(NBUF > 2 ? NBUF - 2 : 0) * NLT>(); break;
-      }
-    };
-    // every buffer's first tile on its way, tile 0 landed
-#pragma unroll
-    for (int b = 0; b < NBUF; ++b)
-      if (b < nk) issue(b);
-    {
-      const int later = min(NBUF, nk) - 1;
-      if (later >= 4) wait_loads<4 * NLT>();
-      else if (later == 3) wait_loads<3 * NLT>();
-      else if (later == 2) wait_loads<2 * NLT>();
-      else if (later == 1) wait_loads<NLT>();
-      else wait_loads<0>();
+    // A wave's loads return in the order of their issue: A 0, W 0, A 1, W 1, W 2, then per
+    // tile t A t + 2, W t + 3. When tile t + 1 is needed, the only younger loads are W's
+    // tile t + 2 (NL loads), which stay on their way.
+    issue_x(0);
+    issue_w(0, 0);
+    if (nk > 1) {
+      issue_x(1);
+      issue_w(1, W_BYTES);
     }
+    if (nk > 2) issue_w(2, 2 * W_BYTES);
+    if (nk > 2) wait_loads<3 * NL>();
+    else if (nk > 1) wait_loads<2 * NL>();
+    else wait_loads<0>();
     __builtin_amdgcn_s_barrier();
-    read_part(0, 0, 0);
-    int t = 0;
-    // steady state, free of conditions: tile t + NBUF exists
-    for (; t + NBUF < nk; ++t) {
+    read_part(0, 0, 0, 0);
+    int t = 0, w_cur = 0;   // w_cur: where W's tile t lies
+    // steady state, free of conditions: W's tile t + 3 exists
+    for (; t + NBW < nk; ++t) {
 #pragma unroll
       for (int kk = 0; kk + 1 < KK; ++kk) {
-        read_part((kk + 1) & 1, t, kk + 1);
+        read_part((kk + 1) & 1, t, w_cur, kk + 1);
         multiply(kk & 1);
         interleave();
       }
       // this wave's loads of tile t + 1 have landed and its last fragments of tile t are in
-      // registers; after the barrier that holds for every wave, and tile t's buffer is free
-      wait_loads_and_lds<(NBUF - 2) * NLT>();
+      // registers; after the barrier that holds for every wave, and tile t's buffers are free
+      wait_loads_and_lds<NL>();
       __builtin_amdgcn_s_barrier();
-      issue(t + NBUF);
-      read_part(KK & 1, t + 1, 0);
+      issue_x(t + NBX);
+      issue_w(t + NBW, w_cur);
+      w_cur = next_w(w_cur);
+      read_part(KK & 1, t + 1, w_cur, 0);
       multiply((KK - 1) & 1);
       interleave();
     }
-    // the last NBUF tiles
+    // the last NBW tiles: A's tile t + 2 still to issue while it exists
     for (; t < nk; ++t) {
 #pragma unroll
       for (int kk = 0; kk + 1 < KK; ++kk) {
-        read_part((kk + 1) & 1, t, kk + 1);
+        read_part((kk + 1) & 1, t, w_cur, kk + 1);
         multiply(kk & 1);
       }
-      wait_tile(max(nk - t - 2, 0));
+      if (t + NBW == nk) wait_loads_and_lds<NL>();   // W's last tile may stay on its way
+      else wait_loads_and_lds<0>();
       __builtin_amdgcn_s_barrier();
-      if (t + 1 < nk) read_part(KK & 1, t + 1, 0);
+      if (t + NBX < nk) issue_x(t + NBX);
+      w_cur = next_w(w_cur);
+      if (t + 1 < nk) read_part(KK & 1, t + 1, w_cur, 0);
       multiply((KK - 1) & 1);
     }
   };
@@ -236,7 +247,7 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
     case 3: run(std::integral_constant<int, 3>{}); break;
     default: run(std::integral_constant<int, 4>{}); break;
   }
-  static_assert(4 * FJ * 32 * FI * 64 <= NBUF * BUF_BYTES, "the epilogue's stage exceeds the buffers");
+  static_assert(4 * FJ * 32 * FI * 64 <= NBX * X_BYTES + NBW * W_BYTES, "the epilogue's stage exceeds the buffers");
   __syncthreads();   // every wave has read its last fragments: the buffers become the epilogue's stage
   write_tile<FI, FJ, SWIGLU, TC>(a, acc, smem + wave * (FJ * 32 * FI * 64), tok0, row0, rows_here,
                                  out0 + OUT_PER_WAVE * wm, row_of);
@@ -247,17 +258,18 @@ bool gemm_tile_direct_takes(const GemmArgs& a) {
          ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0) && a.w_group_stride % 8 == 0;
 }
 
-template <int TK, int NBUF>
+template <int TK>
 static int launch_direct(const GemmArgs& a, hipStream_t stream) {
   using namespace direct;
-  constexpr int LDS_BYTES = NBUF * (TM + TN) * TK * 2;
+  constexpr int LDS_BYTES = (2 * TM + 3 * TN) * TK * 2;
   const bool swiglu = a.epilogue == kEpilogueSwiGLU;
-  const int m_tiles = (a.M + TM - 1) / TM + (a.offsets ? a.groups : 0);
+  int m_tiles = (a.M + TM - 1) / TM + (a.offsets ? a.groups : 0);
+  if (a.offsets) m_tiles = (m_tiles + kXcds - 1) / kXcds * kXcds;   // block_to_tile's bijection
   const int per_block = swiglu ? TN / 2 : TN;
   const dim3 grid(m_tiles, (a.N + per_block - 1) / per_block);
 #define NINFER_DIRECT_LAUNCH(SW, TYPE)                                                          \
   do {                                                                                          \
-    auto kern = gemm_tile_direct_kernel<TK, NBUF, SW, TYPE>;                                    \
+    auto kern = gemm_tile_direct_kernel<TK, SW, TYPE>;                                    \
     hipError_t e = hipFuncSetAttribute((const void*)kern,                                       \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);  \
     if (e != hipSuccess) return set_error(-2, "gemm: cannot get %d bytes of LDS", LDS_BYTES);   \
@@ -277,9 +289,9 @@ int gemm_tile_direct(const GemmArgs& a, hipStream_t stream) {
   if (a.offsets && a.tiles64 && a.big_rows != direct::TM)
     return set_error(-1, "gemm: the grouped tile lists are made for %d rows, not %d", a.big_rows,
                      direct::TM);
-  // k tiles of 64 in two buffers: measured faster than tiles of 32 in four (whole 128-byte
+  // k tiles of 64: measured faster than tiles of 32 in twice the buffers (whole 128-byte
   // lines per row beat the deeper queue of loads)
-  return launch_direct<64, 2>(a, stream);
+  return launch_direct<64>(a, stream);
 }
 
 }  // namespace ninfer

@@ -97,6 +97,32 @@ class _Together:
         return False
 
 
+class _Beside:
+    """Work on a second stream that starts after everything the current stream has been
+    given so far; `HipOps.join()` makes the current stream wait for it."""
+
+    def __init__(self, ops):
+        self.ops = ops
+
+    def __enter__(self):
+        ops = self.ops
+        if ops._side is None:
+            ops._side = torch.cuda.Stream()   # default priority
+        start = torch.cuda.Event()
+        start.record()
+        ops._side.wait_event(start)
+        self._ctx = torch.cuda.stream(ops._side)
+        self._ctx.__enter__()
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        done = torch.cuda.Event()
+        done.record()   # on the second stream, still the current one
+        self._ctx.__exit__(exc_type, exc, tb)
+        self.ops._side_done.append(done)
+        return False
+
+
 class _Tuned:
     def __init__(self, ops, values):
         self.ops, self.values = ops, values
@@ -120,6 +146,9 @@ class HipOps:
         self.lib.ninfer_sample_few_places.restype = ctypes.c_longlong
         self.force_generic = False  # tests: run the plain kernels whatever the shape
         self._held = None           # products held back inside `together()`
+        self._side = None           # the second stream of `beside()`, made at first use
+        self._side_done = []        # ends of `beside()` blocks that `join()` has not waited for
+        self.beside_min_rows = 512  # rows from which independent work is worth a second stream
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
         # ... a SwiGLU's gate/up product only beyond this many: up to here the tile kernel with
         # the activation in its epilogue beats the library's product followed by a kernel for
@@ -370,6 +399,21 @@ class HipOps:
         launch's fixed time is paid once), otherwise one after the other. Outputs
         are valid after the block, not inside it."""
         return _Together(self)
+
+    def beside(self):
+        """Context manager for work that nothing on the current stream waits for until
+        `join()`: it runs on a second stream, so that the device can fill with its blocks
+        the units that the current stream's kernels leave empty (the last, partly filled
+        round of a kernel whose blocks run one per CU). Memory made inside may be read on
+        the current stream after `join()`; what it reads must have been given to the
+        current stream before the block."""
+        return _Beside(self)
+
+    def join(self) -> None:
+        """The current stream waits for every `beside()` block so far."""
+        for done in self._side_done:
+            torch.cuda.current_stream().wait_event(done)
+        self._side_done = []
 
     def _launch_held(self, held):
         force = 1 if self.force_generic else 0

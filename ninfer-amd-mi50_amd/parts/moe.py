@@ -176,9 +176,20 @@ class SparseMoE(FeedForward):
             routing = self.router.route(ctx, self.router.logits(ctx, x))
             self.last_ids = routing.ids
             return PendingRows(self.experts.run(ctx, x, routing), routing.weights)
-        # The shared expert's two products wait for nothing the routed path makes: each goes
-        # together with the routed path's product of the same stage.
+        # The shared expert's two products wait for nothing the routed path makes. Many rows:
+        # they run on a stream of their own beside the routed path, whose kernels leave part
+        # of the device empty in their last round of blocks.
         logits = ctx.empty((x.shape[0], self.router.experts + 1), torch.float32)
+        if x.shape[0] >= ctx.ops.beside_min_rows:
+            with ctx.ops.beside():
+                shared = self.shared.down(ctx, self.shared.gate_up(ctx, x))
+            ctx.ops.linear(x, self.router_and_gate, logits)
+            routing = self.router.route(ctx, logits)
+            self.last_ids = routing.ids
+            y = self.experts.run(ctx, x, routing)
+            ctx.ops.join()
+            return PendingRows(y, routing.weights, shared, logits[:, self.router.experts])
+        # Few rows: each goes together with the routed path's product of the same stage.
         with ctx.ops.together():
             ctx.ops.linear(x, self.router_and_gate, logits)
             h_shared = self.shared.gate_up(ctx, x)

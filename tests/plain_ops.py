@@ -26,6 +26,15 @@ class PlainOps:
         """Independent products: nothing to gain here, they run as they are called."""
         return contextlib.nullcontext()
 
+    beside_min_rows = 8   # low, so that the host tests walk the many-row branch too
+
+    def beside(self):
+        """Work for a second stream: here it simply runs where it is called."""
+        return contextlib.nullcontext()
+
+    def join(self):
+        pass
+
     def fill_nan_pages(self, pool, pages):
         pool.index_fill_(0, pages.long(), float("nan"))
 
