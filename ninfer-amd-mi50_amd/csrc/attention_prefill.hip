@@ -57,6 +57,7 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
   constexpr int KPAD = D + 8;       // bf16 per K row in LDS
   constexpr int VPAD = PK + 4;      // bf16 per V^T row in LDS: 8-byte reads of 32 rows spread over the banks
   constexpr int K_TILE = PK * KPAD, V_TILE = D * VPAD;   // bf16 of a tile in LDS
+  constexpr bool EARLY = NQ == 4;   // 512 threads stage half as much each: registers to spare
   constexpr int MERGE = 2 + DB * 16 + 1;                   // floats a lane hands over at the end (odd stride)
   constexpr int TILES_BYTES = 2 * (K_TILE + V_TILE) * 2, MERGE_BYTES = NQ * 64 * MERGE * 4;
   // two tiles of each (one read, one written); at the end the same memory merges the two key halves
@@ -248,17 +249,50 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
     if (!wave_live || k0 > wave_pos_last || k0 + 32 * NKB <= wave_lo) return;
     const bf16* k_s = k_lds + buf * K_TILE;
     const bf16* vt_s = vt_lds + buf * V_TILE;
+    // Left alone, the compiler reads each fragment from LDS just before the matrix instruction
+    // that needs it (it keeps registers few), and that instruction then waits a whole LDS
+    // latency: 24 such waits in a row per tile. Where registers allow (EARLY), all reads of a
+    // phase are issued first; nothing moves across the asm statement that follows them.
     // S^T = K Q^T : NKB key blocks of 32 x 32 queries
     f32x16 s[NKB];
+    bf16x8 kf[NKB][KS];
+    auto read_keys = [&](int kb, int ks) {
+      kf[kb][ks] = *(const bf16x8*)(k_s + ((NKB * kh + kb) * 32 + c) * KPAD + 16 * ks + 8 * j);
+    };
+    if constexpr (EARLY) {
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) read_keys(kb, ks);
+      // the first fragment passes through the statement, so the chain begins after it
+      asm volatile("" : "+v"(kf[0][0]) : : "memory");
+    }
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        bf16x8 kf = *(const bf16x8*)(k_s + ((NKB * kh + kb) * 32 + c) * KPAD + 16 * ks + 8 * j);
-        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s[kb], 0, 0, 0);
+        if constexpr (!EARLY) read_keys(kb, ks);
+        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb][ks], qf[ks], s[kb], 0, 0, 0);
       }
+    }
+    // the values: with EARLY read here, while the vector units form the probabilities
+    bf16x8 vf[DB][NKB][2];
+    auto read_values = [&](int db, int kb, int hs) {
+      const bf16* vr = vt_s + (db * 32 + c) * VPAD + 32 * (NKB * kh + kb) + 16 * hs + 4 * j;
+      bf16x4 lo4 = *(const bf16x4*)vr;
+      bf16x4 hi4 = *(const bf16x4*)(vr + 8);
+      vf[db][kb][hs] = (bf16x8){lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+    };
+    if constexpr (EARLY) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+          for (int hs = 0; hs < 2; ++hs) read_values(db, kb, hs);
+      asm volatile("" ::: "memory");
     }
     // lane holds, for query c, keys k0 + 32 kb + 8 (v / 4) + 4 j + v % 4
     float mx = -1e30f;
@@ -315,11 +349,8 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
       for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
         for (int hs = 0; hs < 2; ++hs) {
-          const bf16* vr = vt_s + (db * 32 + c) * VPAD + 32 * (NKB * kh + kb) + 16 * hs + 4 * j;
-          bf16x4 lo4 = *(const bf16x4*)vr;
-          bf16x4 hi4 = *(const bf16x4*)(vr + 8);
-          bf16x8 vf = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kb][hs], o[db], 0, 0, 0);
+          if constexpr (!EARLY) read_values(db, kb, hs);
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][kb][hs], pf[kb][hs], o[db], 0, 0, 0);
         }
     }
   };
