@@ -99,7 +99,8 @@ class _Together:
 
 class _Beside:
     """Work on a second stream that starts after everything the current stream has been
-    given so far; `HipOps.join()` makes the current stream wait for it."""
+    given so far; `HipOps.join()` makes the current stream wait for it. The two events are
+    made once and recorded again every time (an event's earlier waits keep their meaning)."""
 
     def __init__(self, ops):
         self.ops = ops
@@ -108,18 +109,19 @@ class _Beside:
         ops = self.ops
         if ops._side is None:
             ops._side = torch.cuda.Stream()   # default priority
-        start = torch.cuda.Event()
-        start.record()
-        ops._side.wait_event(start)
-        self._ctx = torch.cuda.stream(ops._side)
-        self._ctx.__enter__()
+            ops._side_events = (torch.cuda.Event(), torch.cuda.Event())
+        if ops._side_open:
+            raise KernelError("beside(): join() the block before first")
+        self.main = torch.cuda.current_stream()
+        ops._side_events[0].record(self.main)
+        ops._side.wait_event(ops._side_events[0])
+        torch.cuda.set_stream(ops._side)
         return self
 
     def __exit__(self, exc_type, exc, tb):
-        done = torch.cuda.Event()
-        done.record()   # on the second stream, still the current one
-        self._ctx.__exit__(exc_type, exc, tb)
-        self.ops._side_done.append(done)
+        self.ops._side_events[1].record(self.ops._side)
+        torch.cuda.set_stream(self.main)
+        self.ops._side_open = True
         return False
 
 
@@ -147,7 +149,8 @@ class HipOps:
         self.force_generic = False  # tests: run the plain kernels whatever the shape
         self._held = None           # products held back inside `together()`
         self._side = None           # the second stream of `beside()`, made at first use
-        self._side_done = []        # ends of `beside()` blocks that `join()` has not waited for
+        self._side_events = None    # (start, end) of the `beside()` block
+        self._side_open = False     # a `beside()` block that `join()` has not waited for
         self.beside_min_rows = 512  # rows from which independent work is worth a second stream
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
         # ... a SwiGLU's gate/up product only beyond this many: up to here the tile kernel with
@@ -410,10 +413,10 @@ class HipOps:
         return _Beside(self)
 
     def join(self) -> None:
-        """The current stream waits for every `beside()` block so far."""
-        for done in self._side_done:
-            torch.cuda.current_stream().wait_event(done)
-        self._side_done = []
+        """The current stream waits for the `beside()` block before."""
+        if self._side_open:
+            torch.cuda.current_stream().wait_event(self._side_events[1])
+            self._side_open = False
 
     def _launch_held(self, held):
         force = 1 if self.force_generic else 0

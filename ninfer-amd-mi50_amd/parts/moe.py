@@ -181,11 +181,12 @@ class SparseMoE(FeedForward):
         # of the device empty in their last round of blocks.
         logits = ctx.empty((x.shape[0], self.router.experts + 1), torch.float32)
         if x.shape[0] >= ctx.ops.beside_min_rows:
-            with ctx.ops.beside():
-                shared = self.shared.down(ctx, self.shared.gate_up(ctx, x))
+            # routing first: its short kernels would crawl beside the shared expert's long ones
             ctx.ops.linear(x, self.router_and_gate, logits)
             routing = self.router.route(ctx, logits)
             self.last_ids = routing.ids
+            with ctx.ops.beside():
+                shared = self.shared.down(ctx, self.shared.gate_up(ctx, x))
             y = self.experts.run(ctx, x, routing)
             ctx.ops.join()
             return PendingRows(y, routing.weights, shared, logits[:, self.router.experts])
