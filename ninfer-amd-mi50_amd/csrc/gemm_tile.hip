@@ -88,7 +88,9 @@ __global__ __launch_bounds__(NW * 64, OCC) void gemm_tile_kernel(GemmArgs a) {
   // Every block walks its k tiles in a circle from a start of its own: blocks that start
   // together would otherwise read the same columns of rows that lie a power of two apart at
   // the same time, which fall on few memory channels.
-  const int phase = (int)((bx * 5u + by * 3u) % (unsigned)nk);
+  // (Grouped: the start depends on the expert, not on the row tile, so that a row's sum has the
+  // same order whichever tile of its expert the grouping put it in.)
+  const int phase = (int)(((a.offsets ? group : bx) * 5u + by * 3u) % (unsigned)nk);
   // P register stages: the loads of k tile t + P are issued while tile t is multiplied
   bf16x8 xreg[P][XV], wreg[P][WV];
   auto load_tile = [&](int st, int k_lin) {   // k_lin: the tile's place in this block's walk, times TK

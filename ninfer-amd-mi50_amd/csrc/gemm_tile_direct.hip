@@ -112,7 +112,9 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   // together would otherwise read the same columns of rows that lie a power of two apart at
   // the same time, which fall on few memory channels.
   const int nk_all = K / TK;
-  const int phase = (int)((bx * 5u + by * 3u) % (unsigned)nk_all);
+  // (Grouped: the start depends on the expert, not on the row tile, so that a row's sum has the
+  // same order whichever tile of its expert the grouping put it in.)
+  const int phase = (int)(((a.offsets ? group : bx) * 5u + by * 3u) % (unsigned)nk_all);
   // the t-th k tile of this block's walk: A rows into their buffer t % NBX, W rows into
   // theirs at byte w_off (the caller's count of t % NBW)
   auto issue_x = [&](int t) {

@@ -322,9 +322,9 @@ def test_long_prompt_on_the_many_row_kernels(wide_case, dtype):
                                                    num_sequences=2, page_size=16))
     whole = util.run_schedule(runner, util.schedule_whole("a", toks))["a"]
     torch.testing.assert_close(whole, ref, **bound(dtype), msg=lambda m: f"whole: {m}")
-    # at this many rows the shared expert ran on a stream of its own beside the routed path;
-    # on one stream the same kernels meet the same bound (not the same bits: the library's
-    # products of many rows differ in their last bits from run to run on one stream already)
+    # at this many rows the shared expert ran on a stream of its own beside the routed path:
+    # the same kernels on one stream give the same bits (and so does a second run: no result
+    # depends on the order in which the grouping's counters placed an expert's rows)
     ops = runner.ops
     assert ops._side is not None and not ops._side_open
     saved, ops.beside_min_rows = ops.beside_min_rows, 1 << 30
@@ -332,7 +332,9 @@ def test_long_prompt_on_the_many_row_kernels(wide_case, dtype):
         one_stream = util.run_schedule(runner, util.schedule_whole("a1", toks))["a1"]
     finally:
         ops.beside_min_rows = saved
-    torch.testing.assert_close(one_stream, ref, **bound(dtype), msg=lambda m: f"one stream: {m}")
+    assert torch.equal(one_stream, whole)
+    again = util.run_schedule(runner, util.schedule_whole("a2", toks))["a2"]
+    assert torch.equal(again, whole)
     cut = [("b", toks[:200], list(range(200))), ("b", toks[200:260], list(range(60))),
            ("b", toks[260:], list(range(380)))]
     steps = [([entry], ["b"] if i == len(cut) - 1 else []) for i, entry in enumerate(cut)]

@@ -292,6 +292,40 @@ def test_routing_in_one_call_with_tile_lists(ops, gen, t, e, k):
     assert sorted(r1.order.tolist()) == list(range(n))
 
 
+@pytest.mark.parametrize("big", [64, 128, 256])
+def test_grouped_products_do_not_depend_on_the_order_within_an_expert(ops, gen, big):
+    """The grouping leaves the rows of an expert in the order its atomic counters gave
+    them, which differs from run to run. A routed row's result must not depend on its
+    place among its expert's rows (on which tile it lands in): with the places reversed
+    within every expert the products give the same bits."""
+    from ninfer_amd.parts.moe import Routing
+    t, e, k, h, inner = 640, 4, 2, 256, 192
+    n = t * k
+    x = rnd((t, h), torch.bfloat16, gen)
+    wgu = rnd((e, 2 * inner, h), torch.bfloat16, gen, 0.06)
+    wd = rnd((e, h, inner), torch.bfloat16, gen, 0.06)
+    logits = torch.randn(t, e, generator=gen, device="cuda")
+    i32 = lambda *s: torch.zeros(*s, device="cuda", dtype=torch.int32)
+    r = Routing(i32(t, k), torch.zeros(t, k, device="cuda"), i32(e + 1), i32(n),
+                i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2), big_rows=big)
+    ops.moe_route(logits, e, k, False, r)
+
+    def products(routing):
+        hh = torch.empty(n, inner, device="cuda", dtype=torch.bfloat16)
+        y = torch.empty(n, h, device="cuda", dtype=torch.bfloat16)
+        ops.grouped_swiglu(x, wgu, routing.offsets, routing.order, k, hh, tiles=routing)
+        ops.grouped_down(hh, wd, routing.offsets, routing.order, y, tiles=routing)
+        return y
+    y1 = products(r)
+    off = r.offsets.tolist()
+    assert max(b - a for a, b in zip(off, off[1:])) > big   # some expert has more than one tile
+    order = r.order.clone()
+    for a, b in zip(off, off[1:]):
+        order[a:b] = r.order[a:b].flip(0)
+    r.order = order
+    assert torch.equal(products(r), y1)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_rmsnorm_adds_a_sum_of_rows_on_the_fly(ops, gen, dtype):
     from ninfer_amd.parts import PendingRows
