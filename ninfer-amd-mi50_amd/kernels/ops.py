@@ -151,7 +151,9 @@ class HipOps:
         self._side = None           # the second stream of `beside()`, made at first use
         self._side_events = None    # (start, end) of the `beside()` block
         self._side_open = False     # a `beside()` block that `join()` has not waited for
-        self.beside_min_rows = 512  # rows from which independent work is worth a second stream
+        # rows from which independent work is worth a second stream (switching streams costs the
+        # host about 0.1 ms a layer: at 512 rows of the smaller model the host then is the slower)
+        self.beside_min_rows = 1024
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
         # ... a SwiGLU's gate/up product only beyond this many: up to here the tile kernel with
         # the activation in its epilogue beats the library's product followed by a kernel for
