@@ -112,8 +112,8 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
     for (int u = 0; u < UNROLL; ++u) {
       const int j = wbase + (it0 + u) * KPI + kslot;
       ok[u] = j >= lo && j <= pos;
-      kf[u] = *(const bf16x8*)(kpool + koff[it0 + u]);
-      vf[u] = *(const bf16x8*)(vpool + koff[it0 + u]);
+      kf[u] = stream_load((const bf16x8*)(kpool + koff[it0 + u]));
+      vf[u] = stream_load((const bf16x8*)(vpool + koff[it0 + u]));
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {

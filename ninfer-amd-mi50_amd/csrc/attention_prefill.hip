@@ -204,7 +204,9 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
       // For a key that is not there, a row of the last key's page (beyond it) or of the
       // pool's first page (a page given back) is read in its place. Such a key lies in a
       // block that is masked, and the mask replaces its scores whatever they are.
-      kreg[st][i] = *(const bf16x8*)(kpool + max(kpage[st][i], 0) * page_stride + k_in_page[i]);
+      const bf16x8* src = (const bf16x8*)(kpool + max(kpage[st][i], 0) * page_stride + k_in_page[i]);
+      // decoding reads every key once a step; a prompt's keys serve many blocks of rows from L2
+      kreg[st][i] = HEADS ? stream_load(src) : *src;
     }
 #pragma unroll
     for (int i = 0; i < V_PER_THREAD; ++i) {
@@ -215,7 +217,7 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
       // a value that is not there must be zero: its probability is, but 0 x anything is not
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const vvec got = *(const vvec*)(vsrc + r * D);
+        const vvec got = HEADS ? stream_load((const vvec*)(vsrc + r * D)) : *(const vvec*)(vsrc + r * D);
         vreg[st][i][r] = (page >= 0 && kp0 + r <= pos_last) ? got : zero_v;
       }
     }
