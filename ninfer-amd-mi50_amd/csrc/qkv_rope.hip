@@ -64,8 +64,10 @@ __global__ __launch_bounds__(WAVES * 64) void qkv_rope_kernel(QkvRopeArgs a, int
 
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  // a wave's chunks of four steps lie side by side: it walks its part of every row in order
   const int steps = K / 32;
-  for (int c = wave; c * 4 < steps; c += WAVES) {
+  const int chunks = (steps + 3) / 4, per_wave = (chunks + WAVES - 1) / WAVES;
+  for (int c = wave * per_wave; c < min((wave + 1) * per_wave, chunks); ++c) {
     const int s0 = c * 4;
     if (s0 + 4 <= steps) {
       bf16x8 w[4], x[4];
