@@ -62,6 +62,23 @@ __global__ __launch_bounds__(WAVES * 64) void qkv_rope_kernel(QkvRopeArgs a, int
   const bool m_valid = mrow < a.T;
   const bf16* xrow = (const bf16*)a.x + (int64_t)(m_valid ? mrow : 0) * a.lda + 8 * j;
 
+  // The same weight rows as the loads see them: whole 128-byte lines, lane l at row
+  // 8 q + l / 8 (of the block's 16), byte 16 (l % 8) of a 128-byte piece; they reach the
+  // operand's layout through 2 KB of LDS per wave (as in the few-row product kernel).
+  const bf16* wline[2];
+  bool line_valid[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int R = 8 * q + (lane >> 3), p8 = R & 7;
+    line_valid[q] = p8 < pairs;
+    const int nn = head * D + d0 + min(p8, pairs - 1) + (R >> 3) * half;
+    wline[q] = (const bf16*)a.w + (int64_t)nn * K + 8 * (lane & 7);
+  }
+  __shared__ __attribute__((aligned(16))) unsigned char stage[WAVES * 2048];
+  unsigned char* my_stage = stage + wave * 2048;
+  const int st_write = ((lane >> 3) * 128) + 16 * ((lane & 7) ^ ((lane >> 3) & 7));   // + 1024 q
+  const int st_read = r * 128;   // + 16 * ((4 i + j) ^ (r % 8))
+
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   // a wave's chunks of four steps lie side by side: it walks its part of every row in order
@@ -70,14 +87,24 @@ __global__ __launch_bounds__(WAVES * 64) void qkv_rope_kernel(QkvRopeArgs a, int
   for (int c = wave * per_wave; c < min((wave + 1) * per_wave, chunks); ++c) {
     const int s0 = c * 4;
     if (s0 + 4 <= steps) {
-      bf16x8 w[4], x[4];
+      bf16x8 wl[2][2], x[4];   // [piece][q]
 #pragma unroll
-      for (int i = 0; i < 4; ++i) w[i] = w_valid ? *(const bf16x8*)(wrow + (s0 + i) * 32) : zero;
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+          wl[h][q] = line_valid[q] ? stream_load((const bf16x8*)(wline[q] + s0 * 32 + h * 64)) : zero;
 #pragma unroll
       for (int i = 0; i < 4; ++i) x[i] = m_valid ? *(const bf16x8*)(xrow + (s0 + i) * 32) : zero;
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[i], x[i], acc, 0, 0, 0);
+      for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) *(bf16x8*)(my_stage + st_write + 1024 * q) = wl[h][q];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const bf16x8 wf = *(const bf16x8*)(my_stage + st_read + 16 * ((4 * i + j) ^ (r & 7)));
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, x[2 * h + i], acc, 0, 0, 0);
+        }
+      }
     } else {
       for (int s = s0; s < steps; ++s) {
         bf16x8 w = w_valid ? *(const bf16x8*)(wrow + s * 32) : zero;
