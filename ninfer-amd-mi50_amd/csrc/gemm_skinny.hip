@@ -228,9 +228,13 @@ template <bool FULL_A, bool SW_A, typename TC_A, bool FULL_B, bool SW_B, typenam
           bool TWO_A = false>
 __global__ __launch_bounds__(1024) void gemm_skinny_pair_kernel(GemmArgs a, SkinnyPlan pa,
                                                                GemmArgs b, SkinnyPlan pb) {
-  __shared__ float red[16 * 2 * 256];
-  __shared__ __attribute__((aligned(16))) unsigned char stage[16 * 2048];
+  // LDS by the block's waves (the launch passes blockDim.x / 64 * 4 KB): 2 KB of partial sums
+  // (two sets of 256) and 2 KB of weight lines per wave; a fixed array for 16 waves would
+  // hold blocks of 4 waves down to two per CU
+  extern __shared__ __attribute__((aligned(16))) unsigned char pair_lds[];
   __shared__ int tile_info[3];
+  float* red = (float*)pair_lds;
+  unsigned char* stage = pair_lds + (blockDim.x >> 6) * 2048;
   const int wave = threadIdx.x >> 6;
   int id = blockIdx.x;
   const int blocks_b = pb.grid_x * pb.grid_y;
@@ -350,17 +354,18 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream) {
   }
   if (a.offsets && (long)pa.grid_x * pa.grid_y >= 2048) pb.waves = pa.waves;
   const int threads = 64 * max(pa.waves, pb.waves);
+  const size_t lds = (size_t)(threads / 64) * 4096;   // partial sums and weight lines, per wave
   const long blocks = (long)pa.grid_x * pa.grid_y + (long)pb.grid_x * pb.grid_y;
   NINFER_REQUIRE(blocks < (1L << 31), "gemm pair: %ld blocks are too many", blocks);
   if (!a.offsets)
     gemm_skinny_pair_kernel<false, false, float, false, true, bf16>
-        <<<(unsigned)blocks, threads, 0, stream>>>(a, pa, b, pb);
+        <<<(unsigned)blocks, threads, lds, stream>>>(a, pa, b, pb);
   else if (pa.two)
     gemm_skinny_pair_kernel<true, false, bf16, false, false, bf16, true>
-        <<<(unsigned)blocks, threads, 0, stream>>>(a, pa, b, pb);
+        <<<(unsigned)blocks, threads, lds, stream>>>(a, pa, b, pb);
   else
     gemm_skinny_pair_kernel<true, false, bf16, false, false, bf16>
-        <<<(unsigned)blocks, threads, 0, stream>>>(a, pa, b, pb);
+        <<<(unsigned)blocks, threads, lds, stream>>>(a, pa, b, pb);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

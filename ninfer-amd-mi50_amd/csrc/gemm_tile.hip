@@ -91,10 +91,10 @@ __global__ __launch_bounds__(NW * 64, OCC) void gemm_tile_kernel(GemmArgs a) {
   // (Grouped: the start depends on the expert, not on the row tile, so that a row's sum has the
   // same order whichever tile of its expert the grouping put it in.)
   const int phase = (int)(((a.offsets ? group : bx) * 5u + by * 3u) % (unsigned)nk);
-  // An expert whose rows fit one tile has its W panel read by this block alone: non-temporal
-  // loads, so that they do not push out of L2 the rows of A that the expert's other feature
-  // tiles read again.
-  const bool w_once = a.offsets != nullptr && row_end - a.offsets[group] <= TM;
+  // An expert whose rows fit one tile (or a dense product of one row tile) has its W panel
+  // read by this block alone: non-temporal loads, so that they do not push out of L2 the rows
+  // of A that the other feature tiles read again.
+  const bool w_once = a.offsets != nullptr ? row_end - a.offsets[group] <= TM : a.M <= TM;
   // P register stages: the loads of k tile t + P are issued while tile t is multiplied
   bf16x8 xreg[P][XV], wreg[P][WV];
   auto load_tile = [&](int st, int k_lin) {   // k_lin: the tile's place in this block's walk, times TK

@@ -125,11 +125,12 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
     for (int i = 0; i < NL; ++i)
       __builtin_amdgcn_global_load_lds((gptr)(xsrc[i] + kt * TK), (lptr)(buf + i * 4096), 16, 0, 0);
   };
-  // An expert whose rows fit one tile has its W panel read by this block alone: those loads
+  // An expert whose rows fit one tile (or a dense product of one row tile) has its W panel read
+  // by this block alone: those loads
   // are marked non-temporal (the last argument: 2), so that they do not push the rows of A,
   // which the expert's other feature tiles read again, out of L2 (6 to 9% at 137 rows per
   // expert; with two tiles per expert the second finds the panel in L2 and the mark costs 4%).
-  const bool w_once = a.offsets != nullptr && row_end - a.offsets[group] <= TM;
+  const bool w_once = a.offsets != nullptr ? row_end - a.offsets[group] <= TM : a.M <= TM;
   auto issue_w = [&](int t, int w_off) {
     unsigned char* buf = smem + W_BASE + w_off + wave * 1024;
     int kt = t + phase;
