@@ -405,6 +405,12 @@ class HipOps:
         are valid after the block, not inside it."""
         return _Together(self)
 
+    def wants_beside(self, rows: int) -> bool:
+        """Is independent work of this many rows worth the second stream? Not while a graph
+        is being captured: its steps have few rows each, and a fork inside a capture is
+        one more thing a replay would have to get right."""
+        return rows >= self.beside_min_rows and not torch.cuda.is_current_stream_capturing()
+
     def beside(self):
         """Context manager for work that nothing on the current stream waits for until
         `join()`: it runs on a second stream, so that the device can fill with its blocks

@@ -28,6 +28,9 @@ class PlainOps:
 
     beside_min_rows = 8   # low, so that the host tests walk the many-row branch too
 
+    def wants_beside(self, rows):
+        return rows >= self.beside_min_rows
+
     def beside(self):
         """Work for a second stream: here it simply runs where it is called."""
         return contextlib.nullcontext()
