@@ -202,10 +202,12 @@ def main() -> int:
     def profile_calls(label: str, chunks) -> dict:
         """Microseconds by kind of kernel call for one eager step: every call of the kernel
         library is bracketed by device events (calls inside `together()` are launched when
-        it ends and are timed there, as one kind). The reference prints such a table per
-        phase (src/models/model.hip:1066-1081)."""
+        it ends and are timed there, as one kind). Everything runs on one stream here (a long
+        portion's shared expert otherwise runs beside the routed path, and times would
+        overlap). The reference prints such a table per phase (src/models/model.hip:1066-1081)."""
         ops = runner.ops
         spans = []
+        one_stream, ops.beside_min_rows = ops.beside_min_rows, 1 << 30
 
         def kind(name, a):
             if name in ("linear", "swiglu_linear"):
@@ -247,6 +249,7 @@ def main() -> int:
             for n in names:
                 setattr(ops, n, saved[n])
             runner.options.use_graph = use_graph
+            ops.beside_min_rows = one_stream
         table = {}
         for k_, s, e in spans:
             calls, us = table.get(k_, (0, 0.0))
