@@ -7,11 +7,14 @@
 // l % 16, k = 8 (l / 16) .. +7, i.e. 16 contiguous bytes), the activations are
 // the B operand (lane l supplies token l % 16, same k), so the accumulator
 // holds a 16 x 16 tile out[feature 4 (l / 16) + v][token l % 16]. The K range is
-// split over the waves of the block in chunks of 128; partial tiles meet in LDS
-// and are summed in wave order, so the result does not depend on timing.
-// Activations are read straight from global memory (they stay in cache: few
-// rows), weights stream through registers with four 16-byte loads in flight
-// per lane and chunk.
+// split over the waves of the block, each wave a contiguous part that it walks
+// in chunks of 128; partial tiles meet in LDS and are summed in wave order, so
+// the result does not depend on timing. Activations are read straight from
+// global memory (they stay in cache: few rows). Weights are loaded as whole
+// 128-byte lines (8 rows per instruction, four instructions in flight per
+// chunk), non-temporal, and reach the operand's layout through 2 KB of LDS per
+// wave: read that way they stream at 6.4 TB/s, against 5.5 when every lane
+// loads the 16 bytes of its operand itself.
 //
 // A dense product whose 16-feature tiles would be few is cut into tiles of
 // fewer features (some of each matrix instruction's rows stay empty, which
