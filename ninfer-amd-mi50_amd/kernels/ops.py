@@ -110,9 +110,10 @@ class _Beside:
         if ops._side is None:
             ops._side = torch.cuda.Stream()   # default priority
             ops._side_events = (torch.cuda.Event(), torch.cuda.Event())
-        if ops._side_open:
-            raise KernelError("beside(): join() the block before first")
         self.main = torch.cuda.current_stream()
+        if ops._side_open:   # a block that nobody joined (a step that failed half-way): join it now
+            self.main.wait_event(ops._side_events[1])
+            ops._side_open = False
         ops._side_events[0].record(self.main)
         ops._side.wait_event(ops._side_events[0])
         torch.cuda.set_stream(ops._side)
