@@ -7,15 +7,15 @@
 // running max, sum and output of its own that are merged at the end. So every
 // SIMD holds two waves, and the softmax arithmetic of one overlaps the matrix
 // products of the other. Keys and values are walked in tiles of
-// 64 aligned to absolute positions, through LDS: K as stored ([key][d]), V
-// transposed ([d][key]) so that both products read their contraction index
-// contiguously. With v_mfma_f32_32x32x16_bf16 the wave computes
+// 64 aligned to absolute positions, through LDS, both as stored ([key][d]). With
+// v_mfma_f32_32x32x16_bf16 the wave computes
 //   S^T[key][q] = K Q^T      (A = K rows from LDS, B = Q held in registers)
 // whose accumulator layout gives lane l the scores of query l % 32 for keys
 // 8 (v / 4) + 4 (l / 32) + v % 4 of every 32-key block: the softmax of a query
 // runs in the two lanes that share l % 32 (one cross-lane step), and the
 // probabilities, packed to bf16 in place, are already the B operand of
-//   O^T[d][q] += V^T P^T     (A = V^T rows from LDS)
+//   O^T[d][q] += V^T P^T     (A = V^T rows: ds_read_b64_tr_b16 hands a lane four keys of one
+//                             dim out of the [key][d] tile, no transposing store needed)
 // if the contraction index is numbered the way the lanes hold it; so
 // probabilities never leave registers, and the running max and sum of a query
 // live in the lanes that hold its output column. Online softmax as in the
@@ -42,6 +42,8 @@ namespace ninfer {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) short4v lds_short4;
 
 constexpr int PK = 64;   // keys per tile
 
@@ -55,8 +57,9 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
   constexpr int KS = D / 16;        // k-steps of Q K^T
   constexpr int DB = D / 32;        // 32-row blocks of O^T
   constexpr int KPAD = D + 8;       // bf16 per K row in LDS
-  constexpr int VPAD = PK + 4;      // bf16 per V^T row in LDS: 8-byte reads of 32 rows spread over the banks
-  constexpr int K_TILE = PK * KPAD, V_TILE = D * VPAD;   // bf16 of a tile in LDS
+  constexpr int VROW = D + 16;      // bf16 per V row in LDS: 32 bytes more than a row, so that the 4 keys x
+                                    // 4 dim quads that 16 lanes of a transposing read touch fall on 32 banks
+  constexpr int K_TILE = PK * KPAD, V_TILE = PK * VROW;   // bf16 of a tile in LDS
   constexpr bool EARLY = NQ == 4;   // 512 threads stage half as much each: registers to spare
   constexpr int MERGE = 2 + DB * 16 + 1;                   // floats a lane hands over at the end (odd stride)
   constexpr int TILES_BYTES = 2 * (K_TILE + V_TILE) * 2, MERGE_BYTES = NQ * 64 * MERGE * 4;
@@ -68,6 +71,9 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int c = lane & 31, j = lane >> 5;
+  // this lane's part in a transposing read of V (see read_values): group lane / 16 holds dims
+  // 16 (group % 2) .. + 15 and keys 4 (group / 2) .. + 3
+  const int tr_key = 4 * (lane >> 5) + ((lane & 15) >> 2), tr_dim = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
   const int group = a.Hq / a.Hkv;
   int row0, n_rows, seq, g, h, pos_first, pos_last, lo_first, chunk_id = 0;
   if constexpr (HEADS) {
@@ -146,16 +152,11 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
   const float scale2 = a.scale * 1.44269504088896f;
   float m = -1e30f, l = 0.f;
 
-  // global -> LDS mapping. K: thread loads 16 bytes (8 dims) of a key row.
-  // V: thread loads a 4-key x 8-dim block and stores it transposed.
+  // global -> LDS mapping, the same for K and V: thread loads 16 bytes (8 dims) of a key's row.
+  // Both lie in LDS as they lie in the cache ([key][d]); the output products read V through the
+  // transposing LDS read (ds_read_b64_tr_b16), which hands a lane four keys of one dim.
   constexpr int K_VECS = PK * D / 8;                  // 16-byte vectors in a K tile
   constexpr int K_PER_THREAD = (K_VECS + NT - 1) / NT;
-  // V: blocks of 4 keys x VD dims; 8 dims (16-byte loads) unless that leaves threads without
-  // a block, then 4 (8-byte loads, every thread busy)
-  constexpr int VD = (PK / 4) * (D / 8) < NT ? 4 : 8;
-  typedef __bf16 vvec __attribute__((ext_vector_type(VD)));
-  constexpr int V_BLOCKS = (PK / 4) * (D / VD);       // 4 x VD blocks in a V tile
-  constexpr int V_PER_THREAD = (V_BLOCKS + NT - 1) / NT;
   static_assert(K_VECS % NT == 0, "tile does not divide over the block");
 
   // A tile's keys and values travel global -> registers (stage i % NS) -> LDS. Tile i is
@@ -163,12 +164,9 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
   // the other buffer, the loads of tile i + 1 + NS are issued into those registers,
   // and the page numbers of tile i + 1 + 2 NS are fetched: no load waits for another
   // inside the loop.
-  bf16x8 kreg[NS][K_PER_THREAD];
-  vvec vreg[NS][V_PER_THREAD][4];
-  int kpage[NS][K_PER_THREAD], vpage[NS][V_PER_THREAD];
-  vvec zero_v;
-#pragma unroll
-  for (int d = 0; d < VD; ++d) zero_v[d] = 0;
+  bf16x8 kreg[NS][K_PER_THREAD], vreg[NS][K_PER_THREAD];
+  int kpage[NS][K_PER_THREAD];   // K and V of a key lie at the same place of their pools
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   // Every load below is unconditional (a select replaces what is not there by zeros): a
   // load under a condition would have to be waited for where the condition ends.
   auto load_pages = [&](int st, int t0) {
@@ -177,70 +175,40 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
       int kp = t0 + (tid + i * NT) / (D / 8);
       kpage[st][i] = bt[min(kp, pos_last) >> ps_shift];   // always a table entry of the request
     }
-#pragma unroll
-    for (int i = 0; i < V_PER_THREAD; ++i) {
-      int blk = (tid + i * NT) % V_BLOCKS;     // threads beyond the tile repeat a block and store nothing
-      int kp = t0 + 4 * (blk % (PK / 4));      // four keys of one page (the page size is a multiple of 4)
-      vpage[st][i] = bt[min(kp, pos_last) >> ps_shift];
-    }
   };
   // A tile starts at a multiple of the page size, so the place of a thread's piece inside
   // its page is the same in every tile: address = pool + page * page_stride + in_page.
   const int64_t page_stride = ((int64_t)Hkv << ps_shift) * D;
-  int64_t k_in_page[K_PER_THREAD], v_in_page[V_PER_THREAD];
+  int64_t k_in_page[K_PER_THREAD];
 #pragma unroll
   for (int i = 0; i < K_PER_THREAD; ++i) {
     const int vec = tid + i * NT;
     k_in_page[i] = (((int64_t)g << ps_shift) + ((vec / (D / 8)) & ps_mask)) * D + 8 * (vec % (D / 8));
-  }
-#pragma unroll
-  for (int i = 0; i < V_PER_THREAD; ++i) {
-    const int blk = (tid + i * NT) % V_BLOCKS;
-    v_in_page[i] = (((int64_t)g << ps_shift) + ((4 * (blk % (PK / 4))) & ps_mask)) * D + VD * (blk / (PK / 4));
   }
   auto load_regs = [&](int st, int t0) {
 #pragma unroll
     for (int i = 0; i < K_PER_THREAD; ++i) {
       // For a key that is not there, a row of the last key's page (beyond it) or of the
       // pool's first page (a page given back) is read in its place. Such a key lies in a
-      // block that is masked, and the mask replaces its scores whatever they are.
-      const bf16x8* src = (const bf16x8*)(kpool + max(kpage[st][i], 0) * page_stride + k_in_page[i]);
+      // block that is masked, and the mask replaces its scores whatever they are; its value
+      // must be zero: its probability is, but 0 x anything is not.
+      const int page = kpage[st][i];
+      const int64_t at = max(page, 0) * page_stride + k_in_page[i];
+      const int kp = t0 + (tid + i * NT) / (D / 8);
       // decoding reads every key once a step; a prompt's keys serve many blocks of rows from L2
-      kreg[st][i] = HEADS ? stream_load(src) : *src;
-    }
-#pragma unroll
-    for (int i = 0; i < V_PER_THREAD; ++i) {
-      const int blk = (tid + i * NT) % V_BLOCKS;
-      const int page = vpage[st][i];
-      const bf16* vsrc = vpool + max(page, 0) * page_stride + v_in_page[i];
-      const int kp0 = t0 + 4 * (blk % (PK / 4));
-      // a value that is not there must be zero: its probability is, but 0 x anything is not
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const vvec got = HEADS ? stream_load((const vvec*)(vsrc + r * D)) : *(const vvec*)(vsrc + r * D);
-        vreg[st][i][r] = (page >= 0 && kp0 + r <= pos_last) ? got : zero_v;
-      }
+      kreg[st][i] = HEADS ? stream_load((const bf16x8*)(kpool + at)) : *(const bf16x8*)(kpool + at);
+      const bf16x8 got = HEADS ? stream_load((const bf16x8*)(vpool + at)) : *(const bf16x8*)(vpool + at);
+      vreg[st][i] = (page >= 0 && kp <= pos_last) ? got : zero8;
     }
   };
   auto store_regs = [&](int st, int buf) {
     bf16* k_s = k_lds + buf * K_TILE;
-    bf16* vt_s = vt_lds + buf * V_TILE;
+    bf16* v_s = vt_lds + buf * V_TILE;
 #pragma unroll
     for (int i = 0; i < K_PER_THREAD; ++i) {
       int vec = tid + i * NT;
       *(bf16x8*)(k_s + (vec / (D / 8)) * KPAD + 8 * (vec % (D / 8))) = kreg[st][i];
-    }
-#pragma unroll
-    for (int i = 0; i < V_PER_THREAD; ++i) {
-      int blk = tid + i * NT;
-      if (blk < V_BLOCKS) {
-        int kg = blk % (PK / 4), dv = blk / (PK / 4);
-#pragma unroll
-        for (int d = 0; d < VD; ++d) {
-          bf16x4 col = {vreg[st][i][0][d], vreg[st][i][1][d], vreg[st][i][2][d], vreg[st][i][3][d]};
-          *(bf16x4*)(vt_s + (VD * dv + d) * VPAD + 4 * kg) = col;
-        }
-      }
+      *(bf16x8*)(v_s + (vec / (D / 8)) * VROW + 8 * (vec % (D / 8))) = vreg[st][i];
     }
   };
 
@@ -281,11 +249,17 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
     }
     // the values: with EARLY read here, while the vector units form the probabilities
     bf16x8 vf[DB][NKB][2];
+    // The transposing read works in groups of 16 lanes: lane s of a group fetches 8 bytes from
+    // an address of its own, and lane i receives element i % 4 of what lanes i / 4 + 4 v
+    // fetched, v = 0 .. 3. With lane s at key v = s / 4, dims 4 (s % 4) .. + 3 of the group's
+    // 16 dims, lane i gets four consecutive keys of dim i: half of the operand's 8 keys.
     auto read_values = [&](int db, int kb, int hs) {
-      const bf16* vr = vt_s + (db * 32 + c) * VPAD + 32 * (NKB * kh + kb) + 16 * hs + 4 * j;
-      bf16x4 lo4 = *(const bf16x4*)vr;
-      bf16x4 hi4 = *(const bf16x4*)(vr + 8);
-      vf[db][kb][hs] = (bf16x8){lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+      const bf16* vr = vt_s + (32 * (NKB * kh + kb) + 16 * hs + tr_key) * VROW + db * 32 + tr_dim;
+      const short4v lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)vr);
+      const short4v hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vr + 8 * VROW));
+      typedef short short8v __attribute__((ext_vector_type(8)));
+      const short8v both = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+      vf[db][kb][hs] = __builtin_bit_cast(bf16x8, both);
     };
     if constexpr (EARLY) {
 #pragma unroll
@@ -450,7 +424,7 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
 bool attention_decode_heads_takes(const AttnArgs& a) {
   const int group = a.Hq / a.Hkv;
   return a.dtype == kBF16 && (a.D == 64 || a.D == 128) && a.q_stride % 8 == 0 &&
-         PK % a.page_size == 0 && a.page_size % 4 == 0 && group >= 3 && group <= 32 && a.workspace != nullptr &&
+         PK % a.page_size == 0 && group >= 3 && group <= 32 && a.workspace != nullptr &&
          a.row_seq != nullptr;
 }
 
@@ -471,7 +445,7 @@ int attention_decode_heads(const AttnArgs& a, int chunk, int n_chunks, hipStream
 
 bool attention_prefill_takes(const AttnArgs& a) {
   return a.dtype == kBF16 && (a.D == 64 || a.D == 128) && a.q_stride % 8 == 0 &&
-         PK % a.page_size == 0 && a.page_size % 4 == 0 && a.seq_row_start != nullptr;
+         PK % a.page_size == 0 && a.seq_row_start != nullptr;
 }
 
 template <int NQ>
