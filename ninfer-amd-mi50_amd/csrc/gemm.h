@@ -104,6 +104,10 @@ bool gemm_skinny_takes(const GemmArgs& a);
 int gemm_skinny(const GemmArgs& a, hipStream_t stream);
 bool gemm_skinny_pair_takes(const GemmArgs& a, const GemmArgs& b);
 int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream);
+struct RouteArgs;
+bool gemm_skinny_route_pair_takes(const GemmArgs& a, const GemmArgs& b, const RouteArgs& rt);
+int gemm_skinny_route_pair(const GemmArgs& a, const GemmArgs& b, const RouteArgs& rt,
+                           hipStream_t stream);
 bool gemm_tile_takes(const GemmArgs& a);
 int gemm_tile(const GemmArgs& a, hipStream_t stream);
 int gemm_generic(const GemmArgs& a, hipStream_t stream);

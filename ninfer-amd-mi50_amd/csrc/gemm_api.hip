@@ -1,5 +1,6 @@
 // Entry point of the product family: checks the arguments and picks a kernel.
 #include "gemm.h"
+#include "moe_route.h"
 
 using namespace ninfer;
 
@@ -42,4 +43,36 @@ extern "C" int ninfer_gemm_pair(const GemmArgs* a, const GemmArgs* b, int force_
   rc = ninfer_gemm(a, force_generic, stream);
   if (rc) return rc;
   return ninfer_gemm(b, force_generic, stream);
+}
+
+// The pair above, and the routing of the rows by the logits that product `a` writes
+// ([T, >= E] 32-bit: columns beyond the experts' are not the router's). One launch where the
+// few-row kernel holds the router's product in one block; otherwise the products, then the
+// routing kernels.
+extern "C" int ninfer_gemm_pair_route(const GemmArgs* a, const GemmArgs* b, const RouteArgs* rt,
+                                      int force_generic, hipStream_t stream) {
+  int rc = gemm_check(*a);
+  if (rc) return rc;
+  rc = gemm_check(*b);
+  if (rc) return rc;
+  NINFER_REQUIRE(!a->offsets && a->out_dtype == kF32 && a->N >= rt->E && a->ldc >= rt->E,
+                 "gemm_pair_route: the first product must be dense with 32-bit logits of %d experts",
+                 rt->E);
+  NINFER_REQUIRE((!rt->tiles16) == (!rt->tiles64) && (!rt->tiles16) == (!rt->tile_counts),
+                 "gemm_pair_route: tile lists come together or not at all");
+  NINFER_REQUIRE(rt->big_rows == 64 || rt->big_rows == 128 || rt->big_rows == 256,
+                 "gemm_pair_route: big tiles of %d rows", rt->big_rows);
+  if (!force_generic && !many_rows(*a) && !many_rows(*b) && gemm_skinny_route_pair_takes(*a, *b, *rt))
+    return gemm_skinny_route_pair(*a, *b, *rt, stream);
+  rc = ninfer_gemm_pair(a, b, force_generic, stream);
+  if (rc) return rc;
+  const float* logits = (const float*)a->C;
+  if (a->M <= 16)
+    return ninfer_moe_route_small(logits, a->ldc, a->M, rt->E, rt->k, rt->renorm, rt->ids, rt->wts,
+                                  rt->offsets, rt->order, rt->tiles16, rt->tiles64,
+                                  rt->tile_counts, rt->big_rows, stream);
+  rc = ninfer_router_topk(logits, a->ldc, a->M, rt->E, rt->k, rt->renorm, rt->ids, rt->wts, stream);
+  if (rc) return rc;
+  return ninfer_moe_align(rt->ids, a->M * rt->k, rt->E, rt->offsets, rt->order, rt->tiles16,
+                          rt->tiles64, rt->tile_counts, rt->big_rows, stream);
 }

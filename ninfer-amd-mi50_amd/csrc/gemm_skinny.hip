@@ -27,6 +27,7 @@
 // src/ops/gemv.hip:52-93) or one library call per expert
 // (src/models/model.hip:355-427).
 #include "gemm.h"
+#include "moe_route.h"
 
 namespace ninfer {
 
@@ -34,6 +35,78 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int SM = 16;  // rows of A per tile
+
+// What a wave multiplies: SETS sets of 16 weight rows against up to 16 rows of A.
+template <int SETS>
+struct SkinnyOperands {
+  const bf16* wrow[SETS];       // lane (r, j): weight row r of the set at k = 8 j (the operand's view)
+  const bf16* wline[SETS][2];   // lane l: row 8 q + l / 8 at byte 16 (l % 8) (whole lines)
+  bool line_valid[2];
+  bool w_valid;                 // lanes of rows the tile does not have load nothing
+  const bf16* xrow;             // lane (r, j): row r of A at k = 8 j
+  bool m_valid;
+};
+
+// One wave's part of the K range: `waves` waves split K in chunks of four steps (256 bytes
+// of a row); a wave's chunks lie side by side, so that it walks its part of every row from
+// one end to the other (measured with loads alone: 5.9 TB/s, against 5.6 with the waves'
+// chunks interleaved). `my_stage`: this wave's 2 KB of LDS, 16 rows of 128 bytes, the
+// 16-byte units of row R stored in the order u ^ (R % 8), so that the writes (a row per 8
+// lanes) and the fragment reads (lane (r, j): row r, unit 4 i + j) both spread evenly over
+// the banks.
+template <int SETS>
+__device__ __forceinline__ void skinny_walk(const SkinnyOperands<SETS>& o, int K, int wave,
+                                            int waves, unsigned char* my_stage, int lane,
+                                            f32x4 (&acc)[SETS]) {
+  const int r = lane & 15, j = lane >> 4;
+  const int st_write = ((lane >> 3) * 128) + 16 * ((lane & 7) ^ ((lane >> 3) & 7));   // + 1024 q
+  const int st_read = r * 128;   // + 16 * ((4 i + j) ^ (r % 8))
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int steps = K / 32;
+  const int chunks = (steps + 3) / 4, per_wave = (chunks + waves - 1) / waves;
+  for (int c = wave * per_wave; c < min((wave + 1) * per_wave, chunks); ++c) {
+    const int s0 = c * 4;
+    if (s0 + 4 <= steps) {
+      // A chunk is two pieces of 128 bytes per row. Weights are read once and by this wave
+      // alone: whole lines, 8 rows per instruction, marked non-temporal (measured with loads
+      // alone, with each wave walking its part of the rows in order: 6.6 TB/s, against 5.9
+      // when every lane loads its own 16 bytes of the matrix instruction's operand, 64 bytes
+      // of a row per instruction). They reach the operand's layout through LDS.
+      bf16x8 wl[SETS][2][2], x[4];   // [set][piece][q]
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int s = 0; s < SETS; ++s)
+#pragma unroll
+          for (int q = 0; q < 2; ++q)
+            wl[s][h][q] = o.line_valid[q] ? stream_load((const bf16x8*)(o.wline[s][q] + s0 * 32 + h * 64))
+                                          : zero;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] = o.m_valid ? *(const bf16x8*)(o.xrow + (s0 + i) * 32) : zero;
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int s = 0; s < SETS; ++s) {
+#pragma unroll
+          for (int q = 0; q < 2; ++q) *(bf16x8*)(my_stage + st_write + 1024 * q) = wl[s][h][q];
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const bf16x8 wf = *(const bf16x8*)(my_stage + st_read + 16 * ((4 * i + j) ^ (r & 7)));
+            acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, x[2 * h + i], acc[s], 0, 0, 0);
+          }
+        }
+    } else {
+      for (int st = s0; st < steps; ++st) {
+        bf16x8 x = o.m_valid ? *(const bf16x8*)(o.xrow + st * 32) : zero;
+#pragma unroll
+        for (int s = 0; s < SETS; ++s) {
+          bf16x8 w = o.w_valid ? *(const bf16x8*)(o.wrow[s] + st * 32) : zero;
+          acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, x, acc[s], 0, 0, 0);
+        }
+      }
+    }
+  }
+}
 
 // The work of one block: tile (bx, by) of the product `a`. WAVES > 0 fixes the waves that
 // share the K range at compile time; WAVES == 0 takes them from `waves_arg` (waves of the
@@ -80,91 +153,34 @@ __device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, in
   const int K = a.K;
 
   const bf16* W = (const bf16*)a.W + (int64_t)group * a.w_group_stride;
+  SkinnyOperands<SETS> o;
+  o.w_valid = w_valid;
   // set s: feature group s / HALVES; with SwiGLU the odd sets are the up rows, N rows further
-  const bf16* wrow[SETS];
 #pragma unroll
   for (int s = 0; s < SETS; ++s)
-    wrow[s] = W + ((int64_t)min(n0 + 16 * (s / HALVES) + r, a.N - 1) + (s % HALVES ? a.N : 0)) * K +
-              8 * j;
-
+    o.wrow[s] = W + ((int64_t)min(n0 + 16 * (s / HALVES) + r, a.N - 1) + (s % HALVES ? a.N : 0)) * K +
+                8 * j;
   // The same rows as the loads see them: whole 128-byte lines. Lane l reads 16 bytes at row
   // 8 q + l / 8, byte 16 (l % 8) of a 128-byte piece (q = 0, 1).
-  const bf16* wline[SETS][2];
-  bool line_valid[2];
 #pragma unroll
   for (int q = 0; q < 2; ++q) {
     const int R = 8 * q + (lane >> 3);
-    line_valid[q] = FULL || R < rows;
+    o.line_valid[q] = FULL || R < rows;
 #pragma unroll
     for (int s = 0; s < SETS; ++s)
-      wline[s][q] = W + ((int64_t)min(n0 + 16 * (s / HALVES) + R, a.N - 1) + (s % HALVES ? a.N : 0)) * K +
-                    8 * (lane & 7);
+      o.wline[s][q] = W + ((int64_t)min(n0 + 16 * (s / HALVES) + R, a.N - 1) + (s % HALVES ? a.N : 0)) * K +
+                      8 * (lane & 7);
   }
-  // this wave's 2 KB of LDS: 16 rows of 128 bytes, the 16-byte units of row R stored in the
-  // order u ^ (R % 8), so that the writes (a row per 8 lanes) and the fragment reads (lane
-  // (r, j): row r, unit 4 i + j) both spread evenly over the banks
-  unsigned char* my_stage = stage + wave * 2048;
-  const int st_write = ((lane >> 3) * 128) + 16 * ((lane & 7) ^ ((lane >> 3) & 7));   // + 1024 q
-  const int st_read = r * 128;   // + 16 * ((4 i + j) ^ (r % 8))
-
   const int mrow = row0 + r;
-  const bool m_valid = mrow < row_end;
+  o.m_valid = mrow < row_end;
   int64_t a_row = 0;
-  if (m_valid) a_row = a.a_index ? a.a_index[mrow] / a.a_div : mrow;
-  const bf16* xrow = (const bf16*)a.A + a_row * a.lda + 8 * j;
+  if (o.m_valid) a_row = a.a_index ? a.a_index[mrow] / a.a_div : mrow;
+  o.xrow = (const bf16*)a.A + a_row * a.lda + 8 * j;
 
   f32x4 acc[SETS];
 #pragma unroll
   for (int s = 0; s < SETS; ++s) acc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-
-  // The waves split K in chunks of four steps (256 bytes of a row); a wave's chunks lie side by
-  // side, so that it walks its part of every row from one end to the other (measured with
-  // loads alone: 5.9 TB/s, against 5.6 with the waves' chunks interleaved).
-  const int steps = K / 32;
-  const int chunks = (steps + 3) / 4, per_wave = (chunks + waves - 1) / waves;
-  for (int c = wave * per_wave; c < min((wave + 1) * per_wave, chunks); ++c) {
-    const int s0 = c * 4;
-    if (s0 + 4 <= steps) {
-      // A chunk is two pieces of 128 bytes per row. Weights are read once and by this wave
-      // alone: whole lines, 8 rows per instruction, marked non-temporal (measured with loads
-      // alone, with each wave walking its part of the rows in order: 6.6 TB/s, against 5.9
-      // when every lane loads its own 16 bytes of the matrix instruction's operand, 64 bytes
-      // of a row per instruction). They reach the operand's layout through LDS.
-      bf16x8 wl[SETS][2][2], x[4];   // [set][piece][q]
-#pragma unroll
-      for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int s = 0; s < SETS; ++s)
-#pragma unroll
-          for (int q = 0; q < 2; ++q)
-            wl[s][h][q] = line_valid[q] ? stream_load((const bf16x8*)(wline[s][q] + s0 * 32 + h * 64))
-                                        : zero;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) x[i] = m_valid ? *(const bf16x8*)(xrow + (s0 + i) * 32) : zero;
-#pragma unroll
-      for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int s = 0; s < SETS; ++s) {
-#pragma unroll
-          for (int q = 0; q < 2; ++q) *(bf16x8*)(my_stage + st_write + 1024 * q) = wl[s][h][q];
-#pragma unroll
-          for (int i = 0; i < 2; ++i) {
-            const bf16x8 wf = *(const bf16x8*)(my_stage + st_read + 16 * ((4 * i + j) ^ (r & 7)));
-            acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, x[2 * h + i], acc[s], 0, 0, 0);
-          }
-        }
-    } else {
-      for (int st = s0; st < steps; ++st) {
-        bf16x8 x = m_valid ? *(const bf16x8*)(xrow + st * 32) : zero;
-#pragma unroll
-        for (int s = 0; s < SETS; ++s) {
-          bf16x8 w = w_valid ? *(const bf16x8*)(wrow[s] + st * 32) : zero;
-          acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, x, acc[s], 0, 0, 0);
-        }
-      }
-    }
-  }
+  skinny_walk<SETS>(o, K, wave, waves, stage + wave * 2048, lane, acc);
 
   // partial tiles -> LDS, element (feature f, token m) of set s at [m * 16 + f]
 #pragma unroll
@@ -251,6 +267,88 @@ __global__ __launch_bounds__(1024) void gemm_skinny_pair_kernel(GemmArgs a, Skin
     skinny_block<0, FULL_A, SW_A, TC_A, TWO_A>(a, pa.rows, pa.waves, id % pa.grid_x,
                                                id / pa.grid_x, red, stage, tile_info);
   }
+}
+
+// A router's logits and the routing they decide, by one block: the product `a` (dense, at
+// most 16 rows, at most kRouteMaxFeatures features, 32-bit out) is small enough for one
+// block, whose 16 waves share it as feature groups of 16 x parts of the K range; the block
+// then holds every logit of every row and routes the rows itself (softmax, top-k, grouping
+// by expert) out of LDS. As a kernel of its own the routing is a launch and a chain of
+// dependent loads between the router's product and the experts' first one.
+// `red`: 16 x 256 floats; `stage`: 32 KB (the waves' weight lines, then logits, counters
+// and chosen experts). Every thread of the block must call.
+constexpr int kRouteMaxFeatures = 80;
+
+template <int NPL>
+__device__ __forceinline__ void skinny_route_block(const GemmArgs& a, const RouteArgs& rt,
+                                                   float* red, unsigned char* stage) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  const int r = lane & 15, j = lane >> 4;
+  const int N = a.N, K = a.K, T = a.M;
+  const int groups = (N + 15) / 16, parts = waves / groups;
+  const int g = wave / parts, part = wave % parts;   // waves beyond groups x parts have no share
+  if (g < groups) {
+    const int n0 = 16 * g, rows = min(16, N - n0);
+    const bf16* W = (const bf16*)a.W;
+    SkinnyOperands<1> o;
+    o.w_valid = r < rows;
+    o.wrow[0] = W + (int64_t)min(n0 + r, N - 1) * K + 8 * j;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int R = 8 * q + (lane >> 3);
+      o.line_valid[q] = R < rows;
+      o.wline[0][q] = W + (int64_t)min(n0 + R, N - 1) * K + 8 * (lane & 7);
+    }
+    o.m_valid = r < T;
+    o.xrow = (const bf16*)a.A + (int64_t)(o.m_valid ? r : 0) * a.lda + 8 * j;
+    f32x4 acc[1] = {f32x4{0.f, 0.f, 0.f, 0.f}};
+    skinny_walk<1>(o, K, part, parts, stage + wave * 2048, lane, acc);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave * 256 + r * 16 + 4 * j + v] = acc[0][v];
+  }
+  __syncthreads();   // the partial tiles are complete, and the weight lines' LDS is free
+  // logit (row m, feature n): the parts of its group summed in their order; kept in LDS and
+  // written out (the caller may read further columns than the experts', as a gate's logit)
+  const int ldl = 16 * groups;
+  float* logits_s = (float*)stage;
+  for (int i = threadIdx.x; i < T * ldl; i += blockDim.x) {
+    const int m = i / ldl, n = i % ldl;
+    float sum = 0.f;
+    for (int p = 0; p < parts; ++p) sum += red[((n >> 4) * parts + p) * 256 + m * 16 + (n & 15)];
+    logits_s[i] = sum;
+    if (n < N) ((float*)a.C)[(int64_t)m * a.ldc + n] = sum;
+  }
+  __syncthreads();
+  int* cnt = (int*)(logits_s + 16 * ldl);   // E + 1 counters, then the chosen experts
+  int* ids_s = cnt + rt.E + 1;
+  for (int t = wave; t < T; t += waves) {
+    const int mine = route_row<NPL>(logits_s + t * ldl, rt.E, rt.k, rt.renorm, rt.ids + (int64_t)t * rt.k,
+                                    rt.wts + (int64_t)t * rt.k, lane);
+    if (lane < rt.k) ids_s[t * rt.k + lane] = mine;
+  }
+  __syncthreads();
+  align_block(ids_s, T * rt.k, rt.E, rt.offsets, rt.order, rt.tiles16, rt.tiles64, rt.tile_counts,
+              rt.big_rows, cnt);
+}
+
+// The first block is the router's (product `a` and routing `rt`), the others are the tiles of
+// the dense product `b`, which does not depend on it (a shared expert's gate and up).
+template <bool FULL_B, bool SW_B, typename TC_B>
+__global__ __launch_bounds__(1024) void gemm_skinny_route_pair_kernel(GemmArgs a, RouteArgs rt,
+                                                                     GemmArgs b, SkinnyPlan pb) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char pair_lds[];   // 16 waves x 4 KB
+  __shared__ int tile_info[3];
+  float* red = (float*)pair_lds;
+  unsigned char* stage = pair_lds + (blockDim.x >> 6) * 2048;
+  if (blockIdx.x == 0) {
+    if (rt.E <= 64) skinny_route_block<1>(a, rt, red, stage);
+    else skinny_route_block<4>(a, rt, red, stage);
+    return;
+  }
+  const int id = blockIdx.x - 1;
+  if ((int)(threadIdx.x >> 6) >= pb.waves) return;
+  skinny_block<0, FULL_B, SW_B, TC_B>(b, pb.rows, pb.waves, id % pb.grid_x, id / pb.grid_x, red,
+                                      stage, tile_info);
 }
 
 template <int WAVES>
@@ -369,6 +467,31 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream) {
   else
     gemm_skinny_pair_kernel<true, false, bf16, false, false, bf16>
         <<<(unsigned)blocks, threads, lds, stream>>>(a, pa, b, pb);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+// The pair (router's logits, a dense SwiGLU) with the routing of the logits in the same
+// launch: few rows (one tile of 16), few router features (one block streams their weights in
+// the time the other product's blocks take anyway).
+bool gemm_skinny_route_pair_takes(const GemmArgs& a, const GemmArgs& b, const RouteArgs& rt) {
+  if (!gemm_skinny_pair_takes(a, b) || a.offsets) return false;
+  return a.M <= SM && a.N <= kRouteMaxFeatures && a.N >= rt.E && (int64_t)a.N * a.K <= (1 << 19) &&
+         rt.E >= 1 && rt.k >= 1 && rt.k <= rt.E && rt.k <= 64;
+}
+
+int gemm_skinny_route_pair(const GemmArgs& a, const GemmArgs& b, const RouteArgs& rt,
+                           hipStream_t stream) {
+  const SkinnyPlan pb = plan_skinny(b);
+  const int threads = 1024;                      // the router's block has work for 16 waves
+  const size_t lds = (size_t)(threads / 64) * 4096;
+  // the router's block: 5 KB of logits, E + 1 counters and 16 k chosen experts in its 32 KB
+  static_assert(16 * kRouteMaxFeatures * 4 + (kRouteMaxFeatures + 1) * 4 + 16 * 64 * 4 <= 16 * 2048,
+                "the routing block's LDS");
+  const long blocks = 1 + (long)pb.grid_x * pb.grid_y;
+  NINFER_REQUIRE(blocks < (1L << 31), "gemm pair: %ld blocks are too many", blocks);
+  gemm_skinny_route_pair_kernel<false, true, bf16>
+      <<<(unsigned)blocks, threads, lds, stream>>>(a, rt, b, pb);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

@@ -37,6 +37,14 @@ class _GemmArgs(ctypes.Structure):
                 ("force_kernel", ctypes.c_int), ("skinny_two", ctypes.c_int)]
 
 
+class _RouteArgs(ctypes.Structure):
+    _fields_ = [("ids", ctypes.c_void_p), ("wts", ctypes.c_void_p), ("offsets", ctypes.c_void_p),
+                ("order", ctypes.c_void_p), ("tiles16", ctypes.c_void_p),
+                ("tiles64", ctypes.c_void_p), ("tile_counts", ctypes.c_void_p),
+                ("E", ctypes.c_int), ("k", ctypes.c_int), ("renorm", ctypes.c_int),
+                ("big_rows", ctypes.c_int)]
+
+
 class _AttnArgs(ctypes.Structure):
     _fields_ = [("q", ctypes.c_void_p), ("kpool", ctypes.c_void_p), ("vpool", ctypes.c_void_p),
                 ("out", ctypes.c_void_p), ("block_table", ctypes.c_void_p),
@@ -88,12 +96,14 @@ class _Together:
         if self.ops._held is not None:
             raise KernelError("together(): already inside one")
         self.ops._held = []
+        self.ops._held_route = None
         return self
 
     def __exit__(self, exc_type, exc, tb):
         held, self.ops._held = self.ops._held, None
+        route, self.ops._held_route = self.ops._held_route, None
         if exc_type is None:
-            self.ops._launch_held(held)
+            self.ops._launch_held(held, route)
         return False
 
 
@@ -149,6 +159,7 @@ class HipOps:
         self.lib.ninfer_sample_few_places.restype = ctypes.c_longlong
         self.force_generic = False  # tests: run the plain kernels whatever the shape
         self._held = None           # products held back inside `together()`
+        self._held_route = None     # ... and a routing by the logits one of them writes
         self._side = None           # the second stream of `beside()`, made at first use
         self._side_events = None    # (start, end) of the `beside()` block
         self._side_open = False     # a `beside()` block that `join()` has not waited for
@@ -427,8 +438,17 @@ class HipOps:
             torch.cuda.current_stream().wait_event(self._side_events[1])
             self._side_open = False
 
-    def _launch_held(self, held):
+    def _launch_held(self, held, route=None):
         force = 1 if self.force_generic else 0
+        if route is not None:
+            logits, rargs, keep = route
+            if len(held) == 2 and held[0][1][2] is logits:
+                # the router's logits, a product beside them, and the routing: one launch
+                # where the library has a kernel for the three, else it runs them in turn
+                self._ok(self.lib.ninfer_gemm_pair_route(
+                    ctypes.byref(held[0][0]), ctypes.byref(held[1][0]), ctypes.byref(rargs), force,
+                    self._stream()))
+                return
         i = 0
         while i < len(held):
             if i + 1 < len(held):
@@ -439,6 +459,8 @@ class HipOps:
             else:
                 self._ok(self.lib.ninfer_gemm(ctypes.byref(held[i][0]), force, self._stream()))
                 i += 1
+        if route is not None:
+            self._route_now(*route[2])
 
     def linear(self, x, w, out, bias=None):
         """out = x w^T (+ bias); out may be 32-bit whatever the inputs are."""
@@ -560,20 +582,35 @@ class HipOps:
         """Softmax + top-k per row and the grouping by expert, into the routing
         record `r` (ids, weights, offsets, order, tile lists): one launch for up
         to 16 rows (one block does both), two for more (top-k by one wave per
-        row in parallel, then the grouping)."""
+        row in parallel, then the grouping). Inside `together()`, after the
+        product that writes `logits`, it is held back with the products and
+        launched with them (for few rows: by the block that computes the logits)."""
         t = logits.shape[0]
-        if t > 16:
-            self.router_topk(logits, experts, top_k, renorm, r.ids, r.weights)
-            self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r)
-            return
         _dev(logits, "logits", torch.float32, 2)
         _dev(r.ids, "ids", torch.int32, 2)
         _dev(r.weights, "weights", torch.float32, 2)
         _dev(r.offsets, "offsets", torch.int32, 1)
         _dev(r.order, "order", torch.int32, 1)
+        _need(logits.shape[1] >= experts, "moe_route: fewer logits than experts")
         _need(r.ids.shape == (t, top_k) and r.weights.shape == (t, top_k)
               and r.offsets.shape[0] == experts + 1 and r.order.shape[0] == t * top_k,
               "moe_route: output sizes")
+        if self._held is not None:
+            _need(self._held_route is None, "together(): one routing at most")
+            t16, t64, tc = self._tile_ptrs(r, t * top_k, experts)
+            rargs = _RouteArgs(r.ids.data_ptr(), r.weights.data_ptr(), r.offsets.data_ptr(),
+                               r.order.data_ptr(), t16, t64, tc, experts, top_k,
+                               1 if renorm else 0, r.big_rows)
+            self._held_route = (logits, rargs, (logits, experts, top_k, renorm, r))
+            return
+        self._route_now(logits, experts, top_k, renorm, r)
+
+    def _route_now(self, logits, experts, top_k, renorm, r):
+        t = logits.shape[0]
+        if t > 16:
+            self.router_topk(logits, experts, top_k, renorm, r.ids, r.weights)
+            self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r)
+            return
         t16, t64, tc = self._tile_ptrs(r, t * top_k, experts)
         self._ok(self.lib.ninfer_moe_route_small(
             ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, experts, top_k,

@@ -191,11 +191,13 @@ class SparseMoE(FeedForward):
             ctx.ops.join()
             return PendingRows(y, routing.weights, shared, logits[:, self.router.experts])
         # Few rows: each goes together with the routed path's product of the same stage.
+        # The routing goes with them: for a handful of rows the block that computes the logits
+        # routes the rows itself.
         with ctx.ops.together():
             ctx.ops.linear(x, self.router_and_gate, logits)
             h_shared = self.shared.gate_up(ctx, x)
+            routing = self.router.route(ctx, logits)
         gate = logits[:, self.router.experts]
-        routing = self.router.route(ctx, logits)
         self.last_ids = routing.ids
         h = self.experts.gate_up(ctx, x, routing)
         with ctx.ops.together():

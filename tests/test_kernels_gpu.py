@@ -410,6 +410,75 @@ def test_products_launched_together(ops_mode, gen, dtype, t, e, k, h, inner, sha
     close(logits, logits2, torch.float32, scale=math.sqrt(h) * 0.3)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("t,e,k,h,shared_inner,extra", [
+    (1, 60, 4, 2048, 5632, 1), (8, 60, 4, 2048, 1408, 1), (16, 64, 8, 3584, 512, 1),
+    (5, 7, 3, 384, 1000, 0), (16, 79, 5, 256, 96, 1), (2, 8, 8, 64, 96, 1), (11, 33, 1, 160, 48, 2),
+    (17, 60, 4, 256, 352, 1),     # more rows than one tile: products, then the routing kernels
+    (3, 100, 6, 128, 96, 0),      # more experts than the routing block takes
+    (40, 6, 2, 128, 96, 1)])
+def test_routing_launched_with_the_products(ops_mode, gen, dtype, t, e, k, h, shared_inner, extra):
+    """A router's logits, a SwiGLU beside them and the routing by those logits inside one
+    together(): for a handful of rows the block that computes the logits routes the rows.
+    Logits and activations against the twin; the routing against the twin's routing of the
+    very logits the kernel wrote (so that no near-tie can differ), and against the routing
+    kernel on its own."""
+    ops = ops_mode
+    plain = PlainOps()
+    from ninfer_amd.parts.moe import Routing, big_tile_rows
+    n = t * k
+    x = rnd((t, h), dtype, gen)
+    w_router = rnd((e + extra, h), dtype, gen, 0.3)
+    w_gu = rnd((2 * shared_inner, h), dtype, gen, 0.3)
+
+    def record():
+        i32 = lambda *sh: torch.full(sh, -7, device="cuda", dtype=torch.int32)
+        return Routing(i32(t, k), torch.full((t, k), -7.0, device="cuda"), i32(e + 1), i32(n),
+                       i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2),
+                       big_rows=big_tile_rows(n, e))
+    for renorm in (True, False):
+        logits = torch.full((t, e + extra), 9e9, device="cuda")
+        hs = torch.zeros(t, shared_inner, device="cuda", dtype=dtype)
+        r = record()
+        with ops.together():
+            ops.linear(x, w_router, logits)
+            ops.swiglu_linear(x, w_gu, hs)
+            ops.moe_route(logits, e, k, renorm, r)
+        assert ops._held is None and ops._held_route is None
+        logits2, hs2 = torch.zeros_like(logits), torch.zeros_like(hs)
+        plain.linear(x, w_router, logits2)
+        plain.swiglu_linear(x, w_gu, hs2)
+        close(logits, logits2, torch.float32, scale=math.sqrt(h) * 0.3)
+        close(hs, hs2, dtype, scale=h * 0.3)
+        r2, r3 = record(), record()
+        plain.moe_route(logits, e, k, renorm, r2)
+        ops.moe_route(logits, e, k, renorm, r3)
+        assert torch.equal(r.ids, r2.ids)
+        close(r.weights, r2.weights, torch.float32)
+        assert torch.equal(r.offsets, r2.offsets) and torch.equal(r.offsets, r3.offsets)
+        o = r.offsets.tolist()
+        assert o[e] == n
+        flat = r.ids.reshape(-1)
+        for g in range(e):
+            mine = r.order[o[g]:o[g + 1]].tolist()
+            assert sorted(mine) == sorted(r2.order[o[g]:o[g + 1]].tolist())
+            assert all(int(flat[i]) == g for i in mine)
+        assert torch.equal(r.tile_counts, r3.tile_counts)
+        n16, nbig = r.tile_counts.tolist()
+        assert torch.equal(r.tiles16[:n16], r3.tiles16[:n16])
+        assert torch.equal(r.tiles64[:nbig], r3.tiles64[:nbig])
+    # a routing without its logits' product in the block: launched after what is held
+    logits = torch.zeros(t, e + extra, device="cuda")
+    plain.linear(x, w_router, logits)
+    r, r2 = record(), record()
+    with ops.together():
+        ops.swiglu_linear(x, w_gu, hs)
+        ops.moe_route(logits, e, k, True, r)
+    plain.moe_route(logits, e, k, True, r2)
+    assert torch.equal(r.ids, r2.ids) and torch.equal(r.offsets, r2.offsets)
+    close(hs, hs2, dtype, scale=h * 0.3)
+
+
 def test_router_ties_go_to_the_lower_index(ops):
     logits = torch.zeros(2, 8, device="cuda")
     logits[1, 5] = 1.0
