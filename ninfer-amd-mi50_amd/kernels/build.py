@@ -142,7 +142,10 @@ def _compile_and_link(srcs: List[str], out_dir: str, jobs: int) -> str:
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(one, zip(srcs, objs)))
     lib = os.path.join(out_dir, LIB_NAME)
-    _run([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", lib + ".tmp", *objs])
+    # -z defs: a kernel whose host-side stub the compiler dropped (it does so without a word
+    # for some constructs it cannot instantiate on the host) fails here, not at the first load
+    _run([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-Wl,-z,defs", "-o", lib + ".tmp",
+          *objs])
     os.replace(lib + ".tmp", lib)
     with open(os.path.join(out_dir, "fingerprint"), "w") as f:
         f.write(_fingerprint())
