@@ -7,9 +7,18 @@
 // the staged kernel beside it; the reference sends these products to rocBLAS
 // (src/ops/linear.hip:21-35, src/models/model.hip:406-425).
 //
-// A block has 4 waves, one per SIMD, as a 2 x 2 grid; each wave owns 128 W rows
-// x 128 tokens = 4 x 4 tiles of v_mfma_f32_32x32x16_bf16 (256 accumulator
-// registers), which halves the LDS reads per product against 2 x 2 tiles.
+// A block has 8 waves, two per SIMD, as a 4 x 2 grid; each wave owns 64 W rows
+// x 128 tokens = 2 x 4 tiles of v_mfma_f32_32x32x16_bf16 (128 accumulator
+// registers). Four waves of 128 x 128 read a third less from LDS per product,
+// but on this part a CU's loads into LDS and its matrix instructions do not
+// overlap (a block's time is their sum, whatever the order of issue), and what
+// is left to hide is the rest: with two waves per SIMD the epilogue and the
+// waits at the barrier of one run beside the products of the other (3 to 15%
+// on the experts' products of 1,024 to 8,192 tokens).
+// A wave column multiplies only its 32-row blocks that hold rows, and after the
+// first two k tiles a wave loads only the pieces of A that hold rows, so a tile
+// with few rows costs little more than its share: one tile height serves every
+// count of rows per expert.
 //
 // LDS rows are 128 bytes (64 bf16) and unpadded, because a wave's load writes
 // 1 KB contiguously (lane l at 16 l); the eight 16-byte chunks of row r are
@@ -29,9 +38,10 @@ namespace ninfer {
 
 namespace direct {
 constexpr int TM = 256, TN = 256;
-constexpr int WGM = 2, WGN = 2;
+constexpr int WGM = 4, WGN = 2;
+constexpr int WAVES = WGM * WGN;
 constexpr int COL = TM / WGN;             // staged token rows per wave column
-constexpr int FI = 4, FJ = 4;
+constexpr int FI = TN / WGM / 32, FJ = TM / WGN / 32;
 }  // namespace direct
 
 // Wait until at most N of this wave's loads are under way (and, with LDS, until its LDS
@@ -44,7 +54,7 @@ template <int N> __device__ __forceinline__ void wait_loads_and_lds() {
 }
 
 template <int TK, bool SWIGLU, typename TC>
-__global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
+__global__ __launch_bounds__(direct::WAVES * 64, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   using namespace direct;
   constexpr int KK = TK / 16;                // parts of a k tile: one MFMA depth each
   constexpr int ROW_BYTES = TK * 2;
@@ -62,7 +72,8 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   if (!tile_rows<TM>(a, bx, (int*)smem, row0, row_end, group)) return;
   __syncthreads();
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same in every lane: a scalar
   const int wm = wave % WGM, wn = wave / WGM;
   const int K = a.K, N = a.N;
   const bf16* W = (const bf16*)a.W + (int64_t)group * a.w_group_stride;
@@ -77,22 +88,27 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
   // of the W) part of a buffer: RPP rows, lane l at row l / CPR, stored chunk
   // l % CPR, which holds the row's chunk (l % CPR) ^ swizzle(row), where
   // swizzle(row) = (row / (16 / CPR)) % CPR.
-  constexpr int NL = TM * ROW_BYTES / 1024 / 4;   // load instructions per wave, k tile and operand
+  constexpr int NL = TM * ROW_BYTES / 1024 / WAVES;   // load instructions per wave, k tile and operand
   constexpr int NLT = 2 * NL;                     // loads per wave and k tile
   // the row's part of the swizzle that the piece's number leaves: pieces i * 4 + w differ
   // in multiples of 4 RPP rows between the loads of a wave, which the swizzle does not see
   const int chunk = (lane % CPR) ^ (((wave * RPP + lane / CPR) / (16 / CPR)) % CPR);
-  static_assert((4 * RPP / (16 / CPR)) % CPR == 0, "the loads of a wave must share their swizzle");
+  static_assert((WAVES * RPP / (16 / CPR)) % CPR == 0, "the loads of a wave must share their swizzle");
   const bf16* xsrc[NL];
   const bf16* wsrc[NL];
   int x_row[NL];
+  unsigned x_live = 0;   // bit i: piece i of this wave's loads of A holds rows of the tile
 #pragma unroll
   for (int i = 0; i < NL; ++i) {
-    const int l = (i * 4 + wave) * RPP + lane / CPR;
+    const int l = (i * WAVES + wave) * RPP + lane / CPR;
     const int r = row_of(l);
     // rows beyond the tile's last read its first row (one line, from L1): their results are
     // never stored
     x_row[i] = r < rows_here ? row0 + r : row0;
+    // a piece none of whose rows the tile has is loaded with the first tiles only (what the
+    // fragments read there afterwards goes into sums that are never stored); staged rows
+    // of a piece are neighbours in one column, so its first row decides
+    if (row_of((i * WAVES + wave) * RPP) < rows_here) x_live |= 1u << i;
     wsrc[i] = W + (int64_t)staged_w_row<TN, WGM, SWIGLU>(l, out0, N) * K + 8 * chunk;
   }
   if (a.a_index) {   // the index loads in flight together
@@ -123,7 +139,8 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
     kt = kt >= nk_all ? kt - nk_all : kt;
 #pragma unroll
     for (int i = 0; i < NL; ++i)
-      __builtin_amdgcn_global_load_lds((gptr)(xsrc[i] + kt * TK), (lptr)(buf + i * 4096), 16, 0, 0);
+      if (t < NBX || (x_live & (1u << i)))
+        __builtin_amdgcn_global_load_lds((gptr)(xsrc[i] + kt * TK), (lptr)(buf + i * (WAVES * 1024)), 16, 0, 0);
   };
   // An expert whose rows fit one tile (or a dense product of one row tile) has its W panel read
   // by this block alone: those loads
@@ -138,11 +155,11 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
     if (w_once) {
 #pragma unroll
       for (int i = 0; i < NL; ++i)
-        __builtin_amdgcn_global_load_lds((gptr)(wsrc[i] + kt * TK), (lptr)(buf + i * 4096), 16, 0, 2);
+        __builtin_amdgcn_global_load_lds((gptr)(wsrc[i] + kt * TK), (lptr)(buf + i * (WAVES * 1024)), 16, 0, 2);
     } else {
 #pragma unroll
       for (int i = 0; i < NL; ++i)
-        __builtin_amdgcn_global_load_lds((gptr)(wsrc[i] + kt * TK), (lptr)(buf + i * 4096), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr)(wsrc[i] + kt * TK), (lptr)(buf + i * (WAVES * 1024)), 16, 0, 0);
     }
   };
   auto next_w = [](int w_off) { return w_off == (NBW - 1) * W_BYTES ? 0 : w_off + W_BYTES; };
@@ -261,7 +278,7 @@ __global__ __launch_bounds__(256, 1) void gemm_tile_direct_kernel(GemmArgs a) {
     case 3: run(std::integral_constant<int, 3>{}); break;
     default: run(std::integral_constant<int, 4>{}); break;
   }
-  static_assert(4 * FJ * 32 * FI * 64 <= NBX * X_BYTES + NBW * W_BYTES, "the epilogue's stage exceeds the buffers");
+  static_assert(WAVES * FJ * 32 * FI * 64 <= NBX * X_BYTES + NBW * W_BYTES, "the epilogue's stage exceeds the buffers");
   __syncthreads();   // every wave has read its last fragments: the buffers become the epilogue's stage
   write_tile<FI, FJ, SWIGLU, TC>(a, acc, smem + wave * (FJ * 32 * FI * 64), tok0, row0, rows_here,
                                  out0 + OUT_PER_WAVE * wm, row_of);
@@ -287,7 +304,7 @@ static int launch_direct(const GemmArgs& a, hipStream_t stream) {
     hipError_t e = hipFuncSetAttribute((const void*)kern,                                       \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);  \
     if (e != hipSuccess) return set_error(-2, "gemm: cannot get %d bytes of LDS", LDS_BYTES);   \
-    kern<<<grid, 256, LDS_BYTES, stream>>>(a);                                                  \
+    kern<<<grid, direct::WAVES * 64, LDS_BYTES, stream>>>(a);                                                  \
   } while (0)
   if (a.out_dtype == kF32) {
     if (swiglu) NINFER_DIRECT_LAUNCH(true, float); else NINFER_DIRECT_LAUNCH(false, float);
