@@ -275,7 +275,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_pair_kernel(GemmArgs a, Skin
 // then holds every logit of every row and routes the rows itself (softmax, top-k, grouping
 // by expert) out of LDS. As a kernel of its own the routing is a launch and a chain of
 // dependent loads between the router's product and the experts' first one.
-// `red`: 16 x 256 floats; `stage`: 32 KB (the waves' weight lines, then logits, counters
+// `red`: 32 x 256 floats; `stage`: 32 KB (the waves' weight lines, then logits, counters
 // and chosen experts). Every thread of the block must call.
 constexpr int kRouteMaxFeatures = 80;
 
@@ -285,26 +285,40 @@ __device__ __forceinline__ void skinny_route_block(const GemmArgs& a, const Rout
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
   const int r = lane & 15, j = lane >> 4;
   const int N = a.N, K = a.K, T = a.M;
-  const int groups = (N + 15) / 16, parts = waves / groups;
-  const int g = wave / parts, part = wave % parts;   // waves beyond groups x parts have no share
-  if (g < groups) {
-    const int n0 = 16 * g, rows = min(16, N - n0);
+  const int groups = (N + 15) / 16;
+  // A wave multiplies GS feature groups of 16 over its part of K; the waves are shared out as
+  // sets of GS groups x parts of K. Rows beyond N repeat row N - 1: they are computed and
+  // never used. The fewer parts of K per wave, the shorter the chain of dependent loads that
+  // this block, the launch's longest, consists of.
+  constexpr int GS = 2;
+  const int sets = (groups + GS - 1) / GS, parts = waves / sets;
+  const int g = wave / parts, part = wave % parts;   // waves beyond sets x parts have no share
+  if (g < sets) {
     const bf16* W = (const bf16*)a.W;
-    SkinnyOperands<1> o;
-    o.w_valid = r < rows;
-    o.wrow[0] = W + (int64_t)min(n0 + r, N - 1) * K + 8 * j;
+    SkinnyOperands<GS> o;
+    o.w_valid = true;
+#pragma unroll
+    for (int s = 0; s < GS; ++s) o.wrow[s] = W + (int64_t)min(16 * (GS * g + s) + r, N - 1) * K + 8 * j;
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       const int R = 8 * q + (lane >> 3);
-      o.line_valid[q] = R < rows;
-      o.wline[0][q] = W + (int64_t)min(n0 + R, N - 1) * K + 8 * (lane & 7);
+      o.line_valid[q] = true;
+#pragma unroll
+      for (int s = 0; s < GS; ++s)
+        o.wline[s][q] = W + (int64_t)min(16 * (GS * g + s) + R, N - 1) * K + 8 * (lane & 7);
     }
     o.m_valid = r < T;
     o.xrow = (const bf16*)a.A + (int64_t)(o.m_valid ? r : 0) * a.lda + 8 * j;
-    f32x4 acc[1] = {f32x4{0.f, 0.f, 0.f, 0.f}};
-    skinny_walk<1>(o, K, part, parts, stage + wave * 2048, lane, acc);
+    f32x4 acc[GS];
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[wave * 256 + r * 16 + 4 * j + v] = acc[0][v];
+    for (int s = 0; s < GS; ++s) acc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+    skinny_walk<GS>(o, K, part, parts, stage + wave * 2048, lane, acc);
+    // partial tile of group GS g + s from K part `part`: at ((GS g + s) * parts + part) * 256
+#pragma unroll
+    for (int s = 0; s < GS; ++s)
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        red[((GS * g + s) * parts + part) * 256 + r * 16 + 4 * j + v] = acc[s][v];
   }
   __syncthreads();   // the partial tiles are complete, and the weight lines' LDS is free
   // logit (row m, feature n): the parts of its group summed in their order; kept in LDS and
