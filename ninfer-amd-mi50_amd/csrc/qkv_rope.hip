@@ -190,7 +190,7 @@ extern "C" int ninfer_qkv_rope(const QkvRopeArgs* args, hipStream_t stream) {
   dim3 grid((unsigned)blocks, m_tiles);
   const int chunks = a.K / 128;
   const int cus = device_cu_count();
-  if (blocks * m_tiles < cus && chunks >= 16)
+  if (blocks * m_tiles < 2 * cus && chunks >= 16)
     qkv_rope_kernel<16><<<grid, 16 * 64, 0, stream>>>(a, pairs);
   else if (blocks * m_tiles < 8 * cus && chunks >= 8)
     qkv_rope_kernel<8><<<grid, 8 * 64, 0, stream>>>(a, pairs);
