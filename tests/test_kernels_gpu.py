@@ -479,6 +479,40 @@ def test_routing_launched_with_the_products(ops_mode, gen, dtype, t, e, k, h, sh
     close(hs, hs2, dtype, scale=h * 0.3)
 
 
+@pytest.mark.parametrize("counts", [[17, 31, 32, 33, 63], [64, 65, 127, 128, 129], [255, 256, 257, 300, 16],
+                                    [511, 512, 513, 20, 700], [16, 16, 200, 16, 290], [69, 70, 71, 72, 73],
+                                    [96, 97, 160, 161, 192, 193, 224, 225]])
+@pytest.mark.parametrize("h,inner", [(256, 192), (2048, 1408)])
+def test_grouped_products_at_the_edges_of_the_row_blocks(ops, gen, counts, h, inner):
+    """Chosen rows per expert around the 32-row blocks and the 256-row tiles of the tall
+    tile kernel, which loads and multiplies only the blocks that hold rows: an expert with one
+    row more or fewer than a block, a tile and a row, two tiles and a row."""
+    from ninfer_amd.parts.moe import Routing
+    plain = PlainOps()
+    dtype = torch.bfloat16
+    e, n = len(counts), sum(counts)
+    ids = torch.cat([torch.full((c,), i, dtype=torch.int32) for i, c in enumerate(counts)])
+    ids = ids[torch.randperm(n, generator=torch.Generator().manual_seed(n))].cuda().reshape(n, 1)
+    i32 = lambda *sh: torch.zeros(*sh, device="cuda", dtype=torch.int32)
+    r = Routing(ids, torch.ones(n, 1, device="cuda"), i32(e + 1), i32(n), i32(min(n, n // 16 + e), 4),
+                i32(n // 64 + e, 4), i32(2), big_rows=256)
+    ops.moe_align(ids, e, r.offsets, r.order, tiles=r)
+    assert (r.offsets[1:] - r.offsets[:-1]).tolist() == counts
+    x = rnd((n, h), dtype, gen)
+    wgu = rnd((e, 2 * inner, h), dtype, gen, 0.3)
+    wd = rnd((e, h, inner), dtype, gen, 0.3)
+    h1 = torch.full((n, inner), 7.0, device="cuda", dtype=dtype)
+    h2 = torch.zeros_like(h1)
+    ops.grouped_swiglu(x, wgu, r.offsets, r.order, 1, h1, tiles=r)
+    plain.grouped_swiglu(x, wgu, r.offsets, r.order, 1, h2)
+    close(h1, h2, dtype, scale=h * 0.3)
+    y1 = torch.full((n, h), 7.0, device="cuda", dtype=dtype)
+    y2 = torch.zeros_like(y1)
+    ops.grouped_down(h2, wd, r.offsets, r.order, y1, tiles=r)
+    plain.grouped_down(h2, wd, r.offsets, r.order, y2)
+    close(y1, y2, dtype, scale=h2.float().abs().max().item() * math.sqrt(inner) * 0.3)
+
+
 def test_router_ties_go_to_the_lower_index(ops):
     logits = torch.zeros(2, 8, device="cuda")
     logits[1, 5] = 1.0
