@@ -105,6 +105,8 @@ int gemm_skinny(const GemmArgs& a, hipStream_t stream);
 bool gemm_skinny_pair_takes(const GemmArgs& a, const GemmArgs& b);
 int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream);
 struct RouteArgs;
+bool gemm_skinny_route_takes(const GemmArgs& a, const RouteArgs& rt);
+int gemm_skinny_route(const GemmArgs& a, const RouteArgs& rt, hipStream_t stream);
 bool gemm_skinny_route_pair_takes(const GemmArgs& a, const GemmArgs& b, const RouteArgs& rt);
 int gemm_skinny_route_pair(const GemmArgs& a, const GemmArgs& b, const RouteArgs& rt,
                            hipStream_t stream);

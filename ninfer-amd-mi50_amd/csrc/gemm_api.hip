@@ -45,34 +45,57 @@ extern "C" int ninfer_gemm_pair(const GemmArgs* a, const GemmArgs* b, int force_
   return ninfer_gemm(b, force_generic, stream);
 }
 
-// The pair above, and the routing of the rows by the logits that product `a` writes
-// ([T, >= E] 32-bit: columns beyond the experts' are not the router's). One launch where the
-// few-row kernel holds the router's product in one block; otherwise the products, then the
-// routing kernels.
+static int route_by(const GemmArgs& a, const RouteArgs& rt, hipStream_t stream) {
+  const float* logits = (const float*)a.C;
+  if (a.M <= 16)
+    return ninfer_moe_route_small(logits, a.ldc, a.M, rt.E, rt.k, rt.renorm, rt.ids, rt.wts,
+                                  rt.offsets, rt.order, rt.tiles16, rt.tiles64, rt.tile_counts,
+                                  rt.big_rows, stream);
+  int rc = ninfer_router_topk(logits, a.ldc, a.M, rt.E, rt.k, rt.renorm, rt.ids, rt.wts, stream);
+  if (rc) return rc;
+  return ninfer_moe_align(rt.ids, a.M * rt.k, rt.E, rt.offsets, rt.order, rt.tiles16, rt.tiles64,
+                          rt.tile_counts, rt.big_rows, stream);
+}
+
+static int route_check(const GemmArgs& a, const RouteArgs& rt) {
+  NINFER_REQUIRE(!a.offsets && a.out_dtype == kF32 && a.N >= rt.E && a.ldc >= rt.E,
+                 "gemm route: the product must be dense with 32-bit logits of %d experts", rt.E);
+  NINFER_REQUIRE((!rt.tiles16) == (!rt.tiles64) && (!rt.tiles16) == (!rt.tile_counts),
+                 "gemm route: tile lists come together or not at all");
+  NINFER_REQUIRE(rt.big_rows == 64 || rt.big_rows == 128 || rt.big_rows == 256,
+                 "gemm route: big tiles of %d rows", rt.big_rows);
+  return 0;
+}
+
+// A router's logits (product `a`, [T, >= E] 32-bit: columns beyond the experts' are not the
+// router's) and the routing of the rows by them. One launch where one block of the few-row
+// kernel holds the product; otherwise the product, then the routing kernels.
+extern "C" int ninfer_gemm_route(const GemmArgs* a, const RouteArgs* rt, int force_generic,
+                                 hipStream_t stream) {
+  int rc = gemm_check(*a);
+  if (rc) return rc;
+  rc = route_check(*a, *rt);
+  if (rc) return rc;
+  if (!force_generic && !many_rows(*a) && gemm_skinny_route_takes(*a, *rt))
+    return gemm_skinny_route(*a, *rt, stream);
+  rc = ninfer_gemm(a, force_generic, stream);
+  if (rc) return rc;
+  return route_by(*a, *rt, stream);
+}
+
+// The same with a second product `b` that does not depend on the first (a shared expert's gate
+// and up) in the launch.
 extern "C" int ninfer_gemm_pair_route(const GemmArgs* a, const GemmArgs* b, const RouteArgs* rt,
                                       int force_generic, hipStream_t stream) {
   int rc = gemm_check(*a);
   if (rc) return rc;
   rc = gemm_check(*b);
   if (rc) return rc;
-  NINFER_REQUIRE(!a->offsets && a->out_dtype == kF32 && a->N >= rt->E && a->ldc >= rt->E,
-                 "gemm_pair_route: the first product must be dense with 32-bit logits of %d experts",
-                 rt->E);
-  NINFER_REQUIRE((!rt->tiles16) == (!rt->tiles64) && (!rt->tiles16) == (!rt->tile_counts),
-                 "gemm_pair_route: tile lists come together or not at all");
-  NINFER_REQUIRE(rt->big_rows == 64 || rt->big_rows == 128 || rt->big_rows == 256,
-                 "gemm_pair_route: big tiles of %d rows", rt->big_rows);
+  rc = route_check(*a, *rt);
+  if (rc) return rc;
   if (!force_generic && !many_rows(*a) && !many_rows(*b) && gemm_skinny_route_pair_takes(*a, *b, *rt))
     return gemm_skinny_route_pair(*a, *b, *rt, stream);
   rc = ninfer_gemm_pair(a, b, force_generic, stream);
   if (rc) return rc;
-  const float* logits = (const float*)a->C;
-  if (a->M <= 16)
-    return ninfer_moe_route_small(logits, a->ldc, a->M, rt->E, rt->k, rt->renorm, rt->ids, rt->wts,
-                                  rt->offsets, rt->order, rt->tiles16, rt->tiles64,
-                                  rt->tile_counts, rt->big_rows, stream);
-  rc = ninfer_router_topk(logits, a->ldc, a->M, rt->E, rt->k, rt->renorm, rt->ids, rt->wts, stream);
-  if (rc) return rc;
-  return ninfer_moe_align(rt->ids, a->M * rt->k, rt->E, rt->offsets, rt->order, rt->tiles16,
-                          rt->tiles64, rt->tile_counts, rt->big_rows, stream);
+  return route_by(*a, *rt, stream);
 }

@@ -365,6 +365,15 @@ __global__ __launch_bounds__(1024) void gemm_skinny_route_pair_kernel(GemmArgs a
                                       stage, tile_info);
 }
 
+// The router's block alone (a router with nothing to launch beside it).
+__global__ __launch_bounds__(1024) void gemm_skinny_route_kernel(GemmArgs a, RouteArgs rt) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char pair_lds[];   // 16 waves x 4 KB
+  float* red = (float*)pair_lds;
+  unsigned char* stage = pair_lds + (blockDim.x >> 6) * 2048;
+  if (rt.E <= 64) skinny_route_block<1>(a, rt, red, stage);
+  else skinny_route_block<4>(a, rt, red, stage);
+}
+
 template <int WAVES>
 static void launch_skinny(const GemmArgs& a, int rows, bool two, hipStream_t stream) {
   int m_tiles = a.offsets ? min((a.M + SM - 1) / SM + a.groups, a.M) : (a.M + SM - 1) / SM;
@@ -488,10 +497,23 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream) {
 // The pair (router's logits, a dense SwiGLU) with the routing of the logits in the same
 // launch: few rows (one tile of 16), few router features (one block streams their weights in
 // the time the other product's blocks take anyway).
-bool gemm_skinny_route_pair_takes(const GemmArgs& a, const GemmArgs& b, const RouteArgs& rt) {
-  if (!gemm_skinny_pair_takes(a, b) || a.offsets) return false;
+// A router's product of few rows and few features, and the routing by it, in one block.
+bool gemm_skinny_route_takes(const GemmArgs& a, const RouteArgs& rt) {
+  if (!gemm_skinny_takes(a) || a.offsets || a.bias || a.out_dtype != kF32 ||
+      a.epilogue != kEpilogueNone)
+    return false;
   return a.M <= SM && a.N <= kRouteMaxFeatures && a.N >= rt.E && (int64_t)a.N * a.K <= (1 << 19) &&
          rt.E >= 1 && rt.k >= 1 && rt.k <= rt.E && rt.k <= 64;
+}
+
+int gemm_skinny_route(const GemmArgs& a, const RouteArgs& rt, hipStream_t stream) {
+  gemm_skinny_route_kernel<<<1, 1024, 16 * 4096, stream>>>(a, rt);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+bool gemm_skinny_route_pair_takes(const GemmArgs& a, const GemmArgs& b, const RouteArgs& rt) {
+  return gemm_skinny_pair_takes(a, b) && gemm_skinny_route_takes(a, rt);
 }
 
 int gemm_skinny_route_pair(const GemmArgs& a, const GemmArgs& b, const RouteArgs& rt,

@@ -442,6 +442,11 @@ class HipOps:
         force = 1 if self.force_generic else 0
         if route is not None:
             logits, rargs, keep = route
+            if len(held) == 1 and held[0][1][2] is logits:
+                # the router's logits and the routing by them: one block does both for few rows
+                self._ok(self.lib.ninfer_gemm_route(ctypes.byref(held[0][0]), ctypes.byref(rargs),
+                                                    force, self._stream()))
+                return
             if len(held) == 2 and held[0][1][2] is logits:
                 # the router's logits, a product beside them, and the routing: one launch
                 # where the library has a kernel for the three, else it runs them in turn

@@ -171,7 +171,8 @@ class SparseMoE(FeedForward):
 
     def forward(self, ctx: StepContext, x, residual):
         if self.shared is None:
-            routing = self.router.route(ctx, self.router.logits(ctx, x))
+            with ctx.ops.together():   # for few rows the logits' block routes the rows itself
+                routing = self.router.route(ctx, self.router.logits(ctx, x))
             self.last_ids = routing.ids
             return PendingRows(self.experts.run(ctx, x, routing), routing.weights)
         # The shared expert's two products wait for nothing the routed path makes. Many rows:

@@ -467,6 +467,19 @@ def test_routing_launched_with_the_products(ops_mode, gen, dtype, t, e, k, h, sh
         n16, nbig = r.tile_counts.tolist()
         assert torch.equal(r.tiles16[:n16], r3.tiles16[:n16])
         assert torch.equal(r.tiles64[:nbig], r3.tiles64[:nbig])
+    # the router's product and the routing alone (a router without a shared expert beside it)
+    logits4 = torch.full((t, e + extra), 9e9, device="cuda")
+    r4, r5 = record(), record()
+    with ops.together():
+        ops.linear(x, w_router, logits4)
+        ops.moe_route(logits4, e, k, True, r4)
+    close(logits4, logits2, torch.float32, scale=math.sqrt(h) * 0.3)
+    plain.moe_route(logits4, e, k, True, r5)
+    assert torch.equal(r4.ids, r5.ids) and torch.equal(r4.offsets, r5.offsets)
+    close(r4.weights, r5.weights, torch.float32)
+    assert torch.equal(r4.tile_counts, r5.tile_counts)
+    n16 = int(r4.tile_counts[0])
+    assert torch.equal(r4.tiles16[:n16], r5.tiles16[:n16])
     # a routing without its logits' product in the block: launched after what is held
     logits = torch.zeros(t, e + extra, device="cuda")
     plain.linear(x, w_router, logits)
