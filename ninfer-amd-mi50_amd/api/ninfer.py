@@ -140,15 +140,6 @@ class Ninfer:
             raise ValueError(f"{name}: [{offset}, {end}) is outside its {flat.numel()} numbers")
         return flat[offset:end].float().cpu().numpy()
 
-    def close(self) -> None:
-        """Give the engine's device memory back (weights, cache, captured graphs)."""
-        import gc
-        import torch
-        self.runner = None
-        self.sampler = None
-        gc.collect()
-        torch.cuda.empty_cache()
-
     # ---- sessions -------------------------------------------------------------------
     def session(self) -> Session:
         return Session(self)
@@ -183,10 +174,19 @@ class Ninfer:
         return self.sampler.sample(row, [r])[0]
 
     def close(self) -> None:
-        """Give the model and its cache back (reference tools/ninfer_ctypes.py:238-241);
-        the object cannot be used afterwards."""
+        """Give the model, its cache, its captured graphs and the kernels' workspaces back to
+        the device (reference tools/ninfer_ctypes.py:238-241: ninfer_free); the object cannot
+        be used afterwards. After it another engine may take this one's place in memory."""
+        import gc
+        import torch
+        if self.runner is not None:
+            self.runner.release()
         self.runner = None
         self.sampler = None
+        gc.collect()
+        if torch.cuda.is_available():
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
 
     # ---- generation -----------------------------------------------------------------
     def generate(self, prompts: Sequence[Sequence[int]], params: Optional[SamplingParams] = None,
@@ -194,8 +194,7 @@ class Ninfer:
         """Generated token ids for each prompt, through the scheduler."""
         params = params or SamplingParams()
         if stop_ids is None:
-            eos = self.runner.spec.eos_token_id
-            stop_ids = [eos] if eos is not None else []
+            stop_ids = list(self.runner.spec.eos_token_ids)
         sched = Scheduler(self.runner, self.sampler)
         reqs = [Request(str(i), list(p), params, stop_ids) for i, p in enumerate(prompts)]
         for r in reqs:

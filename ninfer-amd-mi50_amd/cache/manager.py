@@ -103,6 +103,11 @@ class CacheManager:
         self.state = torch.zeros((self.max_seqs, max(self.state_floats, 1)),
                                  dtype=torch.float32, device=device)
 
+    def drop_pools(self) -> None:
+        """Give the device memory of every pool and of the state back (the end of an engine)."""
+        self.pools = {}
+        self.state = None
+
     # ---- slots ---------------------------------------------------------------
     @property
     def free_slots(self) -> int:

@@ -20,6 +20,7 @@ class EngineOptions:
     num_pages: Optional[int] = None  # pages per cache group; None: from kv_bytes, else enough for every request at max_context
     kv_bytes: Optional[int] = None   # bytes of paged cache over all layers (the reference sizes its slabs in bytes, src/api/ninfer_c_api.cpp:105-108)
     use_graph: bool = False        # replay decode-only steps from a captured HIP graph
+    max_graphs: int = 32           # most captured graphs kept (one per count of requests and context bound); the least recently replayed goes first
     poison_freed_pages: bool = False  # debugging: fill pages that are given back with NaN
     check_pages: bool = False      # debugging: before every step, check on the host that every page the step reads or writes is held by its request and by no other
     device: str = "cuda:0"
@@ -27,7 +28,7 @@ class EngineOptions:
     def validate(self) -> None:
         if self.dtype not in ("bfloat16", "float32"):
             raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {self.dtype!r}")
-        for name in ("max_context", "prefill_chunk", "num_sequences", "page_size"):
+        for name in ("max_context", "prefill_chunk", "num_sequences", "page_size", "max_graphs"):
             if getattr(self, name) < 1:
                 raise ValueError(f"{name} must be >= 1, got {getattr(self, name)}")
         if self.num_pages is not None and self.num_pages < 1:

@@ -11,7 +11,7 @@ are read here because the architecture has them.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, List, Optional, Tuple
 
 from .base import ConfigError, KeyReader
 
@@ -39,8 +39,12 @@ class Qwen2MoeConfig:
     sliding_window: Optional[int] = None
     max_window_layers: int = 0
     qkv_bias: bool = True
-    eos_token_id: Optional[int] = None
+    eos_token_ids: Tuple[int, ...] = ()   # every id that ends a generation (the key may hold one or a list)
     architecture: str = "Qwen2MoeForCausalLM"
+
+    @property
+    def eos_token_id(self) -> Optional[int]:
+        return self.eos_token_ids[0] if self.eos_token_ids else None
 
     # ---- derived, layer by layer -------------------------------------
     def layer_is_sparse(self, layer: int) -> bool:
@@ -105,13 +109,19 @@ class Qwen2MoeConfig:
         act = r.opt_str("hidden_act", "silu")
         if act != "silu":
             raise ConfigError(f"config.json: key 'hidden_act' must be 'silu', got {act!r}")
-        experts = r.need_int("num_experts", 1)
-        top_k = r.need_int("num_experts_per_tok", 1)
-        if top_k > experts:
-            raise ConfigError(f"config.json: 'num_experts_per_tok' ({top_k}) exceeds "
-                              f"'num_experts' ({experts})")
-        moe_inter = r.need_int("moe_intermediate_size", 1)
-        shared_inter = r.need_int("shared_expert_intermediate_size", 1)
+        # no experts (the key absent or 0): every layer has the dense feed-forward; no shared
+        # expert (absent or 0): a sparse layer is its routed experts alone
+        experts = r.opt_int("num_experts", 0, 0)
+        if experts:
+            top_k = r.need_int("num_experts_per_tok", 1)
+            if top_k > experts:
+                raise ConfigError(f"config.json: 'num_experts_per_tok' ({top_k}) exceeds "
+                                  f"'num_experts' ({experts})")
+            moe_inter = r.need_int("moe_intermediate_size", 1)
+        else:
+            top_k = r.opt_int("num_experts_per_tok", 0, 0)
+            moe_inter = r.opt_int("moe_intermediate_size", 0, 0)
+        shared_inter = r.opt_int("shared_expert_intermediate_size", 0, 0)
         sparse_step = r.opt_int("decoder_sparse_step", 1, 1)
         mlp_only = r.opt_int_list("mlp_only_layers", [])
         for l in mlp_only:
@@ -125,10 +135,11 @@ class Qwen2MoeConfig:
             raise ConfigError("config.json: 'use_sliding_window' is true but "
                               "'sliding_window' is missing")
         eos = r.opt_raw("eos_token_id")
-        if isinstance(eos, list):
-            eos = eos[0] if eos else None
-        if eos is not None and (isinstance(eos, bool) or not isinstance(eos, int)):
-            raise ConfigError("config.json: key 'eos_token_id' must be an integer")
+        eos = [] if eos is None else eos if isinstance(eos, list) else [eos]
+        for e in eos:
+            if isinstance(e, bool) or not isinstance(e, int) or e < 0:
+                raise ConfigError("config.json: key 'eos_token_id' must be a non-negative "
+                                  f"integer or a list of them, got {raw['eos_token_id']!r}")
         return Qwen2MoeConfig(
             vocab_size=vocab, hidden_size=hidden, num_hidden_layers=layers,
             num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=head_dim,
@@ -141,4 +152,4 @@ class Qwen2MoeConfig:
             decoder_sparse_step=sparse_step, mlp_only_layers=mlp_only,
             use_sliding_window=use_win, sliding_window=window,
             max_window_layers=max_win_layers, qkv_bias=r.opt_bool("qkv_bias", True),
-            eos_token_id=eos)
+            eos_token_ids=tuple(eos))

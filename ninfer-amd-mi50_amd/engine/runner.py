@@ -12,6 +12,7 @@ rows, and nothing inside a step waits for the device.
 """
 from __future__ import annotations
 
+from collections import OrderedDict
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence
 
@@ -74,7 +75,11 @@ class ModelRunner:
         self.cache.poison_freed = options.poison_freed_pages
         self.vocab_size = spec.vocab_size
         self.steps_run = 0
-        self._graphs: Dict[tuple, dict] = {}
+        # captured decode steps by (requests, context bound), least recently replayed first;
+        # at most options.max_graphs are kept (each holds a memory pool of its own)
+        self._graphs: "OrderedDict[tuple, dict]" = OrderedDict()
+        self.graphs_dropped = 0
+        self._holds_graphs = False
         self.graph_context_step = 1024   # a graph serves contexts up to the next multiple
 
     # ---- read-back -------------------------------------------------------------
@@ -96,6 +101,20 @@ class ModelRunner:
 
     def close(self, slot: int) -> None:
         self.cache.release(slot)
+
+    def release(self) -> None:
+        """Drop everything this runner holds on the device: captured graphs (and with them
+        their memory pools), staging buffers, the cache's pools, the bound weights. The
+        kernels' workspaces go too once no runner with captured graphs is left. The runner
+        cannot step afterwards."""
+        self._graphs.clear()
+        if self._holds_graphs:
+            self._holds_graphs = False
+            self.ops.graph_holder_gone()
+        self._staging = []
+        self._held = {}
+        self.cache.drop_pools()
+        self.spec = None
 
     # ---- the step ----------------------------------------------------------------
     def step(self, chunks: Sequence[Chunk]) -> Optional[torch.Tensor]:
@@ -261,7 +280,16 @@ class ModelRunner:
         live in the graph's memory and are valid until the next step."""
         key = (shape["S"], shape["max_kv_len"])
         entry = self._graphs.get(key)
+        if entry is not None:
+            self._graphs.move_to_end(key)
         if entry is None:
+            # The least recently replayed graphs make room. Logits handed out by a dropped
+            # graph were valid until this step only, as those of every graph are; the entry's
+            # own reference to them goes with it, and the pool's memory returns to the
+            # allocator once the caller's last reference is gone.
+            while len(self._graphs) >= max(1, self.options.max_graphs):
+                self._graphs.popitem(last=False)
+                self.graphs_dropped += 1
             self._graphs[key] = {"pinned": torch.empty(host.numel(), dtype=torch.int32).pin_memory(),
                                  "meta": torch.empty(host.numel(), dtype=torch.int32,
                                                      device=self.device), "graph": None}
@@ -283,6 +311,9 @@ class ModelRunner:
             with torch.cuda.graph(g):
                 entry["logits"] = self._forward(entry["meta"], shape)
             entry["graph"] = g
+            if not self._holds_graphs:
+                self._holds_graphs = True
+                self.ops.graph_holder_new()
         entry["graph"].replay()
         return entry["logits"]
 

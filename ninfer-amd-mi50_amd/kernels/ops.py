@@ -110,7 +110,14 @@ class _Together:
 class _Beside:
     """Work on a second stream that starts after everything the current stream has been
     given so far; `HipOps.join()` makes the current stream wait for it. The two events are
-    made once and recorded again every time (an event's earlier waits keep their meaning)."""
+    made once and recorded again every time (an event's earlier waits keep their meaning).
+
+    Memory: tensors made inside the block come from the second stream's part of torch's
+    allocator and are read on the main stream after `join()` without `record_stream`. That
+    holds because the second stream is used inside such blocks only, and every block begins
+    by waiting for an event recorded on the main stream at its entry: a tensor of an earlier
+    block that the main stream has been told to read is read before any later block's work
+    can write into memory the allocator has handed out again."""
 
     def __init__(self, ops):
         self.ops = ops
@@ -178,6 +185,20 @@ class HipOps:
         # what tests and measurements ask of the product kernels (see `tuned`); all 0: the
         # library chooses
         self._tune = {"force_kernel": 0, "split_min_bytes": 0, "skinny_two": 0}
+        self._graph_holders = 0  # runners whose captured graphs may hold workspace addresses
+
+    def graph_holder_new(self) -> None:
+        self._graph_holders += 1
+
+    def graph_holder_gone(self) -> None:
+        """A runner with captured graphs has dropped them. When it was the last, nothing can
+        replay into the workspaces any more: they are given back (the next call that needs
+        one makes it anew)."""
+        self._graph_holders = max(0, self._graph_holders - 1)
+        if self._graph_holders == 0:
+            self._outgrown = []
+            self._attn_ws = None
+            self._split_ws = None
 
     def tuned(self, **values):
         """Context manager for tests and measurements: inside it every product call carries
@@ -394,7 +415,14 @@ class HipOps:
         args.skinny_two = self._tune["skinny_two"]
         if only_if_split:
             # a dense product of few dozen rows: the library's unless the kernels here cut it
-            # along K (its output tiles alone would not fill the GPU)
+            # along K (its output tiles alone would not fill the GPU). The one workspace of
+            # the cut belongs to the main stream: work inside `beside()` starts at
+            # `beside_min_rows` rows, a cut ends at `split_max_rows`, and the callers keep the
+            # first above the second; on the second stream nothing is cut (the library's
+            # product runs instead).
+            if self._side is not None \
+                    and torch.cuda.current_stream().cuda_stream == self._side.cuda_stream:
+                return False
             if self._split_ws is None:
                 self._split_ws = torch.empty(1 << 23, dtype=torch.float32, device=a.device)
             args.workspace = self._split_ws.data_ptr()

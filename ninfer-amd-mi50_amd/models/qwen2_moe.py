@@ -46,7 +46,7 @@ def build_qwen2_moe(cfg: Qwen2MoeConfig) -> ModelSpec:
     final_norm = make_part("norm", "rmsnorm", prefix="model.norm.", size=h, eps=cfg.rms_norm_eps)
     head = LMHead("lm_head.", cfg.vocab_size, h,
                   tied_to=embedding if cfg.tie_word_embeddings else None)
-    return ModelSpec(embedding, blocks, final_norm, head, eos_token_id=cfg.eos_token_id)
+    return ModelSpec(embedding, blocks, final_norm, head, eos_token_ids=cfg.eos_token_ids)
 
 
 register_architecture("Qwen2MoeForCausalLM", Qwen2MoeConfig.from_dict, build_qwen2_moe)

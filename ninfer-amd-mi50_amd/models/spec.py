@@ -27,13 +27,13 @@ class LayerCall:
 class ModelSpec:
     def __init__(self, embedding: TokenEmbedding, blocks: List[Block], final_norm: Norm,
                  head: LMHead, plan: Optional[List[LayerCall]] = None,
-                 vocab_size: Optional[int] = None, eos_token_id: Optional[int] = None):
+                 vocab_size: Optional[int] = None, eos_token_ids=()):
         self.embedding = embedding
         self.blocks = blocks
         self.final_norm = final_norm
         self.head = head
         self.vocab_size = vocab_size if vocab_size is not None else head.vocab
-        self.eos_token_id = eos_token_id
+        self.eos_token_ids = tuple(eos_token_ids)   # ids that end a generation by default
         self.plan: List[LayerCall] = []
         self.set_plan(plan if plan is not None else [LayerCall(i) for i in range(len(blocks))])
 

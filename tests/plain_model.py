@@ -220,7 +220,10 @@ def feed_forward(x: Tensor, w: Dict[str, Tensor], cfg: dict, layer: int,
         probe.setdefault("router_logits", {})[layer] = x @ w[p + "gate.weight"].float().T
     ids, wts = router(x, w[p + "gate.weight"], cfg["num_experts_per_tok"],
                       cfg.get("norm_topk_prob", False))
-    return routed_experts(x, ids, wts, w, p) + shared_expert(x, w, p)
+    y = routed_experts(x, ids, wts, w, p)
+    if cfg.get("shared_expert_intermediate_size", 0) > 0:
+        y = y + shared_expert(x, w, p)
+    return y
 
 
 # --------------------------------------------------------------------------

@@ -35,12 +35,13 @@ def test_defaults_follow_the_reference():
 
 @pytest.mark.parametrize("change,word", [
     ({"vocab_size": None}, "vocab_size"), ({"rms_norm_eps": None}, "rms_norm_eps"),
-    ({"num_experts": None}, "num_experts"), ({"hidden_size": "64"}, "hidden_size"),
+    ({"num_experts": -1}, "num_experts"), ({"hidden_size": "64"}, "hidden_size"),
+    ({"moe_intermediate_size": None}, "moe_intermediate_size"), ({"eos_token_id": [3, "x"]}, "eos_token_id"),
     ({"num_key_value_heads": 3}, "num_key_value_heads"), ({"num_experts_per_tok": 9}, "num_experts_per_tok"),
     ({"hidden_act": "gelu"}, "hidden_act"), ({"rope_scaling": {"type": "yarn"}}, "rope_scaling"),
     ({"model_type": "llama"}, "model_type"), ({"use_sliding_window": True}, "sliding_window"),
     ({"mlp_only_layers": [5]}, "mlp_only_layers"), ({"head_dim": 15}, "head_dim"),
-    ({"shared_expert_intermediate_size": None}, "shared_expert_intermediate_size"),
+    ({"shared_expert_intermediate_size": -2}, "shared_expert_intermediate_size"),
     ({"num_hidden_layers": 0}, "num_hidden_layers"), ({"tie_word_embeddings": "yes"}, "tie_word_embeddings"),
 ])
 def test_configuration_errors_name_the_key(change, word):
@@ -76,6 +77,33 @@ def test_rope_keys_and_qkv_bias():
     dropped = set(with_bias.tensor_specs()) - set(without.tensor_specs())
     assert len(dropped) == 3 * CONFIG_A["num_hidden_layers"]
     assert all(n.endswith("_proj.bias") for n in dropped)
+
+
+def test_keys_that_may_be_absent_or_lists():
+    """`eos_token_id` is one id or a list, and every id of the list ends a generation; without
+    experts every layer is dense and asks for no expert tensors; without a shared expert a
+    sparse layer has none of its tensors."""
+    from ninfer_amd import Qwen2MoeConfig
+    from ninfer_amd.loading import build_spec
+    from ninfer_amd.parts import SparseMoE, SwiGLU
+    assert Qwen2MoeConfig.from_dict(CONFIG_A).eos_token_ids == ()
+    assert Qwen2MoeConfig.from_dict(dict(CONFIG_A, eos_token_id=7)).eos_token_ids == (7,)
+    c = Qwen2MoeConfig.from_dict(dict(CONFIG_A, eos_token_id=[9, 4]))
+    assert c.eos_token_ids == (9, 4) and c.eos_token_id == 9
+    _, spec = build_spec(dict(CONFIG_A, eos_token_id=[9, 4]))
+    assert spec.eos_token_ids == (9, 4)
+    dense = {k: v for k, v in CONFIG_A.items() if k not in (
+        "num_experts", "num_experts_per_tok", "moe_intermediate_size",
+        "shared_expert_intermediate_size")}
+    cfg, spec = build_spec(dense)
+    assert cfg.num_experts == 0 and all(type(b.feed_forward) is SwiGLU for b in spec.blocks)
+    assert not any("expert" in n or ".gate.weight" in n for n in spec.tensor_specs())
+    no_shared = {k: v for k, v in CONFIG_A.items() if k != "shared_expert_intermediate_size"}
+    _, spec = build_spec(no_shared)
+    assert all(type(b.feed_forward) is SparseMoE and b.feed_forward.shared is None
+               for b in spec.blocks)
+    assert not any("shared_expert" in n for n in spec.tensor_specs())
+    assert "model.layers.0.mlp.experts.3.up_proj.weight" in spec.tensor_specs()
 
 
 def test_registry_resolves_by_architecture_name():

@@ -280,7 +280,7 @@ def random_config(seed: int) -> dict:
     experts = rng.choice([1, 2, 3, 5, 8, 17, 60, 70])
     window = rng.choice([None, None, 8, 24, 40, 70])
     layers = rng.randint(1, 3)
-    return {
+    cfg = {
         "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe",
         "num_hidden_layers": layers, "hidden_size": rng.choice([48, 64, 72, 96, 100, 128, 136, 160, 200]),
         "num_attention_heads": nkv * group, "num_key_value_heads": nkv,
@@ -296,3 +296,12 @@ def random_config(seed: int) -> dict:
         "rms_norm_eps": rng.choice([1e-6, 1e-5]), "tie_word_embeddings": rng.random() < 0.5,
         "hidden_act": "silu", "qkv_bias": rng.random() < 0.75,
     }
+    # (drawn last, so that the configurations of earlier seeds stay what they were)
+    lacks = rng.random()
+    if lacks < 0.15:     # a sparse layer without a shared expert
+        del cfg["shared_expert_intermediate_size"]
+    elif lacks < 0.22:   # no experts at all: every layer dense
+        for key in ("num_experts", "num_experts_per_tok", "moe_intermediate_size",
+                    "shared_expert_intermediate_size"):
+            del cfg[key]
+    return cfg
