@@ -71,6 +71,7 @@ extern "C" long long ninfer_attention_workspace_floats(int T, int Hq, int D, int
 extern "C" int ninfer_attention_decode_plan(const AttnArgs* a, int* kernel, int* chunk, int* n_chunks) {
   *kernel = 0;
   *chunk = *n_chunks = 0;
+  if (int rc = attention_check(*a)) return rc;
   if (!attention_decode_takes(*a)) return 0;
   bool heads;
   attention_decode_plan(*a, &heads, chunk, n_chunks);

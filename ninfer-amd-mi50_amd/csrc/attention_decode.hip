@@ -56,7 +56,9 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
   const int group = a.Hq / a.Hkv;
   const int h0 = g * group + hg * GQ;                // first query head of this block
   const int n_heads = min(GQ, group - hg * GQ);
-  const int pos = a.positions[t];
+  // (a position beyond the host's bound max_kv_len would index past the chunks the launch
+  // and the workspace were sized for: it is read as the last position inside the bound)
+  const int pos = min(a.positions[t], a.max_kv_len - 1);
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int chunk_id = blockIdx.y;
   const int c0 = chunk_id * kChunk;
@@ -209,9 +211,9 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_merge_kernel(AttnAr
   float* part_s = merge_s + 2 * n_chunks;
   __shared__ float red[2 * kMergeThreads / 64];
   const int t = blockIdx.x, h = blockIdx.y, D = a.D, tid = threadIdx.x;
-  const int pos = a.positions[t];
+  const int pos = min(a.positions[t], a.max_kv_len - 1);   // as in pass 1: never past n_chunks
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
-  const int c_lo = lo / kChunk, c_hi = pos / kChunk;
+  const int c_lo = lo / kChunk, c_hi = min(pos / kChunk, n_chunks - 1);
   const float* ws = a.workspace + ((int64_t)t * a.Hq + h) * n_chunks * (D + 2);
   float mx = -1e30f;
   for (int c = c_lo + tid; c <= c_hi; c += kMergeThreads) {

@@ -81,7 +81,7 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
     row0 = blockIdx.z;
     g = blockIdx.x;
     chunk_id = blockIdx.y;
-    const int pos = a.positions[row0];
+    const int pos = min(a.positions[row0], a.max_kv_len - 1);   // as the merge kernel reads it
     const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
     const int c0 = chunk_id * CHUNK;
     if (c0 > pos || c0 + CHUNK <= lo) return;   // chunk outside the row's keys

@@ -26,6 +26,9 @@ constexpr int kWave = 64;
 // workgroups to them in turn (block id mod 8). Kernels that share operands through L2 map
 // block ids to work with this number.
 constexpr int kXcds = 8;
+// Rows of a tall tile of the grouped products (the height of gemm_tile_direct's tiles):
+// what routing's list of tall tiles is made for.
+constexpr int kGroupedTileRows = 256;
 
 // Butterfly reductions over the 64 lanes of a wave: offsets 32 -> 1.
 __device__ __forceinline__ float wave_sum(float v) {

@@ -17,7 +17,7 @@ struct GemmArgs {
   const int* a_index;    // sorted row -> a_index[r] / a_div is the row of A, or null
   const int* c_index;    // sorted row -> row of C, or null
   const int* tiles16;    // grouped: {expert, first row, end row, 0} per 16-row tile, or null
-  const int* tiles64;    // the same for tiles of big_rows rows
+  const int* tiles_big;  // the same for the tall tiles (256 rows: gemm_tile_direct's)
   const int* tile_counts;  // {number of 16-row tiles, number of big tiles}
   int64_t w_group_stride;  // elements between the weights of two groups
   int M;                 // rows (dense) or number of sorted rows (grouped)
@@ -30,7 +30,6 @@ struct GemmArgs {
   int in_dtype;          // of A and W
   int out_dtype;         // of C
   int epilogue;
-  int big_rows;          // rows of a big grouped tile: 64, 128 or 256 (0: 64)
   int k_parts;           // the K range is cut into this many parts, one per blockIdx.z, part z
                          // writing its sums to C + z * M * ldc (0 or 1: no cut); set by
                          // gemm_split, not by callers
@@ -39,7 +38,8 @@ struct GemmArgs {
   // What tests and measurements ask of one call (all 0: the library chooses). Per call, not
   // state of the library: a caller that forgets to reset it changes nothing for the next.
   int64_t split_min_bytes;  // least bytes of weights for a cut along K (0: 48 MB)
-  int force_kernel;      // many-row kernel: 1, 2, 3 = tiles of 64, 128, 256 rows
+  int force_kernel;      // many-row kernel: 1, 2, 3 = tiles of 64, 128, 256 rows (grouped
+                         // products run 256-row tiles unless told otherwise here)
   int skinny_two;        // few-row grouped products with two feature sets per block: 1 = whenever
                          // the shape allows, -1 = never
 };

@@ -47,23 +47,20 @@ extern "C" int ninfer_gemm_pair(const GemmArgs* a, const GemmArgs* b, int force_
 
 static int route_by(const GemmArgs& a, const RouteArgs& rt, hipStream_t stream) {
   const float* logits = (const float*)a.C;
-  if (a.M <= 16)
-    return ninfer_moe_route_small(logits, a.ldc, a.M, rt.E, rt.k, rt.renorm, rt.ids, rt.wts,
-                                  rt.offsets, rt.order, rt.tiles16, rt.tiles64, rt.tile_counts,
-                                  rt.big_rows, stream);
-  int rc = ninfer_router_topk(logits, a.ldc, a.M, rt.E, rt.k, rt.renorm, rt.ids, rt.wts, stream);
+  if (a.M <= 16) return ninfer_moe_route_small(logits, a.ldc, a.M, &rt, stream);
+  int rc = ninfer_router_topk(logits, a.ldc, a.M, &rt, stream);
   if (rc) return rc;
-  return ninfer_moe_align(rt.ids, a.M * rt.k, rt.E, rt.offsets, rt.order, rt.tiles16, rt.tiles64,
-                          rt.tile_counts, rt.big_rows, stream);
+  return ninfer_moe_align(rt.ids, a.M * rt.k, rt.E, rt.offsets, rt.order, rt.tiles16,
+                          rt.tiles_big, rt.tile_counts, stream);
 }
 
 static int route_check(const GemmArgs& a, const RouteArgs& rt) {
   NINFER_REQUIRE(!a.offsets && a.out_dtype == kF32 && a.N >= rt.E && a.ldc >= rt.E,
                  "gemm route: the product must be dense with 32-bit logits of %d experts", rt.E);
-  NINFER_REQUIRE((!rt.tiles16) == (!rt.tiles64) && (!rt.tiles16) == (!rt.tile_counts),
+  NINFER_REQUIRE((!rt.tiles16) == (!rt.tiles_big) && (!rt.tiles16) == (!rt.tile_counts),
                  "gemm route: tile lists come together or not at all");
-  NINFER_REQUIRE(rt.big_rows == 64 || rt.big_rows == 128 || rt.big_rows == 256,
-                 "gemm route: big tiles of %d rows", rt.big_rows);
+  NINFER_REQUIRE(rt.score == kScoreSoftmax || rt.score == kScoreSigmoid,
+                 "gemm route: score function %d is neither softmax (0) nor sigmoid (1)", rt.score);
   return 0;
 }
 

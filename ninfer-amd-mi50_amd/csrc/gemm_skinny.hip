@@ -336,13 +336,13 @@ __device__ __forceinline__ void skinny_route_block(const GemmArgs& a, const Rout
   int* cnt = (int*)(logits_s + 16 * ldl);   // E + 1 counters, then the chosen experts
   int* ids_s = cnt + rt.E + 1;
   for (int t = wave; t < T; t += waves) {
-    const int mine = route_row<NPL>(logits_s + t * ldl, rt.E, rt.k, rt.renorm, rt.ids + (int64_t)t * rt.k,
+    const int mine = route_row<NPL>(logits_s + t * ldl, rt, rt.ids + (int64_t)t * rt.k,
                                     rt.wts + (int64_t)t * rt.k, lane);
     if (lane < rt.k) ids_s[t * rt.k + lane] = mine;
   }
   __syncthreads();
-  align_block(ids_s, T * rt.k, rt.E, rt.offsets, rt.order, rt.tiles16, rt.tiles64, rt.tile_counts,
-              rt.big_rows, cnt);
+  align_block(ids_s, T * rt.k, rt.E, rt.offsets, rt.order, rt.tiles16, rt.tiles_big,
+              rt.tile_counts, cnt);
 }
 
 // The first block is the router's (product `a` and routing `rt`), the others are the tiles of
@@ -499,8 +499,9 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream) {
 // the time the other product's blocks take anyway).
 // A router's product of few rows and few features, and the routing by it, in one block.
 bool gemm_skinny_route_takes(const GemmArgs& a, const RouteArgs& rt) {
-  if (!gemm_skinny_takes(a) || a.offsets || a.bias || a.out_dtype != kF32 ||
-      a.epilogue != kEpilogueNone)
+  // the routing block reads A by row and writes C by row: no row indices, one group
+  if (!gemm_skinny_takes(a) || a.offsets || a.a_index || a.c_index || a.groups > 1 || a.bias ||
+      a.out_dtype != kF32 || a.epilogue != kEpilogueNone)
     return false;
   return a.M <= SM && a.N <= kRouteMaxFeatures && a.N >= rt.E && (int64_t)a.N * a.K <= (1 << 19) &&
          rt.E >= 1 && rt.k >= 1 && rt.k <= rt.E && rt.k <= 64;

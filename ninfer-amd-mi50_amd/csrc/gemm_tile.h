@@ -55,7 +55,9 @@ __device__ inline bool tile_rows(const GemmArgs& a, int bx, int* info, int& row0
                                  int& group) {
   group = 0;
   if (a.offsets) {
-    if (!grouped_tile(a, a.tiles64, 1, TM, bx, info)) return false;
+    // the tile list is made for the tall tiles; other heights count their tiles from the offsets
+    if (!grouped_tile(a, TM == kGroupedTileRows ? a.tiles_big : nullptr, 1, TM, bx, info))
+      return false;
     __syncthreads();
     group = info[2];
     row0 = info[0];

@@ -228,8 +228,6 @@ constexpr int64_t kSplitMinBytes = 48 << 20;   // GemmArgs::split_min_bytes lowe
 
 template <int TM, int TN, int TK, int NW, int WGM, int P, int OCC = 2>
 static int launch_tile(const GemmArgs& a, hipStream_t stream) {
-  if (a.offsets && a.tiles64 && TM != (a.big_rows ? a.big_rows : 64))
-    return set_error(-1, "gemm: the grouped tile lists are made for %d rows, not %d", a.big_rows, TM);
   const bool swiglu = a.epilogue == kEpilogueSwiGLU;
   int m_tiles = (a.M + TM - 1) / TM + (a.offsets ? a.groups : 0);
   if (a.offsets) m_tiles = (m_tiles + kXcds - 1) / kXcds * kXcds;   // block_to_tile's bijection
@@ -257,14 +255,16 @@ static int launch_tile(const GemmArgs& a, hipStream_t stream) {
 }
 
 int gemm_tile(const GemmArgs& a, hipStream_t stream) {
-  // Tile height. Grouped: as the tile lists were made. Dense: the tallest tile that still
-  // gives every CU a block (taller tiles read less per product, but fewer of them fill the
-  // chip). force_kernel (tests) forces 64, 128 or 256 rows on dense products.
+  // Tile height. Grouped: the tall tile (it loads and multiplies only the 32-row blocks that
+  // hold rows, so it beats the lower ones from 17 rows per expert on, the fewest that come
+  // here). Dense: the tallest tile that still gives every CU a block (taller tiles read less
+  // per product, but fewer of them fill the chip). force_kernel (tests) forces 64, 128 or
+  // 256 rows.
   int rows;
-  if (a.offsets) {
-    rows = a.big_rows ? a.big_rows : 64;
-  } else if (a.force_kernel >= 1 && a.force_kernel <= 3) {
+  if (a.force_kernel >= 1 && a.force_kernel <= 3) {
     rows = 32 << a.force_kernel;
+  } else if (a.offsets) {
+    rows = kGroupedTileRows;
   } else {
     const int n_units = a.epilogue == kEpilogueSwiGLU ? 2 * a.N : a.N;   // W rows
     auto blocks = [&](int tm, int tn) { return ((a.M + tm - 1) / tm) * ((n_units + tn - 1) / tn); };

@@ -317,9 +317,7 @@ static int launch_direct(const GemmArgs& a, hipStream_t stream) {
 }
 
 int gemm_tile_direct(const GemmArgs& a, hipStream_t stream) {
-  if (a.offsets && a.tiles64 && a.big_rows != direct::TM)
-    return set_error(-1, "gemm: the grouped tile lists are made for %d rows, not %d", a.big_rows,
-                     direct::TM);
+  static_assert(direct::TM == kGroupedTileRows, "the grouped tile lists are made for this height");
   // k tiles of 64: measured faster than tiles of 32 in twice the buffers (whole 128-byte
   // lines per row beat the deeper queue of loads)
   return launch_direct<64>(a, stream);

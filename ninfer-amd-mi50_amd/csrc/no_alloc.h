@@ -17,6 +17,13 @@
 //    every GPU the library runs on holds until the process ends): 8 rows of 16
 //    heads of 128 at 30,000 keys, or 64 rows at 3,900; beyond that the call is
 //    refused;
+//  - max_kv_len must exceed every position in `positions` (it sizes the launch and the
+//    chunks a row's partial results are laid out in); a position at or beyond it is read
+//    as max_kv_len - 1, so nothing is written or read outside the array, and the row's
+//    result is then that of the shorter context;
+//  - ninfer_decode_attention_static_init() is best called once per device at set-up and
+//    outside any graph capture: the first lookup of the array's address on a device may
+//    load the library's code object there;
 //  - the workspace and workspace_floats fields of the arguments are ignored;
 //  - nothing in the array has to start at zero: pass 1 writes every entry that
 //    the merge reads, so the last call's contents do not matter;

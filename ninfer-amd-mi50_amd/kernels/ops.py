@@ -26,12 +26,12 @@ class _GemmArgs(ctypes.Structure):
     _fields_ = [("A", ctypes.c_void_p), ("W", ctypes.c_void_p), ("C", ctypes.c_void_p),
                 ("bias", ctypes.c_void_p), ("offsets", ctypes.c_void_p),
                 ("a_index", ctypes.c_void_p), ("c_index", ctypes.c_void_p),
-                ("tiles16", ctypes.c_void_p), ("tiles64", ctypes.c_void_p),
+                ("tiles16", ctypes.c_void_p), ("tiles_big", ctypes.c_void_p),
                 ("tile_counts", ctypes.c_void_p), ("w_group_stride", ctypes.c_int64),
                 ("M", ctypes.c_int), ("N", ctypes.c_int), ("K", ctypes.c_int),
                 ("lda", ctypes.c_int), ("ldc", ctypes.c_int), ("groups", ctypes.c_int),
                 ("a_div", ctypes.c_int), ("in_dtype", ctypes.c_int), ("out_dtype", ctypes.c_int),
-                ("epilogue", ctypes.c_int), ("big_rows", ctypes.c_int),
+                ("epilogue", ctypes.c_int),
                 ("k_parts", ctypes.c_int), ("workspace", ctypes.c_void_p),
                 ("workspace_floats", ctypes.c_int64), ("split_min_bytes", ctypes.c_int64),
                 ("force_kernel", ctypes.c_int), ("skinny_two", ctypes.c_int)]
@@ -40,9 +40,14 @@ class _GemmArgs(ctypes.Structure):
 class _RouteArgs(ctypes.Structure):
     _fields_ = [("ids", ctypes.c_void_p), ("wts", ctypes.c_void_p), ("offsets", ctypes.c_void_p),
                 ("order", ctypes.c_void_p), ("tiles16", ctypes.c_void_p),
-                ("tiles64", ctypes.c_void_p), ("tile_counts", ctypes.c_void_p),
+                ("tiles_big", ctypes.c_void_p), ("tile_counts", ctypes.c_void_p),
+                ("choice_bias", ctypes.c_void_p),
                 ("E", ctypes.c_int), ("k", ctypes.c_int), ("renorm", ctypes.c_int),
-                ("big_rows", ctypes.c_int)]
+                ("score", ctypes.c_int), ("scale", ctypes.c_float)]
+
+
+BIG_TILE_ROWS = 256   # rows of a tall tile of the grouped products (the library's kGroupedTileRows)
+_SCORES = {"softmax": 0, "sigmoid": 1}
 
 
 class _AttnArgs(ctypes.Structure):
@@ -401,15 +406,13 @@ class HipOps:
     def _gemm(self, a, w, c, *, n, k, m, bias=None, offsets=None, a_index=None, c_index=None,
               a_div=1, groups=1, epilogue=0, w_group_stride=0, tiles=None, only_if_split=False):
         t16 = t64 = tc = None
-        big = 0
         if tiles is not None and tiles.tiles16 is not None:
-            t16, t64, tc = tiles.tiles16.data_ptr(), tiles.tiles64.data_ptr(), \
+            t16, t64, tc = tiles.tiles16.data_ptr(), tiles.tiles_big.data_ptr(), \
                 tiles.tile_counts.data_ptr()
-            big = tiles.big_rows
         args = _GemmArgs(a.data_ptr(), w.data_ptr(), c.data_ptr(), _ptr(bias), _ptr(offsets),
                          _ptr(a_index), _ptr(c_index), t16, t64, tc, w_group_stride, m, n, k,
                          a.shape[1],
-                         c.shape[1], groups, a_div, _DT[a.dtype], _DT[c.dtype], epilogue, big)
+                         c.shape[1], groups, a_div, _DT[a.dtype], _DT[c.dtype], epilogue)
         args.force_kernel = self._tune["force_kernel"]
         args.split_min_bytes = self._tune["split_min_bytes"]
         args.skinny_two = self._tune["skinny_two"]
@@ -576,27 +579,48 @@ class HipOps:
                    groups=e, w_group_stride=hidden * inner, tiles=tiles)
 
     # ---- routing ------------------------------------------------------------------
-    def router_topk(self, logits, experts, top_k, renorm, ids, wts):
+    def _route_args(self, experts, top_k, renorm, ids, wts, r=None, score="softmax",
+                    choice_bias=None, scale=1.0):
+        """The router's parameters and the places routing writes, as the library takes them.
+        `score`: 'softmax' over all experts or 'sigmoid' of each logit; `choice_bias` [experts]
+        is added to the scores for the choice of experts only (the weights are the scores);
+        `scale` multiplies every weight, after the renormalisation if there is one."""
+        _need(score in _SCORES, f"routing: score {score!r} is not one of {sorted(_SCORES)}")
+        _need(1 <= top_k <= experts, f"routing: top_k {top_k} not in [1, {experts}]")
+        if choice_bias is not None:
+            _dev(choice_bias, "choice_bias", torch.float32, 1)
+            _need(choice_bias.shape[0] == experts, "routing: one bias per expert")
+        t16 = t64 = tc = offsets = order = None
+        if r is not None:
+            offsets, order = r.offsets.data_ptr(), r.order.data_ptr()
+            t16, t64, tc = self._tile_ptrs(r, r.order.shape[0], experts)
+        args = _RouteArgs(ids.data_ptr(), wts.data_ptr(), offsets, order, t16, t64, tc,
+                          _ptr(choice_bias), experts, top_k, 1 if renorm else 0, _SCORES[score],
+                          float(scale))
+        return args
+
+    def router_topk(self, logits, experts, top_k, renorm, ids, wts, score="softmax",
+                    choice_bias=None, scale=1.0):
         _dev(logits, "logits", torch.float32, 2)
         _dev(ids, "ids", torch.int32, 2)
         _dev(wts, "wts", torch.float32, 2)
         t = logits.shape[0]
         _need(ids.shape == (t, top_k) and wts.shape == (t, top_k), "router_topk: output shapes")
+        args = self._route_args(experts, top_k, renorm, ids, wts, None, score, choice_bias, scale)
         self._ok(self.lib.ninfer_router_topk(
-            ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, experts, top_k,
-            1 if renorm else 0, ctypes.c_void_p(ids.data_ptr()), ctypes.c_void_p(wts.data_ptr()),
+            ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, ctypes.byref(args),
             self._stream()))
 
     def _tile_ptrs(self, tiles, n, experts):
         if tiles is None or tiles.tiles16 is None:
             return None, None, None
         _dev(tiles.tiles16, "tiles16", torch.int32, 2)
-        _dev(tiles.tiles64, "tiles64", torch.int32, 2)
+        _dev(tiles.tiles_big, "tiles_big", torch.int32, 2)
         _dev(tiles.tile_counts, "tile_counts", torch.int32, 1)
         _need(tiles.tiles16.shape == (min(n, n // 16 + experts), 4)
-              and tiles.tiles64.shape == (n // 64 + experts, 4) and tiles.tile_counts.shape[0] == 2,
-              "routing: tile lists have the wrong sizes")
-        return tiles.tiles16.data_ptr(), tiles.tiles64.data_ptr(), tiles.tile_counts.data_ptr()
+              and tiles.tiles_big.shape == (n // BIG_TILE_ROWS + experts, 4)
+              and tiles.tile_counts.shape[0] == 2, "routing: tile lists have the wrong sizes")
+        return tiles.tiles16.data_ptr(), tiles.tiles_big.data_ptr(), tiles.tile_counts.data_ptr()
 
     def moe_align(self, ids, experts, offsets, order, tiles=None):
         _dev(ids, "ids", torch.int32)
@@ -608,16 +632,16 @@ class HipOps:
         self._ok(self.lib.ninfer_moe_align(
             ctypes.c_void_p(ids.data_ptr()), ids.numel(), experts,
             ctypes.c_void_p(offsets.data_ptr()), ctypes.c_void_p(order.data_ptr()),
-            ctypes.c_void_p(t16), ctypes.c_void_p(t64), ctypes.c_void_p(tc),
-            getattr(tiles, "big_rows", 64) if tiles is not None else 64, self._stream()))
+            ctypes.c_void_p(t16), ctypes.c_void_p(t64), ctypes.c_void_p(tc), self._stream()))
 
-    def moe_route(self, logits, experts, top_k, renorm, r):
-        """Softmax + top-k per row and the grouping by expert, into the routing
-        record `r` (ids, weights, offsets, order, tile lists): one launch for up
-        to 16 rows (one block does both), two for more (top-k by one wave per
-        row in parallel, then the grouping). Inside `together()`, after the
-        product that writes `logits`, it is held back with the products and
-        launched with them (for few rows: by the block that computes the logits)."""
+    def moe_route(self, logits, experts, top_k, renorm, r, score="softmax", choice_bias=None,
+                  scale=1.0):
+        """Scores + top-k per row (see `_route_args` for the router's parameters) and the
+        grouping by expert, into the routing record `r` (ids, weights, offsets, order, tile
+        lists): one launch for up to 16 rows (one block does both), two for more (top-k by
+        one wave per row in parallel, then the grouping). Inside `together()`, after the
+        product that writes `logits`, it is held back with the products and launched with
+        them (for few rows: by the block that computes the logits)."""
         t = logits.shape[0]
         _dev(logits, "logits", torch.float32, 2)
         _dev(r.ids, "ids", torch.int32, 2)
@@ -628,29 +652,25 @@ class HipOps:
         _need(r.ids.shape == (t, top_k) and r.weights.shape == (t, top_k)
               and r.offsets.shape[0] == experts + 1 and r.order.shape[0] == t * top_k,
               "moe_route: output sizes")
+        rargs = self._route_args(experts, top_k, renorm, r.ids, r.weights, r, score, choice_bias,
+                                 scale)
         if self._held is not None:
             _need(self._held_route is None, "together(): one routing at most")
-            t16, t64, tc = self._tile_ptrs(r, t * top_k, experts)
-            rargs = _RouteArgs(r.ids.data_ptr(), r.weights.data_ptr(), r.offsets.data_ptr(),
-                               r.order.data_ptr(), t16, t64, tc, experts, top_k,
-                               1 if renorm else 0, r.big_rows)
-            self._held_route = (logits, rargs, (logits, experts, top_k, renorm, r))
+            self._held_route = (logits, rargs, (logits, rargs, r, choice_bias))
             return
-        self._route_now(logits, experts, top_k, renorm, r)
+        self._route_now(logits, rargs, r)
 
-    def _route_now(self, logits, experts, top_k, renorm, r):
+    def _route_now(self, logits, rargs, r, keep=None):
         t = logits.shape[0]
         if t > 16:
-            self.router_topk(logits, experts, top_k, renorm, r.ids, r.weights)
-            self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r)
+            self._ok(self.lib.ninfer_router_topk(
+                ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, ctypes.byref(rargs),
+                self._stream()))
+            self.moe_align(r.ids, rargs.E, r.offsets, r.order, tiles=r)
             return
-        t16, t64, tc = self._tile_ptrs(r, t * top_k, experts)
         self._ok(self.lib.ninfer_moe_route_small(
-            ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, experts, top_k,
-            1 if renorm else 0, ctypes.c_void_p(r.ids.data_ptr()),
-            ctypes.c_void_p(r.weights.data_ptr()), ctypes.c_void_p(r.offsets.data_ptr()),
-            ctypes.c_void_p(r.order.data_ptr()), ctypes.c_void_p(t16), ctypes.c_void_p(t64),
-            ctypes.c_void_p(tc), r.big_rows, self._stream()))
+            ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, ctypes.byref(rargs),
+            self._stream()))
 
     # ---- attention ------------------------------------------------------------------
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,

@@ -4,11 +4,11 @@ from .base import (Block, CacheNeed, CacheView, CallInfo, FeedForward, Mixer, No
 from .block import PreNormBlock
 from .embedding import LMHead, TokenEmbedding
 from .mlp import SwiGLU
-from .moe import RoutedExperts, SoftmaxTopKRouter, SparseMoE
+from .moe import RoutedExperts, Routing, SoftmaxTopKRouter, SparseMoE, TopKRouter
 from .norm import RMSNorm
 from .rotary import NoPosition, Rotary
 
 __all__ = ["Attention", "Block", "CacheNeed", "CacheView", "CallInfo", "FeedForward", "Mixer",
            "Norm", "Part", "PendingRows", "PoolSpec", "settle", "PositionEncoding", "StepContext", "WeightBinder", "PreNormBlock",
-           "LMHead", "TokenEmbedding", "SwiGLU", "RoutedExperts", "SoftmaxTopKRouter",
+           "LMHead", "TokenEmbedding", "SwiGLU", "RoutedExperts", "Routing", "SoftmaxTopKRouter", "TopKRouter",
            "SparseMoE", "RMSNorm", "NoPosition", "Rotary"]

@@ -23,22 +23,41 @@ from .base import FeedForward, Part, PendingRows, StepContext, WeightBinder
 from .mlp import SwiGLU
 
 
-class SoftmaxTopKRouter(Part):
-    def __init__(self, prefix: str, hidden: int, experts: int, top_k: int, renorm: bool):
+class TopKRouter(Part):
+    """logits = x Wr^T (32-bit); scores s = softmax over all experts, or sigmoid of each
+    logit (`score`); the `top_k` experts with the largest s (+ a per-expert bias of the
+    checkpoint, `prefix + "choice_bias"`, when `choice_bias`: it decides the choice only)
+    are chosen, ties to the lower index; their weights are their scores, divided by their
+    sum when `renorm`, times `scale`. Softmax without bias and scale 1 is this
+    architecture's router (reference src/ops/moe.hip:65-82, which always renormalises)."""
+
+    def __init__(self, prefix: str, hidden: int, experts: int, top_k: int, renorm: bool,
+                 score: str = "softmax", scale: float = 1.0, choice_bias: bool = False):
         if top_k > experts:
             raise ValueError(f"top_k ({top_k}) exceeds the number of experts ({experts})")
+        if score not in ("softmax", "sigmoid"):
+            raise ValueError(f"score must be 'softmax' or 'sigmoid', got {score!r}")
         self.prefix = prefix
         self.hidden = hidden
         self.experts = experts
         self.top_k = top_k
         self.renorm = renorm
+        self.score = score
+        self.scale = float(scale)
+        self.has_choice_bias = choice_bias
         self.weight: Optional[torch.Tensor] = None
+        self.choice_bias: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {self.prefix + "weight": TensorSpec((self.experts, self.hidden))}
+        specs = {self.prefix + "weight": TensorSpec((self.experts, self.hidden))}
+        if self.has_choice_bias:
+            specs[self.prefix + "choice_bias"] = TensorSpec((self.experts,), role="bias")
+        return specs
 
     def bind(self, w: WeightBinder) -> None:
         self.weight = w.matrix(self.prefix + "weight")
+        if self.has_choice_bias:
+            self.choice_bias = w.float32(self.prefix + "choice_bias")
 
     def logits(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
         out = ctx.empty((x.shape[0], self.experts), torch.float32)
@@ -53,32 +72,29 @@ class SoftmaxTopKRouter(Part):
         r = Routing(ids=ctx.empty((t, k), torch.int32), weights=ctx.empty((t, k), torch.float32),
                     offsets=ctx.empty((e + 1,), torch.int32), order=ctx.empty((n,), torch.int32),
                     tiles16=ctx.empty((min(n, n // 16 + e), 4), torch.int32),
-                    tiles64=ctx.empty((n // 64 + e, 4), torch.int32),
-                    tile_counts=ctx.empty((2,), torch.int32),
-                    big_rows=big_tile_rows(n, e))
-        ctx.ops.moe_route(logits, e, k, self.renorm, r)
+                    tiles_big=ctx.empty((n // Routing.BIG_ROWS + e, 4), torch.int32),
+                    tile_counts=ctx.empty((2,), torch.int32))
+        ctx.ops.moe_route(logits, e, k, self.renorm, r, score=self.score,
+                          choice_bias=self.choice_bias, scale=self.scale)
         return r
 
 
-def big_tile_rows(routed_rows: int, experts: int) -> int:
-    """Rows of the big tiles of the grouped products (64, 128 or 256): the taller, the
-    fewer times an expert's weights are read. The 256-row kernel loads and multiplies
-    only the 32-row blocks of a tile that hold rows, so a mostly empty tile costs
-    little: measured from 17 rows per expert on (the fewest that take the tile
-    kernels at all), it beats the lower tiles at every size."""
-    return 256
+SoftmaxTopKRouter = TopKRouter   # the default parameters: this architecture's router
 
 
 class Routing:
     """What routing leaves on the device: chosen experts and weights per row,
     the (row, choice) indices grouped by expert (`order`, `offsets`), and the
-    lists of 16-row and 64-row tiles the grouped products walk."""
+    lists of 16-row and of tall (256-row) tiles the grouped products walk:
+    `tiles16` [min(n, n // 16 + experts), 4], `tiles_big` [n // 256 + experts, 4]
+    and `tile_counts` [2] for n routed rows, or all three None."""
 
-    def __init__(self, ids, weights, offsets, order, tiles16=None, tiles64=None, tile_counts=None,
-                 big_rows=64):
+    BIG_ROWS = 256   # rows of a tall tile: one height serves every count of rows per expert
+
+    def __init__(self, ids, weights, offsets, order, tiles16=None, tiles_big=None,
+                 tile_counts=None):
         self.ids, self.weights, self.offsets, self.order = ids, weights, offsets, order
-        self.tiles16, self.tiles64, self.tile_counts = tiles16, tiles64, tile_counts
-        self.big_rows = big_rows   # rows of a tile in `tiles64`: 64, 128 or 256 (big_tile_rows)
+        self.tiles16, self.tiles_big, self.tile_counts = tiles16, tiles_big, tile_counts
 
 
 class RoutedExperts(Part):

@@ -143,20 +143,26 @@ class PlainOps:
                 continue
             out[rows] = (_f(h[off[g]:off[g + 1]]) @ _f(w_down[g]).T).to(out.dtype)
 
-    def router_topk(self, logits, experts, top_k, renorm, ids, wts):
+    def router_topk(self, logits, experts, top_k, renorm, ids, wts, score="softmax",
+                    choice_bias=None, scale=1.0):
         l = logits[:, :experts]
-        p = torch.exp(l - l.max(-1, keepdim=True).values)
-        p = p / p.sum(-1, keepdim=True)
-        work = p.clone()
+        if score == "sigmoid":
+            p = 1 / (1 + torch.exp(-l))
+        else:
+            p = torch.exp(l - l.max(-1, keepdim=True).values)
+            p = p / p.sum(-1, keepdim=True)
+        work = p.clone() if choice_bias is None else p + choice_bias[None, :]
+        rows = torch.arange(work.shape[0])
         for j in range(top_k):
             best = work.max(-1).values
             # lowest index among the maxima
             idx = torch.argmax((work == best[:, None]).to(torch.int32), dim=-1)
             ids[:, j] = idx.to(torch.int32)
-            wts[:, j] = best
-            work[torch.arange(work.shape[0]), idx] = -1.0
+            wts[:, j] = p[rows, idx]
+            work[rows, idx] = -float("inf")
         if renorm:
             wts /= wts.sum(-1, keepdim=True)
+        wts *= scale
 
     def moe_align(self, ids, experts, offsets, order, tiles=None):
         flat = ids.reshape(-1).long()
@@ -166,15 +172,17 @@ class PlainOps:
         order.copy_(torch.sort(flat, stable=True).indices.to(torch.int32))
         if tiles is not None and tiles.tiles16 is not None:
             off = offsets.tolist()
-            for size, out in ((16, tiles.tiles16), (tiles.big_rows, tiles.tiles64)):
+            for size, out in ((16, tiles.tiles16), (256, tiles.tiles_big)):
                 lst = [[e, r, off[e + 1], 0] for e in range(experts)
                        for r in range(off[e], off[e + 1], size)]
                 if lst:
                     out[:len(lst)] = torch.tensor(lst, dtype=torch.int32, device=out.device)
                 tiles.tile_counts[0 if size == 16 else 1] = len(lst)
 
-    def moe_route(self, logits, experts, top_k, renorm, r):
-        self.router_topk(logits, experts, top_k, renorm, r.ids, r.weights)
+    def moe_route(self, logits, experts, top_k, renorm, r, score="softmax", choice_bias=None,
+                  scale=1.0):
+        self.router_topk(logits, experts, top_k, renorm, r.ids, r.weights, score, choice_bias,
+                         scale)
         self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r)
 
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,

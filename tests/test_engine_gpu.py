@@ -311,13 +311,10 @@ def wide_case(tmp_path_factory):
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
 def test_long_prompt_on_the_many_row_kernels(wide_case, dtype):
     from ninfer_amd import EngineOptions, load_model
-    from ninfer_amd.parts.moe import big_tile_rows
     cfg = CONFIG_WIDE
     dirs, toks = wide_case
     rcfg, w = util.read_folder(dirs[dtype])
     ref = plain_model.forward(w, rcfg, toks)
-    k, e = cfg["num_experts_per_tok"], cfg["num_experts"]
-    assert {big_tile_rows(n * k, e) for n in (640, 200, 60)} == {256}   # full, part-empty and mostly empty tiles
     runner = load_model(dirs[dtype], EngineOptions(dtype=dtype, max_context=704, prefill_chunk=640,
                                                    num_sequences=2, page_size=16))
     # with the shared expert on a stream of its own beside the routed path (the engine does so

@@ -159,6 +159,26 @@ def test_toy_routed_feed_forward_and_another_position_encoding(tmp_path):
         torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
 
 
+def test_toy_router_with_other_scores(tmp_path):
+    """A router of another kind (sigmoid scores, a bias of the checkpoint that decides the
+    choice only, renormalised and scaled weights) built from the framework's router part by
+    parameters alone."""
+    import ninfer_amd
+    toy.register_routed()
+    d = str(tmp_path / "toy_scored")
+    ninfer_amd.write_random_model(d, toy.TOY_SCORED_CONFIG, 12, std=0.3)
+    cfg, w = util.read_folder(d)
+    assert w["layers.1.ff.router.choice_bias"].shape == (6,)
+    runner = runner_for(d, seqs=3)
+    reqs = {f"r{i}": util.random_tokens(n, 83, 60 + i) for i, n in enumerate([7, 26, 15])}
+    ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
+    softmax_like = toy.plain_forward_routed(w, dict(cfg, route_scale=1.0), reqs["r1"])
+    assert (softmax_like - ref["r1"]).abs().max() > 1e-3, "the scale must matter"
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=5, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+
+
 def test_toy_interleaved_pairs(tmp_path):
     """The second toy with neighbouring dims as rotation pairs: the pairing is a property of
     the position encoding that attention hands to the rotation, nothing else changes."""

@@ -239,6 +239,45 @@ def test_toy_routed_feed_forward_and_position_on_the_gpu(tmp_path):
         atol=3e-5, rtol=1e-4)
 
 
+def test_toy_router_with_other_scores_on_the_gpu(tmp_path):
+    """The toy whose router has sigmoid scores, a choice bias, renormalised and scaled weights:
+    parameters of the routing kernels, also where the block that computes a decode step's
+    router logits routes the rows itself. 32-bit against the plain model; bfloat16 (the fused
+    launch of few rows) against the 32-bit engine on the same bf16-rounded weights, on rows
+    that route alike."""
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, load_model
+    toy.register_routed()
+    d = str(tmp_path / "toy_scored")
+    ninfer_amd.write_random_model(d, toy.TOY_SCORED_CONFIG, 12, std=0.3)
+    cfg, w = util.read_folder(d)
+    runner = load_model(d, EngineOptions(dtype="float32", max_context=64, num_sequences=3,
+                                         page_size=4, check_pages=True))
+    reqs = {f"r{i}": util.random_tokens(n, 83, 60 + i) for i, n in enumerate([7, 26, 15, 33])}
+    ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=4, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+    torch.testing.assert_close(
+        util.run_schedule(runner, util.schedule_tail("r3", reqs["r3"], 12))["r3"], ref["r3"],
+        atol=3e-5, rtol=1e-4)
+    d16 = str(tmp_path / "toy_scored_bf16")
+    ninfer_amd.write_random_model(d16, toy.TOY_SCORED_CONFIG, 12, dtype="bfloat16", std=0.3)
+    _, w16 = util.read_folder(d16)
+    ref16 = toy.plain_forward_routed(w16, cfg, reqs["r3"])
+    r16 = load_model(d16, EngineOptions(dtype="bfloat16", max_context=64, num_sequences=3,
+                                        page_size=4, check_pages=True))
+    got16 = util.run_schedule(r16, util.schedule_tail("r3", reqs["r3"], 12))["r3"]
+    # Routing is discontinuous, so single rows have no bound in bfloat16. What is asked: the
+    # typical row lies far closer to the plain model with this router than to the one whose
+    # weights are not scaled.
+    other = toy.plain_forward_routed(w16, dict(cfg, route_scale=1.0), reqs["r3"])
+    err = (got16 - ref16).abs().max(-1).values
+    wrong = (got16 - other).abs().max(-1).values
+    assert float(err.median()) < float(wrong.median()) / 3
+    assert float(err.median()) < 0.03 * float(ref16.abs().max())
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_toy_interleaved_pairs_on_the_gpu(tmp_path, dtype):
     """Neighbouring dims as rotation pairs (a partial rotation of 12 of 16 dims), chosen by

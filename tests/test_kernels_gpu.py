@@ -231,14 +231,14 @@ def test_router_align_experts_combine(ops_mode, gen, dtype, t, e, k, h, inner):
     from ninfer_amd.parts.moe import Routing
     n = t * k
     i32 = lambda *sh: torch.zeros(*sh, device="cuda", dtype=torch.int32)
-    for big in (64, 128, 256):   # every height of the big tiles, whatever the rows per expert
-        tl = Routing(ids1, w1, off1, i32(n), i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2),
-                     big_rows=big)
-        ops.moe_align(ids1, e, i32(e + 1), tl.order, tiles=tl)
+    tl = Routing(ids1, w1, off1, i32(n), i32(min(n, n // 16 + e), 4), i32(n // 256 + e, 4), i32(2))
+    ops.moe_align(ids1, e, i32(e + 1), tl.order, tiles=tl)
+    for force in (0, 1, 2, 3):   # the library's choice, then every tile height of the many-row kernels
         h3 = torch.zeros_like(h1)
-        ops.grouped_swiglu(x, wgu, off1, tl.order, k, h3, tiles=tl)
         y3 = torch.zeros_like(y1)
-        ops.grouped_down(h3, wd, off1, tl.order, y3, tiles=tl)
+        with ops.tuned(force_kernel=force):
+            ops.grouped_swiglu(x, wgu, off1, tl.order, k, h3, tiles=tl)
+            ops.grouped_down(h3, wd, off1, tl.order, y3, tiles=tl)
         y4 = torch.zeros_like(y1)
         plain.grouped_down(h3, wd, off1, tl.order, y4)
         close(y3, y4, dtype, scale=h2.float().abs().max().item() * math.sqrt(inner) * 0.3)
@@ -269,8 +269,7 @@ def test_routing_in_one_call_with_tile_lists(ops, gen, t, e, k):
     def routing():
         i32 = lambda *s: torch.zeros(*s, device="cuda", dtype=torch.int32)
         return Routing(i32(t, k), torch.zeros(t, k, device="cuda"), i32(e + 1), i32(n),
-                       i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2),
-                       big_rows=256 if t >= 1000 else 128 if t >= 300 else 64)
+                       i32(min(n, n // 16 + e), 4), i32(n // 256 + e, 4), i32(2))
     r1, r2 = routing(), routing()
     ops.moe_route(logits, e, k, True, r1)
     PlainOps().moe_route(logits, e, k, True, r2)
@@ -279,7 +278,12 @@ def test_routing_in_one_call_with_tile_lists(ops, gen, t, e, k):
     assert torch.equal(r1.tile_counts, r2.tile_counts)
     n16, n64 = r1.tile_counts.tolist()
     assert torch.equal(r1.tiles16[:n16], r2.tiles16[:n16])
-    assert torch.equal(r1.tiles64[:n64], r2.tiles64[:n64])
+    assert torch.equal(r1.tiles_big[:n64], r2.tiles_big[:n64])
+    rows_big = 0
+    for ex, r0, end, _ in r1.tiles_big[:n64].tolist():
+        rows_big += min(r0 + 256, end) - r0
+        assert int(r1.offsets[ex]) <= r0 < end == int(r1.offsets[ex + 1])
+    assert rows_big == n
     covered = []
     for ex, r0, end, _ in r1.tiles16[:n16].tolist():
         covered += list(range(r0, min(r0 + 16, end)))
@@ -292,8 +296,8 @@ def test_routing_in_one_call_with_tile_lists(ops, gen, t, e, k):
     assert sorted(r1.order.tolist()) == list(range(n))
 
 
-@pytest.mark.parametrize("big", [64, 128, 256])
-def test_grouped_products_do_not_depend_on_the_order_within_an_expert(ops, gen, big):
+@pytest.mark.parametrize("force,big", [(1, 64), (2, 128), (0, 256)])
+def test_grouped_products_do_not_depend_on_the_order_within_an_expert(ops, gen, force, big):
     """The grouping leaves the rows of an expert in the order its atomic counters gave
     them, which differs from run to run. A routed row's result must not depend on its
     place among its expert's rows (on which tile it lands in): with the places reversed
@@ -307,14 +311,15 @@ def test_grouped_products_do_not_depend_on_the_order_within_an_expert(ops, gen, 
     logits = torch.randn(t, e, generator=gen, device="cuda")
     i32 = lambda *s: torch.zeros(*s, device="cuda", dtype=torch.int32)
     r = Routing(i32(t, k), torch.zeros(t, k, device="cuda"), i32(e + 1), i32(n),
-                i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2), big_rows=big)
+                i32(min(n, n // 16 + e), 4), i32(n // 256 + e, 4), i32(2))
     ops.moe_route(logits, e, k, False, r)
 
     def products(routing):
         hh = torch.empty(n, inner, device="cuda", dtype=torch.bfloat16)
         y = torch.empty(n, h, device="cuda", dtype=torch.bfloat16)
-        ops.grouped_swiglu(x, wgu, routing.offsets, routing.order, k, hh, tiles=routing)
-        ops.grouped_down(hh, wd, routing.offsets, routing.order, y, tiles=routing)
+        with ops.tuned(force_kernel=force):
+            ops.grouped_swiglu(x, wgu, routing.offsets, routing.order, k, hh, tiles=routing)
+            ops.grouped_down(hh, wd, routing.offsets, routing.order, y, tiles=routing)
         return y
     y1 = products(r)
     off = r.offsets.tolist()
@@ -382,7 +387,7 @@ def test_products_launched_together(ops_mode, gen, dtype, t, e, k, h, inner, sha
     n = t * k
     i32 = lambda *sh: torch.zeros(*sh, device="cuda", dtype=torch.int32)
     r = Routing(i32(t, k), torch.zeros(t, k, device="cuda"), i32(e + 1), i32(n),
-                i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2))
+                i32(min(n, n // 16 + e), 4), i32(n // 256 + e, 4), i32(2))
     ops.moe_route(logits2[:, :e].contiguous(), e, k, True, r)
     hx = rnd((n, inner), dtype, gen)
     wd = rnd((e, h, inner), dtype, gen, 0.3)
@@ -425,7 +430,7 @@ def test_routing_launched_with_the_products(ops_mode, gen, dtype, t, e, k, h, sh
     kernel on its own."""
     ops = ops_mode
     plain = PlainOps()
-    from ninfer_amd.parts.moe import Routing, big_tile_rows
+    from ninfer_amd.parts.moe import Routing
     n = t * k
     x = rnd((t, h), dtype, gen)
     w_router = rnd((e + extra, h), dtype, gen, 0.3)
@@ -434,8 +439,7 @@ def test_routing_launched_with_the_products(ops_mode, gen, dtype, t, e, k, h, sh
     def record():
         i32 = lambda *sh: torch.full(sh, -7, device="cuda", dtype=torch.int32)
         return Routing(i32(t, k), torch.full((t, k), -7.0, device="cuda"), i32(e + 1), i32(n),
-                       i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2),
-                       big_rows=big_tile_rows(n, e))
+                       i32(min(n, n // 16 + e), 4), i32(n // 256 + e, 4), i32(2))
     for renorm in (True, False):
         logits = torch.full((t, e + extra), 9e9, device="cuda")
         hs = torch.zeros(t, shared_inner, device="cuda", dtype=dtype)
@@ -466,7 +470,7 @@ def test_routing_launched_with_the_products(ops_mode, gen, dtype, t, e, k, h, sh
         assert torch.equal(r.tile_counts, r3.tile_counts)
         n16, nbig = r.tile_counts.tolist()
         assert torch.equal(r.tiles16[:n16], r3.tiles16[:n16])
-        assert torch.equal(r.tiles64[:nbig], r3.tiles64[:nbig])
+        assert torch.equal(r.tiles_big[:nbig], r3.tiles_big[:nbig])
     # the router's product and the routing alone (a router without a shared expert beside it)
     logits4 = torch.full((t, e + extra), 9e9, device="cuda")
     r4, r5 = record(), record()
@@ -508,7 +512,7 @@ def test_grouped_products_at_the_edges_of_the_row_blocks(ops, gen, counts, h, in
     ids = ids[torch.randperm(n, generator=torch.Generator().manual_seed(n))].cuda().reshape(n, 1)
     i32 = lambda *sh: torch.zeros(*sh, device="cuda", dtype=torch.int32)
     r = Routing(ids, torch.ones(n, 1, device="cuda"), i32(e + 1), i32(n), i32(min(n, n // 16 + e), 4),
-                i32(n // 64 + e, 4), i32(2), big_rows=256)
+                i32(n // 256 + e, 4), i32(2))
     ops.moe_align(ids, e, r.offsets, r.order, tiles=r)
     assert (r.offsets[1:] - r.offsets[:-1]).tolist() == counts
     x = rnd((n, h), dtype, gen)
@@ -524,6 +528,92 @@ def test_grouped_products_at_the_edges_of_the_row_blocks(ops, gen, counts, h, in
     ops.grouped_down(h2, wd, r.offsets, r.order, y1, tiles=r)
     plain.grouped_down(h2, wd, r.offsets, r.order, y2)
     close(y1, y2, dtype, scale=h2.float().abs().max().item() * math.sqrt(inner) * 0.3)
+
+
+@pytest.mark.parametrize("t,e,k", [(1, 60, 4), (9, 8, 3), (16, 64, 8), (40, 130, 6), (300, 60, 4)])
+@pytest.mark.parametrize("score", ["softmax", "sigmoid"])
+def test_router_parameters(ops, gen, t, e, k, score):
+    """The router's parameters (score function, a per-expert bias that decides the choice
+    only, renormalisation, a scale on the weights) through every way the routing runs: the
+    top-k kernel alone, the routing call (one block for few rows, two kernels for many), and
+    inside together() with the product that writes the logits (for few bf16 rows the block
+    that computes the logits routes them). Against the twin, and against the definition."""
+    from ninfer_amd.parts.moe import Routing
+    plain = PlainOps()
+    h, n = 64, t * k
+    x = rnd((t, h), torch.bfloat16, gen)
+    w_router = rnd((e, h), torch.bfloat16, gen, 0.4)
+    logits = torch.zeros(t, e, device="cuda")
+    plain.linear(x, w_router, logits)
+    bias = torch.randn(e, generator=gen, device="cuda") * 0.5
+
+    def record():
+        i32 = lambda *sh: torch.full(sh, -7, device="cuda", dtype=torch.int32)
+        return Routing(i32(t, k), torch.full((t, k), -7.0, device="cuda"), i32(e + 1), i32(n),
+                       i32(min(n, n // 16 + e), 4), i32(n // 256 + e, 4), i32(2))
+    for renorm, b, scale in ((False, None, 1.0), (True, bias, 2.5), (False, bias, 0.5),
+                             (True, None, 1.0)):
+        kw = dict(score=score, choice_bias=b, scale=scale)
+        want = record()
+        plain.moe_route(logits, e, k, renorm, want, **kw)
+        # the definition, written out once more: scores, choice by score + bias, weights = scores
+        s = torch.sigmoid(logits) if score == "sigmoid" else torch.softmax(logits, dim=-1)
+        chosen = torch.topk(s if b is None else s + b, k, dim=-1).indices
+        wt = torch.gather(s, 1, chosen)
+        wt = (wt / wt.sum(-1, keepdim=True) if renorm else wt) * scale
+        assert torch.equal(chosen.sort(dim=1).values, want.ids.long().sort(dim=1).values)
+        close(torch.gather(wt, 1, chosen.argsort(dim=1)),
+              torch.gather(want.weights, 1, want.ids.long().argsort(dim=1)), torch.float32)
+        ids, wts = torch.empty_like(want.ids), torch.empty_like(want.weights)
+        ops.router_topk(logits, e, k, renorm, ids, wts, **kw)
+        assert torch.equal(ids, want.ids)
+        close(wts, want.weights, torch.float32)
+        got = record()
+        ops.moe_route(logits, e, k, renorm, got, **kw)
+        assert torch.equal(got.ids, want.ids) and torch.equal(got.offsets, want.offsets)
+        close(got.weights, want.weights, torch.float32)
+        fused, logits2 = record(), torch.zeros_like(logits)
+        with ops.together():
+            ops.linear(x, w_router, logits2)
+            ops.moe_route(logits2, e, k, renorm, fused, **kw)
+        want2 = record()
+        plain.moe_route(logits2, e, k, renorm, want2, **kw)   # by the logits the kernel wrote
+        assert torch.equal(fused.ids, want2.ids) and torch.equal(fused.offsets, want2.offsets)
+        close(fused.weights, want2.weights, torch.float32)
+        assert sorted(fused.order.tolist()) == list(range(n))
+    if e >= 8:
+        # a bias changes the choice and not the weight: expert 5 is pushed into every row's
+        # choice, and its weight is its own score
+        push = torch.zeros(e, device="cuda")
+        push[5] = 100.0
+        got = record()
+        ops.moe_route(logits, e, k, False, got, score=score, choice_bias=push)
+        assert (got.ids[:, 0] == 5).all()
+        s = torch.sigmoid(logits) if score == "sigmoid" else torch.softmax(logits, dim=-1)
+        close(got.weights[:, 0], s[:, 5], torch.float32)
+    from ninfer_amd.kernels import KernelError
+    with pytest.raises(KernelError, match="score"):
+        ops.moe_route(logits, e, k, False, record(), score="tanh")
+
+
+def test_router_ties_under_every_score(ops):
+    """Equal scores: the lower index wins, with softmax and with sigmoid, with a bias that
+    ties two experts exactly, for few rows (one block) and many (a wave per row)."""
+    from ninfer_amd.parts.moe import Routing
+    for t in (2, 40):
+        logits = torch.zeros(t, 8, device="cuda")
+        logits[1, 5] = 1.0
+        bias = torch.zeros(8, device="cuda")
+        bias[6] = bias[3] = 0.25     # experts 3 and 6 tie ahead of the rest
+        for score in ("softmax", "sigmoid"):
+            i32 = lambda *sh: torch.zeros(sh, device="cuda", dtype=torch.int32)
+            r = Routing(i32(t, 3), torch.zeros(t, 3, device="cuda"), i32(9), i32(3 * t),
+                        i32(min(3 * t, 3 * t // 16 + 8), 4), i32(3 * t // 256 + 8, 4), i32(2))
+            ops.moe_route(logits, 8, 3, False, r, score=score)
+            assert r.ids[:2].tolist() == [[0, 1, 2], [5, 0, 1]]
+            ops.moe_route(logits, 8, 3, False, r, score=score, choice_bias=bias)
+            assert r.ids[0].tolist() == [3, 6, 0]
+            assert r.ids[1].tolist() == [3, 6, 5]   # 0.25 lifts both above expert 5's lead
 
 
 def test_router_ties_go_to_the_lower_index(ops):
@@ -902,7 +992,7 @@ def test_grouped_down_with_two_feature_sets_per_block(ops, gen, t, e, k, h, inne
     n = t * k
     i32 = lambda *s: torch.zeros(*s, device="cuda", dtype=torch.int32)
     r = Routing(i32(t, k), torch.zeros(t, k, device="cuda"), i32(e + 1), i32(n),
-                i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2), big_rows=64)
+                i32(min(n, n // 16 + e), 4), i32(n // 256 + e, 4), i32(2))
     ops.moe_route(logits, e, k, False, r)
     hh = rnd((n, inner), torch.bfloat16, gen)
     wd = rnd((e, h, inner), torch.bfloat16, gen, 0.2)
@@ -1015,7 +1105,7 @@ def test_router_rows_without_a_softmax_still_choose(ops, t):
     n = t * k
     i32 = lambda *s: torch.full(s, -7, device="cuda", dtype=torch.int32)
     r = Routing(i32(t, k), torch.zeros(t, k, device="cuda"), i32(e + 1), i32(n),
-                i32(min(n, n // 16 + e), 4), i32(n // 64 + e, 4), i32(2), big_rows=64)
+                i32(min(n, n // 16 + e), 4), i32(n // 256 + e, 4), i32(2))
     ops.moe_route(logits, e, k, False, r)
     ids = r.ids.cpu()
     assert int(ids.min()) >= 0 and int(ids.max()) < e

@@ -45,10 +45,10 @@ def _args(AttnArgs, c, out, n_q, n_kv, d, ps, window, workspace=None):
         c["max_kv_len"], 0)
 
 
-@pytest.mark.parametrize("n_q,n_kv,d,ps,window", [(16, 16, 128, 16, 0), (28, 4, 128, 16, 0),
-                                                  (6, 2, 64, 32, 300)],
+@pytest.mark.parametrize("n_q,n_kv,d,ps,window,kernel", [(16, 16, 128, 16, 0, 1), (28, 4, 128, 16, 0, 2),
+                                                         (6, 2, 64, 32, 300, 2)],
                          ids=["scalar", "heads", "heads-d64-window"])
-def test_decode_attention_without_allocation(n_q, n_kv, d, ps, window):
+def test_decode_attention_without_allocation(n_q, n_kv, d, ps, window, kernel):
     from ninfer_amd.kernels.build import ensure_built
     from ninfer_amd.kernels.ops import _AttnArgs
     lib = ctypes.CDLL(ensure_built())
@@ -57,6 +57,13 @@ def test_decode_attention_without_allocation(n_q, n_kv, d, ps, window):
     lib.ninfer_decode_attention_static_max_floats.restype = ctypes.c_longlong
     assert lib.ninfer_decode_attention_static_init() == 0, lib.ninfer_last_error().decode()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # a warm call: whatever the library loads or maps at its first launch on the device (code
+    # objects, the array's backing) has happened before device memory is watched below
+    c = _case([70, 3], n_q, n_kv, d, ps, seed=2)
+    warm = torch.zeros(2, n_q * d, dtype=torch.bfloat16, device="cuda")
+    assert lib.ninfer_decode_attention_static(
+        ctypes.byref(_args(_AttnArgs, c, warm, n_q, n_kv, d, ps, window)), stream) == 0
+    torch.cuda.synchronize()
     calls = [[4000, 4095, 4096, 1023, 77, 2500, 0, 3999],   # 8 rows, contexts to 4,097 keys
              [300, 129, 5],                                  # smaller: 3 rows, 301 keys
              [900, 2047, 2048, 15, 16]]
@@ -70,11 +77,19 @@ def test_decode_attention_without_allocation(n_q, n_kv, d, ps, window):
         a = _args(_AttnArgs, c, want, n_q, n_kv, d, ps, window, ws)
         assert lib.ninfer_paged_attention(ctypes.byref(a), 0, stream) == 0, lib.ninfer_last_error().decode()
         b = _args(_AttnArgs, c, got, n_q, n_kv, d, ps, window)
-        before = torch.cuda.memory_allocated()
+        # the variant this case means to reach (1: scalar FMAs, 2: grouped heads on the matrix cores)
+        which, chunk, chunks = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        assert lib.ninfer_attention_decode_plan(ctypes.byref(a), ctypes.byref(which),
+                                                ctypes.byref(chunk), ctypes.byref(chunks)) == 0
+        assert which.value == kernel
+        torch.cuda.synchronize()
+        # free bytes of the device, not torch's own count: an allocation by the library
+        # itself (hipMalloc, a lazily loaded code object) would show here
+        before, held = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
         rc = lib.ninfer_decode_attention_static(ctypes.byref(b), stream)
         assert rc == 0, lib.ninfer_last_error().decode()
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.mem_get_info()[0] == before and torch.cuda.memory_allocated() == held
         assert want.float().abs().sum() > 0
         assert torch.equal(got, want), f"call {i}: the outputs differ"
     # a shape whose partial results do not fit the array is refused, and nothing runs
@@ -87,6 +102,20 @@ def test_decode_attention_without_allocation(n_q, n_kv, d, ps, window):
     assert rc != 0 and b"workspace" in lib.ninfer_last_error()
     torch.cuda.synchronize()
     assert (out == 7.0).all()
+    # a position at or beyond max_kv_len (a caller's mistake) is read as the last one inside
+    # the bound: the call stays inside the array and gives what the bound's context gives
+    c = _case([600, 40], n_q, n_kv, d, ps, seed=5)
+    want = torch.zeros(2, n_q * d, dtype=torch.bfloat16, device="cuda")
+    got = torch.zeros_like(want)
+    c["max_kv_len"] = 300
+    c["positions"] = torch.tensor([299, 40], dtype=torch.int32, device="cuda")
+    assert lib.ninfer_decode_attention_static(
+        ctypes.byref(_args(_AttnArgs, c, want, n_q, n_kv, d, ps, window)), stream) == 0
+    c["positions"] = torch.tensor([600, 40], dtype=torch.int32, device="cuda")
+    assert lib.ninfer_decode_attention_static(
+        ctypes.byref(_args(_AttnArgs, c, got, n_q, n_kv, d, ps, window)), stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
     # prompt portions are not its business
     c = _case([10, 20], n_q, n_kv, d, ps, seed=4)
     bad = _args(_AttnArgs, c, torch.zeros(2, n_q * d, dtype=torch.bfloat16, device="cuda"),

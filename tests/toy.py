@@ -156,9 +156,32 @@ class BiasedSwitch(FeedForward):
         ctx.ops.linear(x, self.w_router, logits, bias=self.bias)
         i32 = lambda *shape: ctx.empty(shape, torch.int32)
         r = Routing(i32(t, 1), ctx.empty((t, 1), torch.float32), i32(e + 1), i32(t),
-                    i32(min(t, t // 16 + e), 4), i32(t // 64 + e, 4), i32(2))
+                    i32(min(t, t // 16 + e), 4), i32(t // 256 + e, 4), i32(2))
         ctx.ops.moe_route(logits, e, 1, False, r)
         return PendingRows(self.experts.run(ctx, x, r), r.weights)
+
+
+class ScoredExperts(FeedForward):
+    """Routed experts whose router is not this architecture's: sigmoid scores, a per-expert
+    bias of the checkpoint that decides the choice only, the chosen weights renormalised and
+    scaled. All of it is parameters of the framework's router part and routing kernels; the
+    routing goes with the router's product in one together()."""
+
+    def __init__(self, prefix: str, hidden: int, inner: int, experts: int, top_k: int,
+                 scale: float):
+        from ninfer_amd.parts.moe import TopKRouter
+        self.prefix = prefix
+        self.router = TopKRouter(prefix + "router.", hidden, experts, top_k, renorm=True,
+                                 score="sigmoid", scale=scale, choice_bias=True)
+        self.experts = RoutedExperts(prefix + "experts.", hidden, inner, experts)
+
+    def children(self):
+        return [self.router, self.experts]
+
+    def forward(self, ctx, x, residual):
+        with ctx.ops.together():
+            routing = self.router.route(ctx, self.router.logits(ctx, x))
+        return PendingRows(self.experts.run(ctx, x, routing), routing.weights)
 
 
 @dataclass
@@ -180,9 +203,12 @@ def build_toy_routed(cfg: ToyRoutedConfig) -> ModelSpec:
                          HarmonicPosition(c["rot_dim"], c["slope"], c.get("pairing", "half")),
                          qkv_bias=False,
                          window=c["window"])
+        if c.get("router") == "scored":
+            ff = ScoredExperts(p + "ff.", h, c["inner"], c["experts"], c["top_k"], c["route_scale"])
+        else:
+            ff = BiasedSwitch(p + "ff.", h, c["inner"], c["experts"])
         blocks.append(PreNormBlock(RMSNorm(p + "norm1.", h, c["rms_norm_eps"]), attn,
-                                   RMSNorm(p + "norm2.", h, c["rms_norm_eps"]),
-                                   BiasedSwitch(p + "ff.", h, c["inner"], c["experts"])))
+                                   RMSNorm(p + "norm2.", h, c["rms_norm_eps"]), ff))
     return ModelSpec(TokenEmbedding("embed.", c["vocab_size"], h), blocks,
                      RMSNorm("norm.", h, c["rms_norm_eps"]), LMHead("head.", c["vocab_size"], h))
 
@@ -196,6 +222,9 @@ def register_routed() -> None:
 TOY_ROUTED_CONFIG = {"architectures": ["ToyRoutedForCausalLM"], "vocab_size": 83, "hidden_size": 48,
                      "num_hidden_layers": 2, "heads": 3, "kv_heads": 1, "head_dim": 16, "rot_dim": 8,
                      "slope": 0.7, "window": 11, "inner": 24, "experts": 5, "rms_norm_eps": 1e-5}
+
+
+TOY_SCORED_CONFIG = dict(TOY_ROUTED_CONFIG, router="scored", top_k=2, route_scale=1.75, experts=6)
 
 
 def plain_forward_routed(w: Dict[str, torch.Tensor], c: dict, tokens: List[int]) -> torch.Tensor:
@@ -228,9 +257,23 @@ def plain_forward_routed(w: Dict[str, torch.Tensor], c: dict, tokens: List[int])
         o = pm.attention_core(q, k, v, pos, pos, c["window"]).reshape(t, hq * d)
         x = x + o @ w[p + "attn.o_proj.weight"].float().T
         m = pm.rms_norm(x, w[p + "norm2.weight"], c["rms_norm_eps"])
+        y = torch.zeros_like(m)
+        if c.get("router") == "scored":
+            score = torch.sigmoid(m @ w[p + "ff.router.weight"].float().T)
+            biased = score + w[p + "ff.router.choice_bias"].float()
+            for r in range(t):
+                # the k largest biased scores (a stable sort: ties to the lower index) choose;
+                # the weights are the plain scores of the chosen, renormalised and scaled
+                chosen = torch.sort(biased[r], descending=True, stable=True).indices[:c["top_k"]]
+                wt = score[r, chosen] / score[r, chosen].sum() * c["route_scale"]
+                for e, we in zip(chosen.tolist(), wt.tolist()):
+                    pe = f"{p}ff.experts.{e}."
+                    y[r] += we * pm.swiglu_mlp(m[r:r + 1], w[pe + "gate_proj.weight"],
+                                               w[pe + "up_proj.weight"], w[pe + "down_proj.weight"])[0]
+            x = x + y
+            continue
         logits = m @ w[p + "ff.router.weight"].float().T + w[p + "ff.router.bias"].float()
         prob = torch.softmax(logits, dim=-1)
-        y = torch.zeros_like(m)
         for r in range(t):
             e = int(torch.argmax(prob[r]))        # the first maximum: ties to the lower index
             pe = f"{p}ff.experts.{e}."
