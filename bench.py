@@ -10,7 +10,7 @@ keys and values; token ids are seeded random). A step is one decode step: one
 new token for every request of the batch through the engine's step function
 (replayed from a captured HIP graph unless --no-graph) and its device sampler. One JSON line is printed: decoded tokens a second as
 `value`; the 2,048-token prefill under "prefill"; the decode step's memory
-roofline under "roofline" (with the rate of a plain device copy measured beside it, and the
+roofline under "roofline" (with the rate of a plain read of HBM measured beside it, and the
 step's fraction of that); decode at batch 1 and 64 under "points"; and under
 "graph_check" the largest difference between replayed and eager decode steps at
 those batches (untimed; 0.0 when the replays are exact).
@@ -72,8 +72,9 @@ def main() -> int:
                     help="layer sizes: a2.7b (the default and the headline) or 57b-a14b")
     ap.add_argument("--profile", action="store_true",
                     help="also time every kind of kernel call of one eager decode step and one "
-                         "prefill with device events (untimed runs of their own; the table goes "
-                         "to stderr and under \"profile\")")
+                         "prefill with device events, with the bytes and flops of each kind, its "
+                         "floor and the fraction of it reached (untimed runs of their own; the "
+                         "table goes to stderr and under \"profile\")")
     ap.add_argument("--scenario", default="decode", choices=["decode", "long"])
     ap.add_argument("--requests", type=int, default=8, help="--scenario long: concurrent requests")
     ap.add_argument("--prompt", type=int, default=32768, help="--scenario long: prompt tokens")
@@ -199,12 +200,98 @@ def main() -> int:
         runner._graphs.clear()
         return max(float((a - b).abs().max()) for a, b in zip(*outs))
 
+    def call_cost(name, a, kw):
+        """What one call of the kernel library has to move and to compute, from its own
+        arguments: a function, evaluated after the step (it may read device tensors such as
+        the experts' offsets), that returns (bytes, flops). Bytes: every operand read once and
+        every result written once (weights of experts that got rows only; the cached keys and
+        values a request's rows can see, once per request); flops: two per multiply-add."""
+        def nbytes(*ts):
+            return sum(t.numel() * t.element_size() for t in ts if t is not None)
+
+        def product(x_rows, x, w_rows, w, out_rows, out_cols, out):
+            k_ = x.shape[1]
+            return (x_rows * k_ * x.element_size() + w_rows * k_ * w.element_size()
+                    + out_rows * out_cols * out.element_size(), 2.0 * x_rows * w_rows * k_)
+
+        def grouped(x, w, offsets, n_rows, out):
+            def cost():
+                counts = (offsets[1:] - offsets[:-1]).cpu()
+                used = int((counts > 0).sum())
+                per_expert = w.shape[1] * w.shape[2]
+                return (used * per_expert * w.element_size() + n_rows * x.shape[1] * x.element_size()
+                        + nbytes(out), 2.0 * n_rows * per_expert)
+            return cost
+
+        if name == "linear":
+            x, w, out = a[0], a[1], a[2]
+            return lambda: product(x.shape[0], x, w.shape[0], w, out.shape[0], out.shape[1], out)
+        if name == "swiglu_linear":
+            x, w, out = a[0], a[1], a[2]
+            return lambda: product(x.shape[0], x, w.shape[0], w, out.shape[0], out.shape[1], out)
+        if name == "qkv_rope":
+            x, w, qkv = a[0], a[1], a[3]
+            return lambda: product(x.shape[0], x, w.shape[0], w, qkv.shape[0], qkv.shape[1], qkv)
+        if name == "grouped_swiglu":
+            return grouped(a[0], a[1], a[2], a[3].shape[0], a[5])
+        if name == "grouped_down":
+            return grouped(a[0], a[1], a[2], a[3].shape[0], a[4])
+        if name == "paged_attention":
+            qkv, k_pool, sctx, n_q, n_kv, d, window = a[0], a[1], a[4], a[5], a[6], a[7], a[9]
+            out = kw.get("out", a[11] if len(a) > 11 else None)
+
+            def cost():
+                pos = sctx.positions.cpu().tolist()
+                seq = sctx.row_seq.cpu().tolist()
+                seen = [min(p + 1, window) if window else p + 1 for p in pos]
+                keys = {}
+                for s_, p, n_ in zip(seq, pos, seen):     # keys a request's rows see, all told
+                    lo, hi = keys.get(s_, (p - n_ + 1, p))
+                    keys[s_] = (min(lo, p - n_ + 1), max(hi, p))
+                kv = sum(hi - lo + 1 for lo, hi in keys.values()) * 2 * n_kv * d * k_pool.element_size()
+                return (kv + len(pos) * n_q * d * qkv.element_size() + nbytes(out),
+                        4.0 * n_q * d * sum(seen))
+            return cost
+        if name == "rmsnorm":
+            x, out = a[0], a[3]
+            rs = kw.get("rows_sum")
+            extra = nbytes(kw.get("delta")) + (nbytes(rs.y, rs.shared) if rs is not None else 0)
+            touched = out.shape[0] * x.shape[1] * 4
+            return lambda: (2 * touched + nbytes(out) + extra, 0.0)   # residual read and written
+        if name == "_launch_held":
+            def cost():
+                total_b = total_f = 0.0
+                for g, keep in a[0]:
+                    x, w, out, offsets = keep[0], keep[1], keep[2], keep[4]
+                    w_rows = g.N * (2 if g.epilogue else 1)
+                    if offsets is None:
+                        b_, f_ = product(g.M, x, w_rows, w, g.M, g.N, out)
+                    else:
+                        counts = (offsets[1:] - offsets[:-1]).cpu()
+                        used = int((counts > 0).sum())
+                        b_ = (used * w_rows * g.K * w.element_size() + g.M * g.K * x.element_size()
+                              + g.M * g.N * out.element_size())
+                        f_ = 2.0 * g.M * w_rows * g.K
+                    total_b += b_
+                    total_f += f_
+                return total_b, total_f
+            return cost
+        tensors = [t for t in list(a) + list(kw.values()) if isinstance(t, torch.Tensor)]
+        if name in ("embed",):      # a gather: the rows read, not the table
+            return lambda: (2 * nbytes(a[2]), 0.0)
+        if name in ("rope_kv_write",):   # q and k rotated in place, k and v written to pages
+            return lambda: (2 * nbytes(a[0]), 0.0)
+        return lambda: (nbytes(*[t for t in tensors if t.numel() < (1 << 28)]), 0.0)
+
     def profile_calls(label: str, chunks) -> dict:
-        """Microseconds by kind of kernel call for one eager step: every call of the kernel
-        library is bracketed by device events (calls inside `together()` are launched when
-        it ends and are timed there, as one kind). Everything runs on one stream here (a long
-        portion's shared expert otherwise runs beside the routed path, and times would
-        overlap). The reference prints such a table per phase (src/models/model.hip:1066-1081)."""
+        """One eager step by kind of kernel call: microseconds (every call of the kernel
+        library is bracketed by device events; calls inside `together()` are launched when it
+        ends and are timed there, as one kind), the bytes and flops the calls have to move
+        and compute (`call_cost`), their floor max(bytes / 8 TB/s, flops / peak) and the
+        fraction floor / time; the floors add up to the step's. Everything runs on one stream
+        here (a long portion's shared expert otherwise runs beside the routed path, and times
+        would overlap). The reference prints its table of times per phase
+        (src/models/model.hip:1066-1081)."""
         ops = runner.ops
         spans = []
         one_stream, ops.beside_min_rows = ops.beside_min_rows, 1 << 30
@@ -228,6 +315,7 @@ def main() -> int:
                 if (ops._held is not None and n != "_launch_held") or depth[0]:
                     return saved[n](*a, **kw)       # held back (timed when launched), or part of a call that is timed
                 s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                cost = call_cost(n, a, kw)
                 s.record()
                 depth[0] += 1
                 try:
@@ -235,7 +323,8 @@ def main() -> int:
                 finally:
                     depth[0] -= 1
                 e.record()
-                spans.append(("products launched together" if n == "_launch_held" else kind(n, a), s, e))
+                spans.append(("products launched together" if n == "_launch_held" else kind(n, a),
+                              s, e, cost))
                 return out
             return call
 
@@ -250,30 +339,45 @@ def main() -> int:
                 setattr(ops, n, saved[n])
             runner.options.use_graph = use_graph
             ops.beside_min_rows = one_stream
+        peak = FLOP_PEAK[args.dtype]
         table = {}
-        for k_, s, e in spans:
-            calls, us = table.get(k_, (0, 0.0))
-            table[k_] = (calls + 1, us + s.elapsed_time(e) * 1e3)
-        total = sum(us for _, us in table.values())
-        print(f"[bench] {label}: {total:.0f} us in kernel calls (eager, with event overhead)",
-              file=sys.stderr)
-        for k_, (calls, us) in sorted(table.items(), key=lambda kv: -kv[1][1]):
-            print(f"[bench]   {us:9.1f} us {100 * us / total:5.1f}%  {calls:4d} x {k_}", file=sys.stderr)
-        return {k_: round(us, 1) for k_, (_, us) in table.items()}
+        for k_, s, e, cost in spans:
+            b_, f_ = cost()
+            row = table.setdefault(k_, [0, 0.0, 0.0, 0.0, 0.0])
+            row[0] += 1
+            row[1] += s.elapsed_time(e) * 1e3
+            row[2] += b_
+            row[3] += f_
+            row[4] += max(b_ / HBM_PEAK, f_ / peak) * 1e6
+        total = sum(r[1] for r in table.values())
+        floor = sum(r[4] for r in table.values())
+        print(f"[bench] {label}: {total:.0f} us in kernel calls (eager, with event overhead); "
+              f"floor {floor:.0f} us = {floor / total:.3f} of it", file=sys.stderr)
+        print(f"[bench]   {'us':>9} {'%':>5} {'calls':>5} {'MB':>9} {'GFLOP':>9} {'floor us':>9} "
+              f"{'frac':>5}  kind", file=sys.stderr)
+        for k_, (calls, us, b_, f_, fl) in sorted(table.items(), key=lambda kv: -kv[1][1]):
+            print(f"[bench]   {us:9.1f} {100 * us / total:5.1f} {calls:5d} {b_ / 1e6:9.1f} "
+                  f"{f_ / 1e9:9.1f} {fl:9.1f} {fl / us:5.2f}  {k_}", file=sys.stderr)
+        out = {k_: {"us": round(us, 1), "mb": round(b_ / 1e6, 1), "gflop": round(f_ / 1e9, 1),
+                    "floor_us": round(fl, 1), "frac": round(fl / us, 3)}
+               for k_, (_, us, b_, f_, fl) in table.items()}
+        out["step"] = {"us": round(total, 1), "floor_us": round(floor, 1),
+                       "frac": round(floor / total, 3)}
+        return out
 
-    def copy_rate() -> float:
-        """Bytes a second that a plain device copy of 2 GiB moves (read + write): what the
-        memory system gives a kernel that does nothing else."""
-        src = torch.empty(1 << 29, dtype=torch.float32, device=runner.device).normal_()
-        dst = torch.empty_like(src)
+    def read_rate() -> float:
+        """Bytes a second at which a kernel that only reads streams 4 GiB from HBM (the
+        library's read probe: 16-byte non-temporal loads, nothing written): what the memory
+        system gives a decode step's weights and cache at best."""
+        src = torch.empty(1 << 30, dtype=torch.float32, device=runner.device).normal_()
         for _ in range(2):
-            dst.copy_(src)
+            runner.ops.read_probe(src)
         torch.cuda.synchronize()
         t = time.perf_counter()
         for _ in range(5):
-            dst.copy_(src)
+            runner.ops.read_probe(src)
         torch.cuda.synchronize()
-        return 5 * 2 * src.numel() * 4 / (time.perf_counter() - t)
+        return 5 * src.numel() * 4 / (time.perf_counter() - t)
 
     dt, nbytes, n_exp = decode_run(args.batch, args.steps, args.warmup)
     result = {
@@ -293,9 +397,9 @@ def main() -> int:
                      "frac": round(nbytes / dt / HBM_PEAK, 4),
                      "distinct_experts_per_layer": round(n_exp, 1)},
     }
-    copied = copy_rate()
-    result["roofline"]["measured_copy"] = round(copied / 1e9, 1)
-    result["roofline"]["frac_of_copy"] = round(nbytes / dt / copied, 4)
+    plain_read = read_rate()
+    result["roofline"]["measured_read"] = round(plain_read / 1e9, 1)
+    result["roofline"]["frac_of_read"] = round(nbytes / dt / plain_read, 4)
     if not args.no_prefill:
         pt = min(args.prefill_tokens, ctx)
         pdt, flops = prefill_run(pt, 3)

@@ -105,6 +105,9 @@ def main(argv: Optional[List[str]] = None) -> int:
         if args.verify:
             eng.close()   # the golden engine takes the first one's place: never both at once
             del eng
+            import torch
+            log(f"verify: the first engine is closed, {torch.cuda.memory_allocated() >> 20} MiB "
+                f"of device memory still held")
             _verify(args, raw, common, prompts, params, stop, outs)
     except Exception as e:  # the reference exits 1 with the message (src/apps/ninfer.cpp:234-237)
         print(f"ninfer: error: {e}", file=sys.stderr)

@@ -37,6 +37,19 @@ class EngineOptions:
             raise ValueError(f"kv_bytes must be >= 1, got {self.kv_bytes}")
         if self.kv_bytes is not None and self.num_pages is not None:
             raise ValueError("give num_pages or kv_bytes, not both")
+        if self.dtype == "bfloat16" and not self.page_size_suits_fast_attention():
+            import warnings
+            warnings.warn(
+                f"page_size {self.page_size}: the matrix-core attention kernels take pages of "
+                f"1, 2, 4, ... 64 tokens; with this size every bfloat16 step runs the plain "
+                f"attention kernel (one wave per row and head), which is right and many times "
+                f"slower", stacklevel=2)
+
+    def page_size_suits_fast_attention(self) -> bool:
+        """The bfloat16 prompt kernel walks keys in tiles of 64 that whole pages must fill,
+        and both fast kernels find a key's page by a shift: a power of two up to 64."""
+        ps = self.page_size
+        return ps >= 1 and ps & (ps - 1) == 0 and ps <= 64
 
     def pages_per_request(self) -> int:
         return -(-self.max_context // self.page_size)

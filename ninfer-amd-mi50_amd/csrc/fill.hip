@@ -61,9 +61,45 @@ __global__ void fill_nan_pages_kernel(T* __restrict__ pool, const int* __restric
     dst[i] = nan;
 }
 
+// A kernel that only reads: every block walks its share of the buffer with 16-byte
+// non-temporal loads, four on their way per lane, and writes nothing unless the words add
+// up to a value they never add up to (which keeps the loads). What it reaches is the rate at
+// which this part streams memory that is read once: the measure a decode step's weights
+// and cache are held against.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void read_probe_kernel(const u32x4* __restrict__ p, int64_t n_vec,
+                                                         unsigned* __restrict__ sink) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  unsigned acc = 0;
+  for (; i + 3 * stride < n_vec; i += 4 * stride) {
+    const u32x4 a = __builtin_nontemporal_load(p + i), b = __builtin_nontemporal_load(p + i + stride),
+                c = __builtin_nontemporal_load(p + i + 2 * stride),
+                d = __builtin_nontemporal_load(p + i + 3 * stride);
+    acc += (a.x ^ a.y ^ a.z ^ a.w) + (b.x ^ b.y ^ b.z ^ b.w) + (c.x ^ c.y ^ c.z ^ c.w) +
+           (d.x ^ d.y ^ d.z ^ d.w);
+  }
+  for (; i < n_vec; i += stride) {
+    const u32x4 a = __builtin_nontemporal_load(p + i);
+    acc += a.x ^ a.y ^ a.z ^ a.w;
+  }
+  if (acc == 0x9e3779b9u && sink) *sink = acc;
+}
+
 }  // namespace ninfer
 
 using namespace ninfer;
+
+// Reads `bytes` bytes from `p` (16-byte aligned; a tail of fewer than 16 bytes is not read)
+// and writes nothing: for measuring the rate of a plain read.
+extern "C" int ninfer_read_probe(const void* p, long long bytes, hipStream_t stream) {
+  NINFER_REQUIRE(p && bytes >= 16 && ((uintptr_t)p & 15) == 0, "read_probe: %lld bytes at %p", bytes, p);
+  const int blocks = 8 * device_cu_count();
+  read_probe_kernel<<<blocks, 256, 0, stream>>>((const u32x4*)p, bytes / 16, nullptr);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
 
 extern "C" int ninfer_fill_random(void* out, long long n, unsigned long long key, float std,
                                   float mean, int dtype, hipStream_t stream) {

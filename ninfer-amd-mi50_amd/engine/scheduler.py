@@ -129,14 +129,15 @@ class Scheduler:
 
     def _fits_alone(self, total: int) -> bool:
         """Could a request of `total` tokens run with every page to itself? A group that
-        keeps all keys must hold them all; a windowed group never holds more than the window
-        and the portion of one step (pages the window has passed are given back after every
-        step), plus the two pages that the ends of that span may share with their neighbours."""
+        keeps all keys must hold them all; a windowed group never holds more than the span a
+        step of n tokens touches, the window - 1 keys before its first row and its n rows
+        (pages the window has passed are given back after every step): window + n - 1
+        positions, which lie in at most ceil(that / page) + 1 pages wherever they start."""
         ps = self.cache.page_size
         for g in self.cache.groups:
             most = -(-total // ps)
             if g.window is not None:
-                most = min(most, -(-(g.window + self.max_batch_tokens) // ps) + 2)
+                most = min(most, -(-(g.window + self.max_batch_tokens - 1) // ps) + 1)
             if most > g.allocator.num_pages:
                 return False
         return True

@@ -253,6 +253,14 @@ class HipOps:
             ctypes.c_ulonglong(key & ((1 << 64) - 1)), ctypes.c_float(std), ctypes.c_float(mean),
             _DT[out.dtype], self._stream()))
 
+    def read_probe(self, t):
+        """Streams the tensor's bytes through a kernel that only reads (measurements: the rate
+        of a plain read of HBM)."""
+        _dev(t, "t")
+        self._ok(self.lib.ninfer_read_probe(ctypes.c_void_p(t.data_ptr()),
+                                            ctypes.c_longlong(t.numel() * t.element_size()),
+                                            self._stream()))
+
     # ---- row-wise ---------------------------------------------------------------
     def embed(self, tokens, table, out):
         _dev(tokens, "tokens", torch.int32, 1)

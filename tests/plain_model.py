@@ -173,14 +173,16 @@ def routed_experts(x: Tensor, ids: Tensor, wts: Tensor, w: Dict[str, Tensor],
     Reference: src/models/model.hip:352-433 (gather, per-expert MLP, scale,
     scatter-add); summed here in 32-bit in the order of `ids`.
     """
+    t, k = ids.shape
+    per = torch.zeros(t, k, x.shape[1], dtype=x.dtype)      # expert output for choice j of row t
+    for e in torch.unique(ids).tolist():
+        rows, choice = torch.nonzero(ids == e, as_tuple=True)
+        p = f"{prefix}experts.{e}."
+        per[rows, choice] = swiglu_mlp(x[rows], w[p + "gate_proj.weight"], w[p + "up_proj.weight"],
+                                       w[p + "down_proj.weight"])
     y = torch.zeros_like(x)
-    for t in range(x.shape[0]):
-        for j in range(ids.shape[1]):
-            e = int(ids[t, j])
-            p = f"{prefix}experts.{e}."
-            y[t] += wts[t, j] * swiglu_mlp(x[t:t + 1], w[p + "gate_proj.weight"],
-                                           w[p + "up_proj.weight"],
-                                           w[p + "down_proj.weight"])[0]
+    for j in range(k):                                      # summed in the order of `ids`
+        y += wts[:, j:j + 1] * per[:, j]
     return y
 
 

@@ -475,6 +475,60 @@ def test_one_layer_at_real_sizes_against_the_plain_model(model, dtype):
     assert runner.cache.pages_reused() > 0
 
 
+@pytest.mark.parametrize("model,dtype", [("a2.7b", "float32"), ("a2.7b", "bfloat16"),
+                                         ("57b-a14b", "bfloat16")])
+def test_two_layers_at_real_sizes_against_the_plain_model(model, dtype):
+    """Two layers at the benchmark models' layer sizes against the plain model on the weights
+    the engine holds: a prompt of 312 tokens fed as 256 + 56 (the 256-row grouped tiles at
+    K = 2048 / 1408 and 3584 / 2560, the library's dense products, the expert sum of one layer
+    added by the next layer's norm at real width), then 8 tokens decoded at batch 8 from a
+    replayed graph beside seven short requests. In bfloat16 a row is compared when its routing
+    is clear of rounding noise in both layers; the bound on such rows is the file's, its
+    absolute part scaled by the size of the logits (the file's bound was made for logits of
+    standard deviation 0.9)."""
+    from bench import MODELS
+    from ninfer_amd import Chunk, EngineOptions, random_model
+    raw = dict(MODELS[model][1], num_hidden_layers=2, vocab_size=2048)
+    runner = random_model(raw, 31, EngineOptions(dtype=dtype, max_context=384, prefill_chunk=256,
+                                                 num_sequences=8, page_size=16, use_graph=True,
+                                                 check_pages=True))
+    w = {n: runner.tensor(n).float().cpu() for n in runner.tensor_names()}
+    reqs = [util.random_tokens(320, 2048, 5)] + \
+        [util.random_tokens(12 + i, 2048, 50 + i) for i in range(7)]
+    refs = [plain_model.forward(w, raw, t) for t in reqs]
+    need = 1e-3 if dtype == "float32" else 0.04
+    clear = [util.routing_margins(w, raw, t) > need for t in reqs]
+    tol = bound(dtype)
+    spread = float(refs[0].std())
+    assert spread > 0.5, "logits of size 1"
+    tol["atol"] *= max(1.0, spread / 0.9)
+    slots = [runner.open() for _ in reqs]
+    a = runner.step([Chunk(slots[0], reqs[0][:256], list(range(256)))]).float().cpu()
+    b = runner.step([Chunk(slots[0], reqs[0][256:312], list(range(56)))]).float().cpu()
+    got = torch.cat([a, b])
+    keep = clear[0][:312]
+    assert int(keep.sum()) >= (250 if dtype == "float32" else 10), f"{int(keep.sum())} clear rows"
+    torch.testing.assert_close(got[keep], refs[0][:312][keep], **tol,
+                               msg=lambda m: f"{model} {dtype} prompt: {m}")
+    if dtype == "bfloat16":   # rows that may route otherwise are still near: no kernel is off by much
+        err = (got - refs[0][:312]).abs().amax(dim=1)
+        assert float(err.median()) < tol["atol"] and float(err.max()) < 0.2 * float(refs[0].abs().max())
+    for s, t in zip(slots[1:], reqs[1:]):
+        runner.step([Chunk(s, t[:-8], [])])
+    first = [312] + [len(t) - 8 for t in reqs[1:]]
+    compared = 0
+    for i in range(8):
+        logits = runner.step([Chunk(s, [t[f + i]], [0]) for s, t, f in zip(slots, reqs, first)])
+        logits = logits.float().cpu()
+        for j, (t, f) in enumerate(zip(reqs, first)):
+            if clear[j][f + i]:
+                compared += 1
+                torch.testing.assert_close(logits[j], refs[j][f + i], **tol,
+                                           msg=lambda m: f"{model} {dtype} decode {j} at {f + i}: {m}")
+    assert compared >= (56 if dtype == "float32" else 4)
+    assert any(e["graph"] is not None for e in runner._graphs.values())
+
+
 @pytest.mark.parametrize("seed", list(range(24)))
 def test_random_configurations(tmp_path, seed):
     """Configurations drawn at random (head sizes that only the plain kernels take, heads in

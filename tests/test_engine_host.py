@@ -269,6 +269,22 @@ def test_cache_sized_in_bytes(model_dirs):
                    EngineOptions(dtype="float32", kv_bytes=100, device="cpu"), ops=PlainOps())
 
 
+def test_a_page_size_the_fast_attention_kernels_do_not_take_is_said(recwarn):
+    """bfloat16 with pages that are no power of two, or of more than 64 tokens, runs on the plain
+    attention kernel: right and slow, and the options say so; 32-bit runs it anyway."""
+    import warnings
+    from ninfer_amd import EngineOptions
+    for ps in (1, 4, 16, 64):
+        EngineOptions(dtype="bfloat16", page_size=ps).validate()
+    EngineOptions(dtype="float32", page_size=48).validate()
+    assert not [w for w in recwarn.list if "page_size" in str(w.message)]
+    for ps in (48, 128, 24):
+        with pytest.warns(UserWarning, match=f"page_size {ps}.*plain attention kernel"):
+            EngineOptions(dtype="bfloat16", page_size=ps).validate()
+    with pytest.raises(ValueError, match="max_graphs"):
+        EngineOptions(max_graphs=0).validate()
+
+
 def test_weights_can_be_read_back_by_name(model_dirs):
     """What the engine holds under a checkpoint name, fused and stacked tensors included,
     is what the folder holds."""

@@ -240,11 +240,22 @@ def test_a_windowed_group_admits_what_its_window_can_serve(model_dirs):
     assert req.status == "finished", req.error
     assert req.output == plain_model.greedy_generate(w, raw, req.prompt, 8)
     assert runner.cache.groups[0].window_freed > 0
-    # a pool smaller than the window and a portion still refuses it at admission
-    opt.num_pages = 5
+    # The boundary: a step of 16 tokens touches the 7 keys before its first row and its own 16
+    # positions, 23 in all, which lie in at most ceil(23 / 4) + 1 = 7 pages. With exactly 7
+    # the request runs (every step's tables checked); with 6 it is refused at admission.
+    opt.num_pages = 7
     runner = load_model(d, opt, ops=PlainOps())
     sched = Scheduler(runner, Sampler(PlainOps(), runner.device))
-    req2 = Request("long", list(req.prompt), SamplingParams.greedy(8))
-    sched.add(req2)
+    req3 = Request("long", list(req.prompt), SamplingParams.greedy(8))
+    sched.add(req3)
     sched.run()
-    assert req2.status == "failed" and "fit" in req2.error
+    assert req3.status == "finished", req3.error
+    assert req3.output == req.output and req3.preemptions == 0
+    for pages in (6, 5):
+        opt.num_pages = pages
+        runner = load_model(d, opt, ops=PlainOps())
+        sched = Scheduler(runner, Sampler(PlainOps(), runner.device))
+        req2 = Request("long", list(req.prompt), SamplingParams.greedy(8))
+        sched.add(req2)
+        sched.run()
+        assert req2.status == "failed" and "fit" in req2.error
