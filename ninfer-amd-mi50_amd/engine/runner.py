@@ -110,7 +110,7 @@ class ModelRunner:
         self._graphs.clear()
         if self._holds_graphs:
             self._holds_graphs = False
-            self.ops.graph_holder_gone()
+            self.ops.graph_holder_gone(self)
         self._staging = []
         self._held = {}
         self.cache.drop_pools()
@@ -313,7 +313,7 @@ class ModelRunner:
             entry["graph"] = g
             if not self._holds_graphs:
                 self._holds_graphs = True
-                self.ops.graph_holder_new()
+                self.ops.graph_holder_new(self)
         entry["graph"].replay()
         return entry["logits"]
 

@@ -8,6 +8,7 @@ loaded, `load_ops` raises.
 from __future__ import annotations
 
 import ctypes
+import weakref
 from typing import Optional
 
 import torch
@@ -190,17 +191,19 @@ class HipOps:
         # what tests and measurements ask of the product kernels (see `tuned`); all 0: the
         # library chooses
         self._tune = {"force_kernel": 0, "split_min_bytes": 0, "skinny_two": 0}
-        self._graph_holders = 0  # runners whose captured graphs may hold workspace addresses
+        # runners whose captured graphs may hold workspace addresses (held weakly: a runner
+        # that is simply dropped leaves the set by itself)
+        self._graph_holders = weakref.WeakSet()
 
-    def graph_holder_new(self) -> None:
-        self._graph_holders += 1
+    def graph_holder_new(self, runner) -> None:
+        self._graph_holders.add(runner)
 
-    def graph_holder_gone(self) -> None:
-        """A runner with captured graphs has dropped them. When it was the last, nothing can
+    def graph_holder_gone(self, runner) -> None:
+        """A runner with captured graphs has dropped them. When no other is left, nothing can
         replay into the workspaces any more: they are given back (the next call that needs
         one makes it anew)."""
-        self._graph_holders = max(0, self._graph_holders - 1)
-        if self._graph_holders == 0:
+        self._graph_holders.discard(runner)
+        if len(self._graph_holders) == 0:
             self._outgrown = []
             self._attn_ws = None
             self._split_ws = None
@@ -712,7 +715,8 @@ class HipOps:
                 if self._attn_ws is not None:
                     self._outgrown.append(self._attn_ws)
                     ws_floats = max(ws_floats, 2 * self._attn_ws.numel())
-                self._attn_ws = torch.empty(ws_floats, dtype=torch.float32, device=qkv.device)
+                # zeros: the workspace begins with counters that the kernels find and leave at zero
+                self._attn_ws = torch.zeros(ws_floats, dtype=torch.float32, device=qkv.device)
             ws_floats = self._attn_ws.numel()
             ws = self._attn_ws.data_ptr()
         args = _AttnArgs(

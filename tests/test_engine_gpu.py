@@ -516,16 +516,20 @@ def test_two_layers_at_real_sizes_against_the_plain_model(model, dtype):
     for s, t in zip(slots[1:], reqs[1:]):
         runner.step([Chunk(s, t[:-8], [])])
     first = [312] + [len(t) - 8 for t in reqs[1:]]
-    compared = 0
+    compared, errs = 0, []
     for i in range(8):
         logits = runner.step([Chunk(s, [t[f + i]], [0]) for s, t, f in zip(slots, reqs, first)])
         logits = logits.float().cpu()
         for j, (t, f) in enumerate(zip(reqs, first)):
+            errs.append(float((logits[j] - refs[j][f + i]).abs().max()))
             if clear[j][f + i]:
                 compared += 1
                 torch.testing.assert_close(logits[j], refs[j][f + i], **tol,
                                            msg=lambda m: f"{model} {dtype} decode {j} at {f + i}: {m}")
-    assert compared >= (56 if dtype == "float32" else 4)
+    # (with 64 experts top-8 in two layers hardly a row's routing is clear in bfloat16: the
+    # decoded rows are then held to the typical error, as the prompt's rows above)
+    assert compared >= (56 if dtype == "float32" else 1)
+    assert sorted(errs)[len(errs) // 2] < tol["atol"]
     assert any(e["graph"] is not None for e in runner._graphs.values())
 
 

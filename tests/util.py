@@ -35,7 +35,7 @@ def routing_margins(w, cfg, tokens) -> torch.Tensor:
     import plain_model
     probe: dict = {}
     plain_model.forward(w, cfg, tokens, probe=probe)
-    k = cfg["num_experts_per_tok"]
+    k = cfg.get("num_experts_per_tok", 0)   # (a model without experts has no routing to tie)
     worst = torch.full((len(tokens),), float("inf"))
     for logits in probe.get("router_logits", {}).values():
         if logits.shape[1] <= k:
