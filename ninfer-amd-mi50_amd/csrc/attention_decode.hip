@@ -14,9 +14,7 @@
 // heads that share the kv head, so keys and values are read once for all of
 // them. Lane groups, then waves, are merged by the usual log-sum-exp rule and
 // the chunk's (m, l, acc) goes to the workspace.
-// Pass 2 merges the chunks of a row in a fixed order. In the scalar kernel it is the work of
-// the block that finishes a (row, kv head)'s last chunk (see `finish_row`): no second launch.
-// Otherwise it is a kernel of its own, grid (rows, query heads).
+// Pass 2, grid (rows, query heads): merges the chunks of a row in a fixed order.
 // With three or more query heads per kv head (and heads of 64 or 128), pass 1 is the
 // matrix-core kernel of attention_prefill.hip with the heads of a kv head as its rows;
 // it writes the same (m, l, acc) per chunk, and pass 2 is the same.
@@ -43,97 +41,8 @@ __device__ __forceinline__ void cvt8(const bf16x8& v, float* f) {
   for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
 }
 
-// Values that blocks hand to one another inside a launch. The L2 caches of the chip's XCDs
-// do not see each other's lines, so such values are written and read with device-scope
-// atomic operations (relaxed: plain stores and loads that go past the caches; no fence,
-// which would write back and invalidate a whole L2 per block).
-__device__ __forceinline__ void put_shared(float* p, float v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float get_shared(const float* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// The merge of a row's chunks (pass 2) by the block that finishes last among the blocks of
-// one (row, group of query heads): every block, once its partial results are written (with
-// `put_shared`, and waited for), draws a ticket from the group's counter; the one that draws
-// the last ticket finds every other block's results written, merges them as the merge
-// kernel does, and puts the counter back to zero for the next launch. Nobody waits for
-// anybody. `lds`: 2 x chunks + blockDim.x floats. Called by every thread of a block of
-// kDecWaves waves.
-//   out[t, h, :] = sum_c acc_c exp(m_c - M) / sum_c l_c exp(m_c - M), chunks in order.
-template <int D>
-__device__ __forceinline__ void finish_row(const AttnArgs& a, int* counter, int t, int h0,
-                                           int n_heads, int n_chunks, int c_lo, int c_hi,
-                                           float* lds) {
-  constexpr int NT = kDecWaves * 64;
-  __shared__ int last;
-  __shared__ float red[2 * kDecWaves];
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this thread's partial results have arrived
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const int ticket = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    last = ticket == c_hi - c_lo;
-    if (last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  __syncthreads();
-  if (!last) return;
-  const int tid = threadIdx.x, live = c_hi - c_lo + 1;
-  float* scale_s = lds;
-  float* l_s = lds + live;
-  float* part_s = lds + 2 * live;
-  for (int i = 0; i < n_heads; ++i) {
-    const float* ws = a.workspace + (((int64_t)t * a.Hq + h0 + i) * n_chunks + c_lo) * (D + 2);
-    float mx = -1e30f;
-    for (int c = tid; c < live; c += NT) {
-      const float m = get_shared(ws + c * (D + 2) + D), l = get_shared(ws + c * (D + 2) + D + 1);
-      scale_s[c] = m;
-      l_s[c] = l;
-      mx = fmaxf(mx, m);
-    }
-    mx = wave_max(mx);
-    if ((tid & 63) == 0) red[tid >> 6] = mx;
-    __syncthreads();
-    float M = red[0];
-#pragma unroll
-    for (int w = 1; w < kDecWaves; ++w) M = fmaxf(M, red[w]);
-    float lsum = 0.f;
-    for (int c = tid; c < live; c += NT) {
-      const float sc = __expf(scale_s[c] - M);
-      scale_s[c] = sc;
-      lsum += l_s[c] * sc;
-    }
-    lsum = wave_sum(lsum);
-    if ((tid & 63) == 0) red[kDecWaves + (tid >> 6)] = lsum;
-    __syncthreads();
-    float total = 0.f;
-#pragma unroll
-    for (int w = 0; w < kDecWaves; ++w) total += red[kDecWaves + w];
-    // thread (d, part) sums the chunks c = part mod parts of dim d, all loads in flight at
-    // once; the parts are added in part order
-    constexpr int PARTS = NT / D >= 1 ? NT / D : 1;
-    static_assert(D <= NT, "one thread per dim at least");
-    const int d = tid % D, part = tid / D;
-    float acc = 0.f;
-#pragma unroll 8
-    for (int c = part; c < live; c += PARTS) acc = fmaf(get_shared(ws + c * (D + 2) + d), scale_s[c], acc);
-    part_s[tid] = acc;
-    __syncthreads();
-    if (tid < D) {
-      float sum = 0.f;
-#pragma unroll
-      for (int p = 0; p < PARTS; ++p) sum += part_s[p * D + tid];
-      ((bf16*)a.out)[((int64_t)t * a.Hq + h0 + i) * D + tid] = __float2bfloat16(sum / total);
-    }
-    __syncthreads();   // the next head reuses scale_s, l_s, part_s and red
-  }
-}
-
-// FINISH: the last block of a (row, group of heads) merges the row's chunks itself
-// (`counters`: one int per (row, blockIdx.x), zero between launches).
-template <int LPK, int GQ, int kChunk, bool FINISH>
-__global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a, int head_groups,
-                                                                     int* counters) {
+template <int LPK, int GQ, int kChunk>
+__global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a, int head_groups) {
   constexpr int D = 8 * LPK;
   constexpr int KPI = 64 / LPK;             // keys per wave instruction
   constexpr int KEYS_PER_WAVE = kChunk / kDecWaves;
@@ -279,24 +188,11 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
       aa += merge[w][i][d] * sc;
     }
     float* ws = a.workspace + (((int64_t)t * a.Hq + h0 + i) * n_chunks + chunk_id) * (D + 2);
-    if (FINISH) {
-      put_shared(ws + d, aa);
-      if (d == 0) {
-        put_shared(ws + D, mm);
-        put_shared(ws + D + 1, ll);
-      }
-    } else {
-      ws[d] = aa;
-      if (d == 0) {
-        ws[D] = mm;
-        ws[D + 1] = ll;
-      }
+    ws[d] = aa;
+    if (d == 0) {
+      ws[D] = mm;
+      ws[D + 1] = ll;
     }
-  }
-  if (FINISH) {
-    extern __shared__ float finish_lds[];
-    finish_row<D>(a, counters + (int64_t)t * gridDim.x + blockIdx.x, t, h0, n_heads, n_chunks,
-                  lo / kChunk, pos / kChunk, finish_lds);
   }
 }
 
@@ -360,15 +256,9 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_merge_kernel(AttnAr
   }
 }
 
-// The workspace begins with the tickets' counters (ints, zero between launches: whoever
-// makes a workspace clears it once, every launch leaves them zero), always at the same
-// place, so that a later call of another shape never finds partial results where it expects
-// zeros; the partial results follow.
-constexpr int kCounterInts = 16384;
-
 int64_t attention_decode_workspace_floats(int T, int Hq, int D, int max_kv_len) {
   int n_chunks = (max_kv_len + 127) / 128;   // the smaller chunk size bounds the need
-  return kCounterInts + (int64_t)T * Hq * n_chunks * (D + 2);
+  return (int64_t)T * Hq * n_chunks * (D + 2);
 }
 
 bool attention_decode_takes(const AttnArgs& a) {
@@ -378,40 +268,26 @@ bool attention_decode_takes(const AttnArgs& a) {
   return a.dtype == kBF16 && d_ok && ps_ok && a.q_stride % 8 == 0 && a.workspace != nullptr;
 }
 
-// counters != null: the kernel's last blocks merge the chunks (FINISH); else the caller
-// launches the merge kernel.
 template <int LPK, int CHUNK>
-static void launch_decode(const AttnArgs& a, int n_chunks, int* counters, hipStream_t stream) {
+static void launch_decode(const AttnArgs& a, int n_chunks, hipStream_t stream) {
   int group = a.Hq / a.Hkv;
   dim3 block(kDecWaves * 64);
-  const size_t lds = counters ? (2 * (size_t)n_chunks + kDecWaves * 64) * sizeof(float) : 0;
-#define NINFER_DECODE(GQ, HG)                                                                    \
-  do {                                                                                           \
-    if (counters)                                                                                \
-      attn_decode_kernel<LPK, GQ, CHUNK, true><<<dim3(a.Hkv * (HG), n_chunks, a.T), block, lds, stream>>>( \
-          a, HG, counters);                                                                      \
-    else                                                                                         \
-      attn_decode_kernel<LPK, GQ, CHUNK, false><<<dim3(a.Hkv * (HG), n_chunks, a.T), block, 0, stream>>>( \
-          a, HG, nullptr);                                                                       \
-  } while (0)
   if (group == 1) {
-    NINFER_DECODE(1, 1);
+    attn_decode_kernel<LPK, 1, CHUNK><<<dim3(a.Hkv, n_chunks, a.T), block, 0, stream>>>(a, 1);
   } else if (group == 2) {
-    NINFER_DECODE(2, 1);
+    attn_decode_kernel<LPK, 2, CHUNK><<<dim3(a.Hkv, n_chunks, a.T), block, 0, stream>>>(a, 1);
   } else {
-    const int hg = (group + 3) / 4;
-    NINFER_DECODE(4, hg);
+    int hg = (group + 3) / 4;
+    attn_decode_kernel<LPK, 4, CHUNK><<<dim3(a.Hkv * hg, n_chunks, a.T), block, 0, stream>>>(a, hg);
   }
-#undef NINFER_DECODE
 }
 
 template <int LPK>
-static void launch_decode_chunk(const AttnArgs& a, int chunk, int n_chunks, int* counters,
-                                hipStream_t stream) {
+static void launch_decode_chunk(const AttnArgs& a, int chunk, int n_chunks, hipStream_t stream) {
   if (chunk == 128)
-    launch_decode<LPK, 128>(a, n_chunks, counters, stream);
+    launch_decode<LPK, 128>(a, n_chunks, stream);
   else
-    launch_decode<LPK, 256>(a, n_chunks, counters, stream);
+    launch_decode<LPK, 256>(a, n_chunks, stream);
 }
 
 // Which pass-1 kernel a decode step runs and how it cuts the contexts: the matrix-core
@@ -432,37 +308,27 @@ void attention_decode_plan(const AttnArgs& a, bool* heads, int* chunk, int* n_ch
   *n_chunks = (a.max_kv_len + *chunk - 1) / *chunk;
 }
 
-int attention_decode(const AttnArgs& args, hipStream_t stream) {
+int attention_decode(const AttnArgs& a, hipStream_t stream) {
   bool heads;
   int chunk, n_chunks;
-  attention_decode_plan(args, &heads, &chunk, &n_chunks);
-  NINFER_REQUIRE(args.workspace_floats >= attention_decode_workspace_floats(args.T, args.Hq, args.D, args.max_kv_len),
-                 "paged_attention: workspace of %lld floats is too small", (long long)args.workspace_floats);
+  attention_decode_plan(a, &heads, &chunk, &n_chunks);
+  NINFER_REQUIRE(a.workspace_floats >= attention_decode_workspace_floats(a.T, a.Hq, a.D, a.max_kv_len),
+                 "paged_attention: workspace of %lld floats is too small", (long long)a.workspace_floats);
   const size_t merge_lds = (2 * (size_t)n_chunks + kMergeThreads) * sizeof(float);
   NINFER_REQUIRE(merge_lds <= 48 * 1024, "paged_attention: a context of %d keys has too many chunks to merge",
-                 args.max_kv_len);
-  AttnArgs a = args;   // the kernels see the partial results' part of the workspace
-  int* counters = (int*)args.workspace;
-  a.workspace = args.workspace + kCounterInts;
-  a.workspace_floats = args.workspace_floats - kCounterInts;
+                 a.max_kv_len);
   if (heads) {
     // three or more query heads per kv head: their products go to the matrix cores
     if (int rc = attention_decode_heads(a, chunk, n_chunks, stream)) return rc;
   } else {
-    // the scalar kernel's last blocks merge, where every (row, group of heads) has a counter
-    const int group = a.Hq / a.Hkv, hg = group <= 2 ? 1 : (group + 3) / 4;
-    const bool finish = (int64_t)a.T * a.Hkv * hg <= kCounterInts;
-    int* cnt = finish ? counters : nullptr;
     switch (a.D) {
-      case 16: launch_decode_chunk<2>(a, chunk, n_chunks, cnt, stream); break;
-      case 32: launch_decode_chunk<4>(a, chunk, n_chunks, cnt, stream); break;
-      case 64: launch_decode_chunk<8>(a, chunk, n_chunks, cnt, stream); break;
-      case 128: launch_decode_chunk<16>(a, chunk, n_chunks, cnt, stream); break;
-      case 256: launch_decode_chunk<32>(a, chunk, n_chunks, cnt, stream); break;
+      case 16: launch_decode_chunk<2>(a, chunk, n_chunks, stream); break;
+      case 32: launch_decode_chunk<4>(a, chunk, n_chunks, stream); break;
+      case 64: launch_decode_chunk<8>(a, chunk, n_chunks, stream); break;
+      case 128: launch_decode_chunk<16>(a, chunk, n_chunks, stream); break;
+      case 256: launch_decode_chunk<32>(a, chunk, n_chunks, stream); break;
       default: return set_error(-1, "paged_attention: decode kernel does not take head size %d", a.D);
     }
-    NINFER_LAUNCH_CHECK();
-    if (finish) return 0;
   }
   NINFER_LAUNCH_CHECK();
   attn_decode_merge_kernel<<<dim3(a.T, a.Hq), kMergeThreads, merge_lds, stream>>>(a, n_chunks, chunk);

@@ -25,10 +25,8 @@
 //    outside any graph capture: the first lookup of the array's address on a device may
 //    load the library's code object there;
 //  - the workspace and workspace_floats fields of the arguments are ignored;
-//  - the array's first 64 KB are counters that every call finds at zero and leaves at zero
-//    (a device array starts zeroed; a call that runs to its end puts back what it counted);
-//    of the rest nothing has to start at zero: pass 1 writes every entry that the merge
-//    reads, so the last call's contents do not matter;
+//  - nothing in the array has to start at zero: pass 1 writes every entry that
+//    the merge reads, so the last call's contents do not matter;
 //  - every call on a GPU shares that GPU's array: calls that overlap on one GPU
 //    (two streams, two threads) race. Calls on one stream are ordered.
 // Neither call allocates or frees device or pinned memory.

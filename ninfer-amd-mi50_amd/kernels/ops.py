@@ -715,8 +715,7 @@ class HipOps:
                 if self._attn_ws is not None:
                     self._outgrown.append(self._attn_ws)
                     ws_floats = max(ws_floats, 2 * self._attn_ws.numel())
-                # zeros: the workspace begins with counters that the kernels find and leave at zero
-                self._attn_ws = torch.zeros(ws_floats, dtype=torch.float32, device=qkv.device)
+                self._attn_ws = torch.empty(ws_floats, dtype=torch.float32, device=qkv.device)
             ws_floats = self._attn_ws.numel()
             ws = self._attn_ws.data_ptr()
         args = _AttnArgs(

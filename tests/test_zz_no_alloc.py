@@ -71,7 +71,7 @@ def test_decode_attention_without_allocation(n_q, n_kv, d, ps, window, kernel):
         c = _case(last, n_q, n_kv, d, ps, seed=11 + i)
         s = len(last)
         need = lib.ninfer_attention_workspace_floats(s, n_q, d, c["max_kv_len"])
-        ws = torch.zeros(need, dtype=torch.float32, device="cuda")   # it begins with counters
+        ws = torch.empty(need, dtype=torch.float32, device="cuda")
         want = torch.zeros(s, n_q * d, dtype=torch.bfloat16, device="cuda")
         got = torch.zeros_like(want)
         a = _args(_AttnArgs, c, want, n_q, n_kv, d, ps, window, ws)
