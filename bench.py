@@ -312,8 +312,11 @@ def main() -> int:
 
         def wrap(n):
             def call(*a, **kw):
-                if (ops._held is not None and n != "_launch_held") or depth[0]:
-                    return saved[n](*a, **kw)       # held back (timed when launched), or part of a call that is timed
+                if depth[0]:
+                    return saved[n](*a, **kw)       # part of a call that is timed
+                # inside `together()` a call is either held back (it is launched, and timed,
+                # when the block ends) or runs at once (the vendor library's products do)
+                waiting = (len(ops._held), ops._held_route) if ops._held is not None else None
                 s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 cost = call_cost(n, a, kw)
                 s.record()
@@ -323,6 +326,9 @@ def main() -> int:
                 finally:
                     depth[0] -= 1
                 e.record()
+                if waiting is not None and ops._held is not None \
+                        and (len(ops._held), ops._held_route) != waiting:
+                    return out                      # held back
                 spans.append(("products launched together" if n == "_launch_held" else kind(n, a),
                               s, e, cost))
                 return out

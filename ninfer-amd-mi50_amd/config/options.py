@@ -41,15 +41,17 @@ class EngineOptions:
             import warnings
             warnings.warn(
                 f"page_size {self.page_size}: the matrix-core attention kernels take pages of "
-                f"1, 2, 4, ... 64 tokens; with this size every bfloat16 step runs the plain "
+                f"8, 16, 32 or 64 tokens (4 too with heads of 128); with this size every bfloat16 step runs the plain "
                 f"attention kernel (one wave per row and head), which is right and many times "
                 f"slower", stacklevel=2)
 
     def page_size_suits_fast_attention(self) -> bool:
-        """The bfloat16 prompt kernel walks keys in tiles of 64 that whole pages must fill,
-        and both fast kernels find a key's page by a shift: a power of two up to 64."""
+        """The bfloat16 prompt kernel walks keys in tiles of 64 that whole pages must fill, one of
+        its loads (1 KB of a head's rows: 4 rows of heads of 128, 8 of 64) must stay inside a
+        page, and both fast kernels find a key's page by a shift: a power of two from 4 to 64
+        (pages of 4 with heads of 64 still run the plain kernel for prompt portions)."""
         ps = self.page_size
-        return ps >= 1 and ps & (ps - 1) == 0 and ps <= 64
+        return ps >= 4 and ps & (ps - 1) == 0 and ps <= 64
 
     def pages_per_request(self) -> int:
         return -(-self.max_context // self.page_size)

@@ -7,7 +7,9 @@
 // running max, sum and output of its own that are merged at the end. So every
 // SIMD holds two waves, and the softmax arithmetic of one overlaps the matrix
 // products of the other. Keys and values are walked in tiles of
-// 64 aligned to absolute positions, through LDS, both as stored ([key][d]). With
+// 64 aligned to absolute positions, through LDS, both as stored ([key][d]); they
+// are loaded from the cache's pages straight into LDS (global_load_lds_dwordx4: no
+// staging registers, no LDS stores), two or three tiles deep. With
 // v_mfma_f32_32x32x16_bf16 the wave computes
 //   S^T[key][q] = K Q^T      (A = K rows from LDS, B = Q held in registers)
 // whose accumulator layout gives lane l the scores of query l % 32 for keys
@@ -25,7 +27,7 @@
 //
 // A row at position p sees keys lo..p, lo = max(0, p - window + 1). Pages that
 // a window has passed may be gone (block-table entry -1): their keys are never
-// visible and are loaded as zeros.
+// visible, and the last key's row is loaded in their place.
 //
 // The same kernel serves decoding for models whose kv heads are shared by three
 // or more query heads (HEADS): the 32 "rows" of a block are then the query
@@ -47,27 +49,56 @@ typedef __attribute__((address_space(3))) short4v lds_short4;
 
 constexpr int PK = 64;   // keys per tile
 
+// Two transposing LDS reads (ds_read_b64_tr_b16) at byte offsets OFF0 and OFF1 from `addr`,
+// issued and not waited for: `wait_values` must come before the results are used. They are
+// written in assembly because the compiler makes the intrinsic wait for every load into LDS
+// that is under way (it cannot tell that those fill other stages); what it does not see it
+// does not wait for. LDS operations return in order and only add to the counter the
+// compiler's own waits count against, so those stay sufficient.
+template <int OFF0, int OFF1>
+__device__ __forceinline__ void tr_read2(unsigned addr, short4v& r0, short4v& r1) {
+  asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+               : "=&v"(r0), "=&v"(r1)
+               : "v"(addr), "n"(OFF0), "n"(OFF1));
+}
+
 template <int D, int NQ, bool HEADS>   // HEADS: rows are the query heads of one token (decode)
-__global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, int CHUNK) {
+__global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, int CHUNK,
+                                                                   int paired) {
   constexpr int KH = 2;             // waves per group of 32 rows: each meets one half of a tile's keys
-  constexpr int NT = NQ * KH * 64;
-  constexpr int NS = 2;              // tiles on their way in registers
+  constexpr int NW = NQ * KH;       // waves
+  constexpr int NT = NW * 64;
   constexpr int NKB = 2 / KH;       // 32-key blocks of a tile that one wave meets
   constexpr int PQ = NQ * 32;       // query rows per block
   constexpr int KS = D / 16;        // k-steps of Q K^T
   constexpr int DB = D / 32;        // 32-row blocks of O^T
-  constexpr int KPAD = D + 8;       // bf16 per K row in LDS
-  constexpr int VROW = D + 16;      // bf16 per V row in LDS: 32 bytes more than a row, so that the 4 keys x
-                                    // 4 dim quads that 16 lanes of a transposing read touch fall on 32 banks
-  constexpr int K_TILE = PK * KPAD, V_TILE = PK * VROW;   // bf16 of a tile in LDS
-  constexpr bool EARLY = NQ == 4;   // 512 threads stage half as much each: registers to spare
-  constexpr int MERGE = 2 + DB * 16 + 1;                   // floats a lane hands over at the end (odd stride)
-  constexpr int TILES_BYTES = 2 * (K_TILE + V_TILE) * 2, MERGE_BYTES = NQ * 64 * MERGE * 4;
-  // two tiles of each (one read, one written); at the end the same memory merges the two key halves
-  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[TILES_BYTES > MERGE_BYTES ? TILES_BYTES : MERGE_BYTES];
-  bf16* const k_lds = (bf16*)lds_raw;                  // [2][K_TILE]
-  bf16* const vt_lds = k_lds + 2 * K_TILE;             // [2][V_TILE]
-  __shared__ int tile_info[3];
+  // Keys and values lie in LDS as they lie in the cache, [key][d], rows of 2 D bytes without
+  // padding: they are loaded from global memory straight into LDS (global_load_lds_dwordx4:
+  // no staging registers, no LDS stores), and such a load fills 1 KB of LDS contiguously,
+  // lane l at byte 16 l. Bank conflicts of the reads are avoided by a swizzle made on the
+  // global side instead: position p of a row's 16-byte chunks holds the row's chunk
+  // p ^ swizzle(row), one swizzle for the keys' row-wise reads, another for the values'
+  // transposing reads.
+  constexpr int ROW_BYTES = 2 * D;
+  constexpr int CPR = ROW_BYTES / 16;        // 16-byte chunks of a row
+  constexpr int RPP = 64 / CPR;              // rows that one load of a wave fills (1 KB)
+  constexpr int TILE_BYTES = PK * ROW_BYTES; // of the keys, and of the values, of a tile
+  constexpr int KPT = PK / RPP / NW;         // loads per wave for a tile's keys (as many for its values)
+  static_assert(PK % (RPP * NW) == 0, "tile does not divide over the block's waves");
+  // Tiles in LDS: the one being multiplied and NST - 1 on their way. Three where one block
+  // fills a CU anyway; two for the blocks of four waves, so that two of them fit a CU.
+  constexpr int NST = NQ == 4 ? 3 : 2;
+  // All LDS reads of a phase are issued before the matrix instructions that need them.
+  constexpr bool EARLY = true;
+  // All stages lie in one array of dynamic LDS, a tile's keys, then its values, stage after
+  // stage; tile_info's three ints and the merge's (max, sum) pairs behind them.
+  constexpr int STAGE_BYTES = 2 * TILE_BYTES;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char stages[];   // NST x STAGE_BYTES + kPrefillExtra
+  // At the end the stages merge the two key halves: the output registers of a group of 32
+  // rows' second wave, 16 DB floats per lane stored [register][lane], two groups to a stage.
+  static_assert(2 * 16 * DB * 64 * 4 <= STAGE_BYTES && NQ <= 4, "two groups' outputs fit a stage");
+  float (*const merge_ml)[64][2] = (float (*)[64][2])(stages + NST * STAGE_BYTES + 16);   // [NQ][64][2]
+  int* const tile_info = (int*)(stages + NST * STAGE_BYTES);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int c = lane & 31, j = lane >> 5;
@@ -98,10 +129,22 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
     // see the most keys, come first.
     const int total = gridDim.x * gridDim.y;
     const int id = blockIdx.x + gridDim.x * blockIdx.y;
-    const int x = id % kXcds, q = total / kXcds, rem8 = total % kXcds;
-    const int w = x * q + min(x, rem8) + id / kXcds;   // a bijection: x < rem8 own one id more
-    h = w / gridDim.x;
-    const int tile = gridDim.x - 1 - w % gridDim.x;
+    int tile;
+    if (paired > 0) {
+      // Two blocks fit a CU and all blocks are resident at once: nothing is dealt out later,
+      // so what a CU gets at the start decides when it ends. The device deals block ids to
+      // the CUs in turn, the first `paired` ids one to each, the rest as their second: id k
+      // of the first gets the k-th longest piece of work (later row tiles see more keys),
+      // id paired + k the k-th shortest, so that every CU holds about the same.
+      const int rank = id < paired ? id : total - 1 - (id - paired);   // 0: the longest
+      tile = gridDim.x - 1 - rank / (int)gridDim.y;
+      h = rank % (int)gridDim.y;
+    } else {
+      const int x = id % kXcds, q = total / kXcds, rem8 = total % kXcds;
+      const int w = x * q + min(x, rem8) + id / kXcds;   // a bijection: x < rem8 own one id more
+      h = w / gridDim.x;
+      tile = gridDim.x - 1 - w % gridDim.x;
+    }
     if (!find_tile(a.seq_row_start, a.S, PQ, tile, tile_info)) return;
     row0 = tile_info[0];
     seq = tile_info[2];
@@ -152,73 +195,87 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
   const float scale2 = a.scale * 1.44269504088896f;
   float m = -1e30f, l = 0.f;
 
-  // global -> LDS mapping, the same for K and V: thread loads 16 bytes (8 dims) of a key's row.
-  // Both lie in LDS as they lie in the cache ([key][d]); the output products read V through the
-  // transposing LDS read (ds_read_b64_tr_b16), which hands a lane four keys of one dim.
-  constexpr int K_VECS = PK * D / 8;                  // 16-byte vectors in a K tile
-  constexpr int K_PER_THREAD = (K_VECS + NT - 1) / NT;
-  static_assert(K_VECS % NT == 0, "tile does not divide over the block");
-
-  // A tile's keys and values travel global -> registers (stage i % NS) -> LDS. Tile i is
-  // multiplied from LDS buffer i % 2 while tile i + 1 moves from its registers to
-  // the other buffer, the loads of tile i + 1 + NS are issued into those registers,
-  // and the page numbers of tile i + 1 + 2 NS are fetched: no load waits for another
-  // inside the loop.
-  bf16x8 kreg[NS][K_PER_THREAD], vreg[NS][K_PER_THREAD];
-  int kpage[NS][K_PER_THREAD];   // K and V of a key lie at the same place of their pools
-  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  // Every load below is unconditional (a select replaces what is not there by zeros): a
-  // load under a condition would have to be waited for where the condition ends.
-  auto load_pages = [&](int st, int t0) {
-#pragma unroll
-    for (int i = 0; i < K_PER_THREAD; ++i) {
-      int kp = t0 + (tid + i * NT) / (D / 8);
-      kpage[st][i] = bt[min(kp, pos_last) >> ps_shift];   // always a table entry of the request
-    }
-  };
-  // A tile starts at a multiple of the page size, so the place of a thread's piece inside
-  // its page is the same in every tile: address = pool + page * page_stride + in_page.
+  // Loads. Load i of wave w fills piece i NW + w of a tile's keys (and the same piece of its
+  // values): RPP rows, lane l at row l / CPR, position l % CPR, which takes the row's chunk
+  // (l % CPR) ^ swizzle(row). A key and its value lie at the same place of their pools.
+  // Every load is unconditional: for a key that is not there (beyond the last key, or on a
+  // page that a window has passed and given back) the row of the last key is loaded in its
+  // place. Such a key lies in a block that is masked, and the mask replaces its scores whatever
+  // they are; its value must be finite, since its probability is 0 and 0 x NaN is not
+  // (pages that were given back may hold anything): the last key's value is.
+  typedef const __attribute__((address_space(1))) void* gptr;
+  typedef __attribute__((address_space(3))) void* lptr;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int l_row = lane / CPR, l_pos = lane % CPR;
+  auto k_swizzle = [](int row) { return (row / (16 / CPR)) % CPR; };
+  auto v_swizzle = [](int row) { return 4 * ((row / (16 / CPR)) % (CPR / 4)); };
+  // A tile starts at a multiple of the page size, so the place of a lane's row inside its
+  // page is the same in every tile: address = pool + page * page_stride + in_page + chunk.
   const int64_t page_stride = ((int64_t)Hkv << ps_shift) * D;
-  int64_t k_in_page[K_PER_THREAD];
+  int in_page[KPT], k_chunk[KPT], v_chunk[KPT];   // in elements
 #pragma unroll
-  for (int i = 0; i < K_PER_THREAD; ++i) {
-    const int vec = tid + i * NT;
-    k_in_page[i] = (((int64_t)g << ps_shift) + ((vec / (D / 8)) & ps_mask)) * D + 8 * (vec % (D / 8));
+  for (int i = 0; i < KPT; ++i) {
+    const int row = (i * NW + wave_u) * RPP + l_row;
+    in_page[i] = (((int64_t)g << ps_shift) + (row & ps_mask)) * D;
+    k_chunk[i] = 8 * (l_pos ^ k_swizzle(row));
+    v_chunk[i] = 8 * (l_pos ^ v_swizzle(row));
   }
-  auto load_regs = [&](int st, int t0) {
+  const int pos_last_u = __builtin_amdgcn_readfirstlane(pos_last);
+  const int64_t last_at =
+      (int64_t)bt[pos_last >> ps_shift] * page_stride + (((int64_t)g << ps_shift) + (pos_last & ps_mask)) * D;
+  // Page numbers, fetched NST tiles ahead of the keys with scalar loads: the rows of one load
+  // lie in one page (a page holds at least RPP rows: see attention_prefill_takes), so its
+  // number is the same in every lane, and scalar loads do not count among the vector loads
+  // that the waits below count. (The table is read through the constant address space, which
+  // is what makes the compiler use scalar loads; nothing writes it while the kernel runs.)
+  typedef const __attribute__((address_space(4))) int* table_ptr;
+  // (the same in every lane, and said so: an address the compiler took for a lane's own
+  // would become a vector load, which the waits below would have to count)
+  const uintptr_t bt_bits = (uintptr_t)bt;
+  const table_ptr bt_c = (table_ptr)(((uintptr_t)__builtin_amdgcn_readfirstlane((unsigned)(bt_bits >> 32)) << 32) |
+                                     __builtin_amdgcn_readfirstlane((unsigned)bt_bits));
+  int kpage[NST][KPT];
+  auto load_pages = [&](int slot, int t0) {
 #pragma unroll
-    for (int i = 0; i < K_PER_THREAD; ++i) {
-      // For a key that is not there, a row of the last key's page (beyond it) or of the
-      // pool's first page (a page given back) is read in its place. Such a key lies in a
-      // block that is masked, and the mask replaces its scores whatever they are; its value
-      // must be zero: its probability is, but 0 x anything is not.
-      const int page = kpage[st][i];
-      const int64_t at = max(page, 0) * page_stride + k_in_page[i];
-      const int kp = t0 + (tid + i * NT) / (D / 8);
-      // decoding reads every key once a step; a prompt's keys serve many blocks of rows from L2
-      kreg[st][i] = HEADS ? stream_load((const bf16x8*)(kpool + at)) : *(const bf16x8*)(kpool + at);
-      const bf16x8 got = HEADS ? stream_load((const bf16x8*)(vpool + at)) : *(const bf16x8*)(vpool + at);
-      vreg[st][i] = (page >= 0 && kp <= pos_last) ? got : zero8;
+    for (int i = 0; i < KPT; ++i) {
+      const int kp = t0 + (i * NW + wave_u) * RPP;   // the load's first row
+      kpage[slot][i] = bt_c[__builtin_amdgcn_readfirstlane(min(kp, pos_last_u) >> ps_shift)];   // always a table entry of the request
     }
   };
-  auto store_regs = [&](int st, int buf) {
-    bf16* k_s = k_lds + buf * K_TILE;
-    bf16* v_s = vt_lds + buf * V_TILE;
+  // the tile at keys t0.. into stage `buf`, with the page numbers of slot `slot`
+  auto issue_tile = [&](int buf, int slot, int t0) {
+    unsigned char* kb = stages + buf * STAGE_BYTES + wave_u * 1024;
+    unsigned char* vb = kb + TILE_BYTES;
 #pragma unroll
-    for (int i = 0; i < K_PER_THREAD; ++i) {
-      int vec = tid + i * NT;
-      *(bf16x8*)(k_s + (vec / (D / 8)) * KPAD + 8 * (vec % (D / 8))) = kreg[st][i];
-      *(bf16x8*)(v_s + (vec / (D / 8)) * VROW + 8 * (vec % (D / 8))) = vreg[st][i];
+    for (int i = 0; i < KPT; ++i) {
+      const int page = kpage[slot][i];
+      const int kp = t0 + (i * NW + wave_u) * RPP + l_row;
+      const int64_t at = (page >= 0 && kp <= pos_last) ? page * page_stride + in_page[i] : last_at;
+      // decoding reads every key once a step (marked non-temporal: the last argument); a
+      // prompt's keys serve many blocks of rows from L2
+      __builtin_amdgcn_global_load_lds((gptr)(kpool + at + k_chunk[i]), (lptr)(kb + i * (NW * 1024)), 16, 0,
+                                       HEADS ? 2 : 0);
+      __builtin_amdgcn_global_load_lds((gptr)(vpool + at + v_chunk[i]), (lptr)(vb + i * (NW * 1024)), 16, 0,
+                                       HEADS ? 2 : 0);
     }
   };
 
+  // This lane's part in the transposing reads of V (see the output products below): its key
+  // row tr_key of the wave's 32 keys, dims 32 db + tr_dim .. + 3, as a byte offset into a
+  // stage. Rows + 8, + 16 and + 24 have the row's swizzle: constant offsets reach them.
+  unsigned v_at[DB];
+  {
+    const int row = 32 * NKB * kh + tr_key;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+      v_at[db] = TILE_BYTES + row * ROW_BYTES + 16 * ((4 * db + tr_dim / 8) ^ v_swizzle(row)) + 2 * (tr_dim % 8);
+  }
   // the products of this wave's part of the tile at keys t0.. in LDS buffer buf
   auto multiply = [&](int buf, int t0) {
     const int k0 = t0 + 32 * NKB * kh;
     // not for tiles beyond the last key, or out of sight of every row of the wave
     if (!wave_live || k0 > wave_pos_last || k0 + 32 * NKB <= wave_lo) return;
-    const bf16* k_s = k_lds + buf * K_TILE;
-    const bf16* vt_s = vt_lds + buf * V_TILE;
+    const unsigned char* k_s = stages + buf * STAGE_BYTES;
     // Left alone, the compiler reads each fragment from LDS just before the matrix instruction
     // that needs it (it keeps registers few), and that instruction then waits a whole LDS
     // latency: 24 such waits in a row per tile. Where registers allow (EARLY), all reads of a
@@ -227,7 +284,8 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
     f32x16 s[NKB];
     bf16x8 kf[NKB][KS];
     auto read_keys = [&](int kb, int ks) {
-      kf[kb][ks] = *(const bf16x8*)(k_s + ((NKB * kh + kb) * 32 + c) * KPAD + 16 * ks + 8 * j);
+      const int row = (NKB * kh + kb) * 32 + c;
+      kf[kb][ks] = *(const bf16x8*)(k_s + row * ROW_BYTES + 16 * ((2 * ks + j) ^ k_swizzle(row)));
     };
     if constexpr (EARLY) {
 #pragma unroll
@@ -247,28 +305,20 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
         s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb][ks], qf[ks], s[kb], 0, 0, 0);
       }
     }
-    // the values: with EARLY read here, while the vector units form the probabilities
-    bf16x8 vf[DB][NKB][2];
+    // The values are read here, while the vector units form the probabilities.
     // The transposing read works in groups of 16 lanes: lane s of a group fetches 8 bytes from
     // an address of its own, and lane i receives element i % 4 of what lanes i / 4 + 4 v
     // fetched, v = 0 .. 3. With lane s at key v = s / 4, dims 4 (s % 4) .. + 3 of the group's
     // 16 dims, lane i gets four consecutive keys of dim i: half of the operand's 8 keys.
-    auto read_values = [&](int db, int kb, int hs) {
-      const bf16* vr = vt_s + (32 * (NKB * kh + kb) + 16 * hs + tr_key) * VROW + db * 32 + tr_dim;
-      const short4v lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)vr);
-      const short4v hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4*)(vr + 8 * VROW));
-      typedef short short8v __attribute__((ext_vector_type(8)));
-      const short8v both = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-      vf[db][kb][hs] = __builtin_bit_cast(bf16x8, both);
-    };
-    if constexpr (EARLY) {
+    static_assert(NKB == 1, "one block of 32 keys per wave and tile");
+    short4v vlo[DB][2], vhi[DB][2];
+    {
+      const unsigned base = (unsigned)(uintptr_t)(lds_short4*)k_s;
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-          for (int hs = 0; hs < 2; ++hs) read_values(db, kb, hs);
-      asm volatile("" ::: "memory");
+      for (int db = 0; db < DB; ++db) {
+        tr_read2<0, 8 * ROW_BYTES>(base + v_at[db], vlo[db][0], vhi[db][0]);
+        tr_read2<16 * ROW_BYTES, 24 * ROW_BYTES>(base + v_at[db], vlo[db][1], vhi[db][1]);
+      }
     }
     // lane holds, for query c, keys k0 + 32 kb + 8 (v / 4) + 4 j + v % 4
     float mx = -1e30f;
@@ -319,69 +369,84 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
         pf[kb][v >> 3][v & 7] = (__bf16)p;
       }
     l += psum;
+    // the values have arrived (every register the reads fill passes through this statement)
+    if constexpr (DB == 4)
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(vlo[0][0]), "+v"(vhi[0][0]), "+v"(vlo[0][1]), "+v"(vhi[0][1]), "+v"(vlo[1][0]),
+                     "+v"(vhi[1][0]), "+v"(vlo[1][1]), "+v"(vhi[1][1]), "+v"(vlo[2][0]), "+v"(vhi[2][0]),
+                     "+v"(vlo[2][1]), "+v"(vhi[2][1]), "+v"(vlo[3][0]), "+v"(vhi[3][0]), "+v"(vlo[3][1]),
+                     "+v"(vhi[3][1]));
+    else
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(vlo[0][0]), "+v"(vhi[0][0]), "+v"(vlo[0][1]), "+v"(vhi[0][1]), "+v"(vlo[1][0]),
+                     "+v"(vhi[1][0]), "+v"(vlo[1][1]), "+v"(vhi[1][1]));
+    static_assert(DB == 4 || DB == 2, "head sizes 128 and 64");
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
 #pragma unroll
-      for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-        for (int hs = 0; hs < 2; ++hs) {
-          if constexpr (!EARLY) read_values(db, kb, hs);
-          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][kb][hs], pf[kb][hs], o[db], 0, 0, 0);
-        }
+      for (int hs = 0; hs < 2; ++hs) {
+        typedef short short8v __attribute__((ext_vector_type(8)));
+        const short4v lo4 = vlo[db][hs], hi4 = vhi[db][hs];
+        const short8v both = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf[0][hs], o[db], 0, 0, 0);
+      }
     }
   };
 
+  // A wave's loads return in the order of their issue. Per tile it issues 2 KPT loads into
+  // LDS (and nothing else that the vector memory counter counts); when tile i is needed, the
+  // loads issued after its own are those of the NST - 2 tiles after it.
+  constexpr int YOUNGER = (NST - 2) * 2 * KPT;
   const int t_first = (lo_first / PK) * PK;
 #pragma unroll
-  for (int st = 0; st < NS; ++st) load_pages(st, t_first + st * PK);
+  for (int st = 0; st < NST; ++st) load_pages(st, t_first + st * PK);
 #pragma unroll
-  for (int st = 0; st < NS; ++st) {
-    load_regs(st, t_first + st * PK);
-    load_pages(st, t_first + (NS + st) * PK);
+  for (int st = 0; st + 1 < NST; ++st) {
+    issue_tile(st, st, t_first + st * PK);
+    load_pages(st, t_first + (NST + st) * PK);
   }
-  store_regs(0, 0);
-  load_regs(0, t_first + NS * PK);
-  load_pages(0, t_first + 2 * NS * PK);
-  lds_barrier();
-  // NS tiles per turn, so that the register stage and the buffer of each are constants.
-  // Nothing in the loop stands under a condition: tiles beyond the last key are loaded as
-  // zeros and skipped by the products, so the wait before a store counts exactly the loads
-  // issued after the ones it needs.
-  for (int t0 = t_first; t0 <= pos_last; t0 += NS * PK) {
+  // NST tiles per turn, so that the stage and the page slot of each are constants. Nothing
+  // in the loop stands under a condition: tiles beyond the last key are loaded (the last
+  // key's row, over and over) and skipped by the products, so the wait counts exactly the
+  // loads issued after the ones it needs.
+  for (int t0 = t_first; t0 <= pos_last; t0 += NST * PK) {
 #pragma unroll
-    for (int u = 0; u < NS; ++u) {
-      const int st = (u + 1) % NS;
-      store_regs(st, (u + 1) % 2);
-      load_regs(st, t0 + (u + 1 + NS) * PK);
-      load_pages(st, t0 + (u + 1 + 2 * NS) * PK);
-      multiply(u % 2, t0 + u * PK);
-      lds_barrier();   // the next tile is whole, this one has been read by every wave
+    for (int u = 0; u < NST; ++u) {
+      // this wave's part of tile u has landed; after the barrier everybody's has, and the
+      // tile before has been read by every wave (one statement: nothing moves across it)
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(YOUNGER) : "memory");
+      constexpr int FREE = (NST - 1);   // (u + NST - 1) % NST: the stage of the tile before
+      issue_tile((u + FREE) % NST, (u + FREE) % NST, t0 + (u + NST - 1) * PK);
+      load_pages((u + FREE) % NST, t0 + (u + 2 * NST - 1) * PK);
+      multiply(u, t0 + u * PK);
     }
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may land in LDS after this
+  __syncthreads();
 
   // Merge the two key halves of every row group: the waves of the second half hand their
   // max, sum and output over through LDS (the last barrier of the loop has freed it).
-  float* mine = (float*)lds_raw + (qg * 64 + lane) * MERGE;
+  float* mine = (float*)(stages + (qg >> 1) * STAGE_BYTES) + (qg & 1) * (16 * DB * 64) + lane;
   if (kh == 1) {
-    mine[0] = m;
-    mine[1] = l;
+    merge_ml[qg][lane][0] = m;
+    merge_ml[qg][lane][1] = l;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) mine[2 + 16 * db + v] = o[db][v];
+      for (int v = 0; v < 16; ++v) mine[(16 * db + v) * 64] = o[db][v];
   }
   __syncthreads();
   if (kh == 1) return;
   float m_all;
   {
-    const float m1 = mine[0], l1 = mine[1];
+    const float m1 = merge_ml[qg][lane][0], l1 = merge_ml[qg][lane][1];
     m_all = fmaxf(m, m1);
     const float a0 = __builtin_amdgcn_exp2f(m - m_all), a1 = __builtin_amdgcn_exp2f(m1 - m_all);
     l = l * a0 + l1 * a1;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) o[db][v] = o[db][v] * a0 + mine[2 + 16 * db + v] * a1;
+      for (int v = 0; v < 16; ++v) o[db][v] = o[db][v] * a0 + mine[(16 * db + v) * 64] * a1;
   }
   // the two lanes of a query hold partial sums of l
   l += __shfl_xor(l, 32, 64);
@@ -420,11 +485,40 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
   }
 }
 
+// LDS of a block beside its stages: tile_info, then the merge's (max, sum) pairs.
+constexpr int kPrefillExtra = 16 + 4 * 64 * 2 * 4;
+
+// Bytes of dynamic LDS of attn_prefill_kernel<D, NQ, .> (as the kernel lays them out).
+static size_t prefill_lds(int D, int nq) {
+  const int stages = nq == 4 ? 3 : 2;
+  return (size_t)stages * 2 * PK * 2 * D + kPrefillExtra;
+}
+
+// Pages the matrix-core kernels take: a power of two that divides the tile of 64 keys and
+// holds the rows that one load into LDS fills (1 KB: 4 rows of heads of 128, 8 of 64), so
+// that a load's rows share their page.
+static bool prefill_page_ok(const AttnArgs& a) {
+  return PK % a.page_size == 0 && a.page_size * 2 * a.D >= 1024;
+}
+
+template <int D, int NQ, bool HEADS>
+static int launch_attn(const AttnArgs& a, dim3 grid, int chunk, int paired, hipStream_t stream) {
+  auto kern = attn_prefill_kernel<D, NQ, HEADS>;
+  const size_t lds = prefill_lds(D, NQ);
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return set_error(-2, "paged_attention: cannot get %zu bytes of LDS", lds);
+  }
+  kern<<<grid, NQ * 128, lds, stream>>>(a, chunk, paired);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
 // Decoding with grouped heads: bf16, head size 64 or 128, 3 to 32 query heads per kv head.
 bool attention_decode_heads_takes(const AttnArgs& a) {
   const int group = a.Hq / a.Hkv;
   return a.dtype == kBF16 && (a.D == 64 || a.D == 128) && a.q_stride % 8 == 0 &&
-         PK % a.page_size == 0 && group >= 3 && group <= 32 && a.workspace != nullptr &&
+         prefill_page_ok(a) && group >= 3 && group <= 32 && a.workspace != nullptr &&
          a.row_seq != nullptr;
 }
 
@@ -435,35 +529,44 @@ int attention_decode_heads(const AttnArgs& a, int chunk, int n_chunks, hipStream
   NINFER_REQUIRE(chunk > 0 && chunk % PK == 0, "paged_attention: chunks of %d keys are no "
                  "multiple of %d", chunk, PK);
   dim3 grid(a.Hkv, n_chunks, a.T);
-  if (a.D == 128)
-    attn_prefill_kernel<128, 2, true><<<grid, 256, 0, stream>>>(a, chunk);
-  else
-    attn_prefill_kernel<64, 2, true><<<grid, 256, 0, stream>>>(a, chunk);
-  NINFER_LAUNCH_CHECK();
-  return 0;
+  if (a.D == 128) return launch_attn<128, 2, true>(a, grid, chunk, 0, stream);
+  return launch_attn<64, 2, true>(a, grid, chunk, 0, stream);
 }
 
 bool attention_prefill_takes(const AttnArgs& a) {
   return a.dtype == kBF16 && (a.D == 64 || a.D == 128) && a.q_stride % 8 == 0 &&
-         PK % a.page_size == 0 && a.seq_row_start != nullptr;
+         prefill_page_ok(a) && a.seq_row_start != nullptr;
 }
 
+// Row tiles of PQ rows that the launch enumerates (one more per request than whole tiles:
+// a request's last tile may be partial; tiles that do not exist exit at once).
+static int prefill_tiles(const AttnArgs& a, int pq) { return (a.T + pq - 1) / pq + a.S; }
+
 template <int NQ>
-static int launch_prefill(const AttnArgs& a, hipStream_t stream) {
+static int launch_prefill(const AttnArgs& a, int paired, hipStream_t stream) {
   constexpr int PQ = NQ * 32;
-  dim3 grid((a.T + PQ - 1) / PQ + a.S, a.Hq);
-  if (a.D == 128)
-    attn_prefill_kernel<128, NQ, false><<<grid, NQ * 128, 0, stream>>>(a, 0);
-  else
-    attn_prefill_kernel<64, NQ, false><<<grid, NQ * 128, 0, stream>>>(a, 0);
-  NINFER_LAUNCH_CHECK();
-  return 0;
+  dim3 grid(prefill_tiles(a, PQ), a.Hq);
+  if (a.D == 128) return launch_attn<128, NQ, false>(a, grid, 0, paired, stream);
+  return launch_attn<64, NQ, false>(a, grid, 0, paired, stream);
 }
 
 int attention_prefill(const AttnArgs& a, hipStream_t stream) {
-  // 128 rows per block when requests bring that many: every key loaded serves more rows
-  if (a.max_qlen > 64) return launch_prefill<4>(a, stream);
-  return launch_prefill<2>(a, stream);
+  // 128 rows per block when requests bring that many: every key loaded serves more rows.
+  // But a causal prompt's row tiles differ in length by their number, and while the 128-row
+  // blocks are no more than the CUs, each CU gets at most one and the longest decides (2,048
+  // rows of 16 heads: 256 blocks, the last of 16 times the first's length). Blocks of 64 rows
+  // fit two to a CU: twice as many, all resident at once, and when they are more than the
+  // CUs they are handed out so that every CU holds a long and a short one (measured at 16
+  // heads of 128: 40 against 44 us at 2,048 rows, 21.5 against 26 at 1,024, 15 against 18 at
+  // 512; from 3,072 rows on the 128-row blocks win, 62 against 70 us).
+  const int cus = device_cu_count();
+  if (a.max_qlen > 64) {
+    // (tiles that hold rows; the launch enumerates a few more, which exit at once)
+    const long big = (long)((a.T + 127) / 128) * a.Hq, small = (long)((a.T + 63) / 64) * a.Hq;
+    if (big > cus) return launch_prefill<4>(a, 0, stream);
+    return launch_prefill<2>(a, small > cus ? cus : 0, stream);
+  }
+  return launch_prefill<2>(a, 0, stream);
 }
 
 }  // namespace ninfer

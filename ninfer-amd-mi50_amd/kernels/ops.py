@@ -177,8 +177,9 @@ class HipOps:
         self._side_events = None    # (start, end) of the `beside()` block
         self._side_open = False     # a `beside()` block that `join()` has not waited for
         # rows from which independent work is worth a second stream (switching streams costs the
-        # host about 0.1 ms a layer: at 512 rows of the smaller model the host then is the slower)
-        self.beside_min_rows = 1024
+        # host about 0.1 ms a layer; a 512-token portion of the smaller model: 7.95 ms with it,
+        # 8.32 without, 256 tokens 7.30 against 7.28)
+        self.beside_min_rows = 512
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
         # ... a SwiGLU's gate/up product only beyond this many: up to here the tile kernel with
         # the activation in its epilogue beats the library's product followed by a kernel for
@@ -430,10 +431,8 @@ class HipOps:
         if only_if_split:
             # a dense product of few dozen rows: the library's unless the kernels here cut it
             # along K (its output tiles alone would not fill the GPU). The one workspace of
-            # the cut belongs to the main stream: work inside `beside()` starts at
-            # `beside_min_rows` rows, a cut ends at `split_max_rows`, and the callers keep the
-            # first above the second; on the second stream nothing is cut (the library's
-            # product runs instead).
+            # the cut belongs to the main stream: on the second stream nothing is cut (the
+            # library's product runs instead).
             if self._side is not None \
                     and torch.cuda.current_stream().cuda_stream == self._side.cuda_stream:
                 return False
