@@ -231,9 +231,12 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
   typedef const __attribute__((address_space(4))) int* table_ptr;
   // (the same in every lane, and said so: an address the compiler took for a lane's own
   // would become a vector load, which the waits below would have to count)
+  // (the halves go through unsigned: the intrinsic returns an int, and a low half with its top
+  // bit set would otherwise widen with ones all over the high half)
   const uintptr_t bt_bits = (uintptr_t)bt;
-  const table_ptr bt_c = (table_ptr)(((uintptr_t)__builtin_amdgcn_readfirstlane((unsigned)(bt_bits >> 32)) << 32) |
-                                     __builtin_amdgcn_readfirstlane((unsigned)bt_bits));
+  const unsigned bt_hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(bt_bits >> 32));
+  const unsigned bt_lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)bt_bits);
+  const table_ptr bt_c = (table_ptr)(((uintptr_t)bt_hi << 32) | (uintptr_t)bt_lo);
   int kpage[NST][KPT];
   auto load_pages = [&](int slot, int t0) {
 #pragma unroll
