@@ -61,26 +61,31 @@ __global__ void fill_nan_pages_kernel(T* __restrict__ pool, const int* __restric
     dst[i] = nan;
 }
 
-// A kernel that only reads: every block walks its share of the buffer with 16-byte
-// non-temporal loads, four on their way per lane, and writes nothing unless the words add
-// up to a value they never add up to (which keeps the loads). What it reaches is the rate at
-// which this part streams memory that is read once: the measure a decode step's weights
+// A kernel that only reads: every wave walks a contiguous part of the buffer from one end to
+// the other (whole 1 KB pieces per instruction, 16-byte non-temporal loads, eight on their
+// way per lane: the pattern that streams fastest on this part) and writes nothing unless the
+// words add up to a value they never add up to (which keeps the loads). What it reaches is
+// the rate at which memory that is read once streams: the measure a decode step's weights
 // and cache are held against.
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(256) void read_probe_kernel(const u32x4* __restrict__ p, int64_t n_vec,
                                                          unsigned* __restrict__ sink) {
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t waves = (int64_t)gridDim.x * (blockDim.x >> 6);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int64_t per = (n_vec / 64 + waves - 1) / waves * 64;   // vectors of a wave's part
+  const int64_t end = min(n_vec, (wave + 1) * per);
+  int64_t i = wave * per + lane;
   unsigned acc = 0;
-  for (; i + 3 * stride < n_vec; i += 4 * stride) {
-    const u32x4 a = __builtin_nontemporal_load(p + i), b = __builtin_nontemporal_load(p + i + stride),
-                c = __builtin_nontemporal_load(p + i + 2 * stride),
-                d = __builtin_nontemporal_load(p + i + 3 * stride);
-    acc += (a.x ^ a.y ^ a.z ^ a.w) + (b.x ^ b.y ^ b.z ^ b.w) + (c.x ^ c.y ^ c.z ^ c.w) +
-           (d.x ^ d.y ^ d.z ^ d.w);
+  for (; i + 7 * 64 < end; i += 8 * 64) {
+    u32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(p + i + 64 * u);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
   }
-  for (; i < n_vec; i += stride) {
+  for (; i < end; i += 64) {
     const u32x4 a = __builtin_nontemporal_load(p + i);
     acc += a.x ^ a.y ^ a.z ^ a.w;
   }
@@ -95,7 +100,7 @@ using namespace ninfer;
 // and writes nothing: for measuring the rate of a plain read.
 extern "C" int ninfer_read_probe(const void* p, long long bytes, hipStream_t stream) {
   NINFER_REQUIRE(p && bytes >= 16 && ((uintptr_t)p & 15) == 0, "read_probe: %lld bytes at %p", bytes, p);
-  const int blocks = 8 * device_cu_count();
+  const int blocks = 16 * device_cu_count();
   read_probe_kernel<<<blocks, 256, 0, stream>>>((const u32x4*)p, bytes / 16, nullptr);
   NINFER_LAUNCH_CHECK();
   return 0;

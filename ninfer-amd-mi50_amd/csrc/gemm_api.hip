@@ -48,6 +48,7 @@ extern "C" int ninfer_gemm_pair(const GemmArgs* a, const GemmArgs* b, int force_
 static int route_by(const GemmArgs& a, const RouteArgs& rt, hipStream_t stream) {
   const float* logits = (const float*)a.C;
   if (a.M <= 16) return ninfer_moe_route_small(logits, a.ldc, a.M, &rt, stream);
+  if (rt.parts) return ninfer_moe_route_many(logits, a.ldc, a.M, &rt, stream);
   int rc = ninfer_router_topk(logits, a.ldc, a.M, &rt, stream);
   if (rc) return rc;
   return ninfer_moe_align(rt.ids, a.M * rt.k, rt.E, rt.offsets, rt.order, rt.tiles16,

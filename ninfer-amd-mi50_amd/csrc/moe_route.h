@@ -26,6 +26,8 @@ struct RouteArgs {
   int* tiles_big;
   int* tile_counts;
   const float* choice_bias;  // [E] added to the scores for the choice only, or null
+  int* parts;        // [ceil(T / kAlignRowsPerBlock), E] scratch for the routing of many rows
+                     // (counts of the chosen experts per block of rows), or null
   int E;
   int k;
   int renorm;
@@ -34,6 +36,9 @@ struct RouteArgs {
 };
 
 constexpr int kMaxExpertsPerLane = 16;  // up to 1024 experts
+// Many rows: the grouping runs as blocks of this many rows side by side (a launch that counts
+// what each block's rows chose, then one that places them).
+constexpr int kAlignRowsPerBlock = 1024;
 
 // One wave per row: scores, choice and weights as RouteArgs says; writes ids[0..k) and
 // wts[0..k). Returns the expert that lane j < k chose as its j-th (the value it writes to
@@ -198,5 +203,10 @@ extern "C" int ninfer_router_topk(const float* logits, int ld, int T, const ninf
 extern "C" int ninfer_moe_align(const int* ids, int n, int E, int* offsets, int* order,
                                 int* tiles16, int* tiles_big, int* tile_counts,
                                 hipStream_t stream);
+// Scores + top-k and the grouping of many rows (T > 16) in three launches whose blocks work
+// side by side; needs rt->parts. Without it (or for few rows) callers run ninfer_router_topk
+// and ninfer_moe_align, whose grouping is one block.
+extern "C" int ninfer_moe_route_many(const float* logits, int ld, int T,
+                                     const ninfer::RouteArgs* rt, hipStream_t stream);
 extern "C" int ninfer_moe_route_small(const float* logits, int ld, int T,
                                       const ninfer::RouteArgs* rt, hipStream_t stream);

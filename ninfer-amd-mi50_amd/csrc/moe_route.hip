@@ -21,6 +21,89 @@ __global__ void moe_align_kernel(const int* __restrict__ ids, int n, int E,
   align_block(ids, n, E, offsets, order, tiles16, tiles_big, tile_counts, cnt);
 }
 
+// Many rows, after the top-k kernel: block b counts the experts that rows
+// [b, b + 1) x kAlignRowsPerBlock chose; the counts go to parts[b][E].
+__global__ __launch_bounds__(1024) void moe_count_kernel(int T, RouteArgs rt) {
+  extern __shared__ int cnt[];   // E
+  const int E = rt.E;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  const int i0 = blockIdx.x * kAlignRowsPerBlock * rt.k, i1 = min(T * rt.k, i0 + kAlignRowsPerBlock * rt.k);
+  for (int i = i0 + threadIdx.x; i < i1; i += blockDim.x) atomicAdd(&cnt[min(max(rt.ids[i], 0), E - 1)], 1);
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += blockDim.x) rt.parts[(int64_t)blockIdx.x * E + e] = cnt[e];
+}
+
+// Many rows, last launch: block b groups rows [b, b + 1) x kAlignRowsPerBlock. Every block
+// adds up the counts of all blocks (an expert's total, and what lies before its own rows), scans the totals into the experts' ranges, and places its rows with cursors of its
+// own in LDS; block 0 also writes the ranges and the tile lists. The order inside an expert
+// is rows of earlier blocks first; within a block it is not fixed (no result depends on it).
+__global__ __launch_bounds__(1024) void moe_align_parts_kernel(int T, RouteArgs rt, int n_parts) {
+  extern __shared__ int lds[];   // total[E], cursor[E], one more
+  int* total = lds;
+  int* cursor = lds + rt.E;
+  const int E = rt.E, k = rt.k;
+  const int first_part = blockIdx.x;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) total[e] = cursor[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_parts * E; i += blockDim.x) {   // (sums of ints: any order)
+    const int c = rt.parts[i];
+    if (c) {
+      atomicAdd(&total[i % E], c);
+      if (i / E < first_part) atomicAdd(&cursor[i % E], c);
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    // the first wave scans 64 experts at a time: rows, 16-row tiles, tall tiles
+    constexpr int big = kGroupedTileRows;
+    const int lane = threadIdx.x;
+    const bool writes = blockIdx.x == 0;
+    int run0 = 0, n16 = 0, nbig = 0;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+      const int e = e0 + lane;
+      const int c = e < E ? total[e] : 0;
+      const int t16 = (c + 15) / 16, tb = (c + big - 1) / big;
+      int ic = c, i16 = t16, ib = tb;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        int a1 = __shfl_up(ic, off, 64), a2 = __shfl_up(i16, off, 64), a3 = __shfl_up(ib, off, 64);
+        if (lane >= off) {
+          ic += a1;
+          i16 += a2;
+          ib += a3;
+        }
+      }
+      const int run = run0 + ic - c;
+      if (e < E) {
+        cursor[e] += run;
+        if (writes) {
+          rt.offsets[e] = run;
+          if (rt.tiles16) {
+            int p16 = n16 + i16 - t16, pb = nbig + ib - tb;
+            for (int r = run; r < run + c; r += 16) ((int4*)rt.tiles16)[p16++] = make_int4(e, r, run + c, 0);
+            for (int r = run; r < run + c; r += big) ((int4*)rt.tiles_big)[pb++] = make_int4(e, r, run + c, 0);
+          }
+        }
+      }
+      run0 += __shfl(ic, 63, 64);
+      n16 += __shfl(i16, 63, 64);
+      nbig += __shfl(ib, 63, 64);
+    }
+    if (writes && lane == 0) {
+      rt.offsets[E] = run0;
+      if (rt.tile_counts) {
+        rt.tile_counts[0] = n16;
+        rt.tile_counts[1] = nbig;
+      }
+    }
+  }
+  __syncthreads();
+  const int i0 = blockIdx.x * kAlignRowsPerBlock * k, i1 = min(T * k, i0 + kAlignRowsPerBlock * k);
+  for (int i = i0 + threadIdx.x; i < i1; i += blockDim.x)
+    rt.order[atomicAdd(&cursor[min(max(rt.ids[i], 0), E - 1)], 1)] = i;
+}
+
 // Few rows (decode): scores + top-k of every row and the grouping by expert
 // in one launch of one block.
 template <int NPL>
@@ -88,6 +171,28 @@ extern "C" int ninfer_moe_align(const int* ids, int n, int E, int* offsets, int*
                  "moe_align: tile lists come together or not at all");
   moe_align_kernel<<<1, 1024, (E + 1) * sizeof(int), stream>>>(ids, n, E, offsets, order, tiles16,
                                                                tiles_big, tile_counts);
+  NINFER_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int ninfer_moe_route_many(const float* logits, int ld, int T, const RouteArgs* rt,
+                                     hipStream_t stream) {
+  NINFER_REQUIRE(T > 0, "moe_route_many: T=%d must be positive", T);
+  int rc = route_args_check("moe_route_many", *rt, ld);
+  if (rc) return rc;
+  NINFER_REQUIRE(rt->offsets && rt->order && rt->parts, "moe_route_many: no place for the grouping "
+                 "or its counts");
+  NINFER_REQUIRE((!rt->tiles16) == (!rt->tiles_big) && (!rt->tiles16) == (!rt->tile_counts),
+                 "moe_route_many: tile lists come together or not at all");
+  NINFER_REQUIRE((int64_t)T * rt->k < (1LL << 31), "moe_route_many: %d rows of %d choices are too many", T,
+                 rt->k);
+  const int E = rt->E;
+  rc = ninfer_router_topk(logits, ld, T, rt, stream);
+  if (rc) return rc;
+  const int blocks = (T + kAlignRowsPerBlock - 1) / kAlignRowsPerBlock;
+  moe_count_kernel<<<blocks, 1024, E * sizeof(int), stream>>>(T, *rt);
+  NINFER_LAUNCH_CHECK();
+  moe_align_parts_kernel<<<blocks, 1024, (2 * E + 1) * sizeof(int), stream>>>(T, *rt, blocks);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

@@ -42,12 +42,17 @@ class _RouteArgs(ctypes.Structure):
     _fields_ = [("ids", ctypes.c_void_p), ("wts", ctypes.c_void_p), ("offsets", ctypes.c_void_p),
                 ("order", ctypes.c_void_p), ("tiles16", ctypes.c_void_p),
                 ("tiles_big", ctypes.c_void_p), ("tile_counts", ctypes.c_void_p),
-                ("choice_bias", ctypes.c_void_p),
+                ("choice_bias", ctypes.c_void_p), ("parts", ctypes.c_void_p),
                 ("E", ctypes.c_int), ("k", ctypes.c_int), ("renorm", ctypes.c_int),
                 ("score", ctypes.c_int), ("scale", ctypes.c_float)]
 
 
 BIG_TILE_ROWS = 256   # rows of a tall tile of the grouped products (the library's kGroupedTileRows)
+ROUTE_ROWS_PER_BLOCK = 1024  # the library's kAlignRowsPerBlock
+# rows (tokens) from which the grouping runs as several blocks side by side: 12.5 against 13 us
+# at 2,048 rows of 60 experts top-4 (11 against 10 at 1,024), 19 against 37 at 8,192, 46 against 127
+# at 32,768
+ROUTE_MANY_MIN_ROWS = 2048
 _SCORES = {"softmax": 0, "sigmoid": 1}
 
 
@@ -600,13 +605,20 @@ class HipOps:
         if choice_bias is not None:
             _dev(choice_bias, "choice_bias", torch.float32, 1)
             _need(choice_bias.shape[0] == experts, "routing: one bias per expert")
-        t16 = t64 = tc = offsets = order = None
+        t16 = t64 = tc = offsets = order = parts = None
         if r is not None:
             offsets, order = r.offsets.data_ptr(), r.order.data_ptr()
             t16, t64, tc = self._tile_ptrs(r, r.order.shape[0], experts)
+            if ids.shape[0] >= ROUTE_MANY_MIN_ROWS:
+                # many rows: the grouping runs as several blocks, which meet through counts
+                # per block of rows (scratch that lives with the routing record)
+                n_parts = -(-ids.shape[0] // ROUTE_ROWS_PER_BLOCK)
+                if getattr(r, "parts", None) is None or r.parts.numel() < n_parts * experts:
+                    r.parts = torch.empty(n_parts * experts, dtype=torch.int32, device=ids.device)
+                parts = r.parts.data_ptr()
         args = _RouteArgs(ids.data_ptr(), wts.data_ptr(), offsets, order, t16, t64, tc,
-                          _ptr(choice_bias), experts, top_k, 1 if renorm else 0, _SCORES[score],
-                          float(scale))
+                          _ptr(choice_bias), parts, experts, top_k, 1 if renorm else 0,
+                          _SCORES[score], float(scale))
         return args
 
     def router_topk(self, logits, experts, top_k, renorm, ids, wts, score="softmax",
@@ -672,6 +684,11 @@ class HipOps:
 
     def _route_now(self, logits, rargs, r, keep=None):
         t = logits.shape[0]
+        if t > 16 and rargs.parts:
+            self._ok(self.lib.ninfer_moe_route_many(
+                ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, ctypes.byref(rargs),
+                self._stream()))
+            return
         if t > 16:
             self._ok(self.lib.ninfer_router_topk(
                 ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, ctypes.byref(rargs),

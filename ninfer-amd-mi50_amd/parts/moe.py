@@ -95,6 +95,7 @@ class Routing:
                  tile_counts=None):
         self.ids, self.weights, self.offsets, self.order = ids, weights, offsets, order
         self.tiles16, self.tiles_big, self.tile_counts = tiles16, tiles_big, tile_counts
+        self.parts = None   # scratch of the routing of many rows (made by the kernel library's call)
 
 
 class RoutedExperts(Part):

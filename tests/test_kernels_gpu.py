@@ -258,10 +258,12 @@ def test_router_align_experts_combine(ops_mode, gen, dtype, t, e, k, h, inner):
 
 @pytest.mark.parametrize("t,e,k", [(1, 60, 4), (8, 60, 4), (64, 64, 8), (200, 8, 3), (300, 60, 4),
                                    (1000, 5, 2), (7, 130, 6), (40, 300, 5), (16, 65, 64),
-                                   (3, 1000, 9)])
+                                   (3, 1000, 9), (1024, 60, 4), (2048, 64, 8), (1500, 8, 3),
+                                   (4100, 130, 6), (8192, 60, 4), (1025, 1, 1), (3000, 300, 5)])
 def test_routing_in_one_call_with_tile_lists(ops, gen, t, e, k):
-    """moe_route (one launch for few rows, two for many) against the twins; the
-    tile lists cover every routed row exactly once, expert by expert."""
+    """moe_route (one launch for few rows, two for more; from 1,024 rows the grouping runs
+    as several blocks side by side) against the twins; the tile lists cover every routed row
+    exactly once, expert by expert."""
     from ninfer_amd.parts.moe import Routing
     logits = torch.randn(t, e + 1, generator=gen, device="cuda") * 2   # one more column: ignored
     n = t * k
@@ -530,7 +532,8 @@ def test_grouped_products_at_the_edges_of_the_row_blocks(ops, gen, counts, h, in
     close(y1, y2, dtype, scale=h2.float().abs().max().item() * math.sqrt(inner) * 0.3)
 
 
-@pytest.mark.parametrize("t,e,k", [(1, 60, 4), (9, 8, 3), (16, 64, 8), (40, 130, 6), (300, 60, 4)])
+@pytest.mark.parametrize("t,e,k", [(1, 60, 4), (9, 8, 3), (16, 64, 8), (40, 130, 6), (300, 60, 4),
+                                   (1100, 60, 4)])
 @pytest.mark.parametrize("score", ["softmax", "sigmoid"])
 def test_router_parameters(ops, gen, t, e, k, score):
     """The router's parameters (score function, a per-expert bias that decides the choice
