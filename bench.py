@@ -304,7 +304,7 @@ def main() -> int:
             return name
 
         names = ["embed", "rmsnorm", "qkv_rope", "rope_kv_write", "paged_attention", "linear",
-                 "swiglu_linear", "silu_mul", "grouped_swiglu", "grouped_down", "moe_route",
+                 "swiglu_linear", "grouped_swiglu", "grouped_down", "moe_route",
                  "moe_combine", "_launch_held"]
         saved = {n: getattr(ops, n) for n in names}
 

@@ -337,33 +337,9 @@ __global__ void moe_combine_kernel(float* __restrict__ residual, const T* __rest
   residual[t * H + i] += acc;
 }
 
-// out[r, i] = silu(x[r, i]) * x[r, I + i]   (reference src/ops/kernels.hip:131-140)
-template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ x, T* __restrict__ out, int inner) {
-  int64_t r = blockIdx.x;
-  const T* xr = x + r * 2 * inner;
-  T* orow = out + r * inner;
-  for (int i = threadIdx.x; i < inner; i += blockDim.x) {
-    float g = to_f32(xr[i]), u = to_f32(xr[i + inner]);
-    orow[i] = from_f32<T>(g / (1.f + expf(-g)) * u);
-  }
-}
-
 }  // namespace ninfer
 
 using namespace ninfer;
-
-extern "C" int ninfer_silu_mul(const void* x, void* out, int rows, int inner, int dtype,
-                               hipStream_t stream) {
-  NINFER_REQUIRE(rows > 0 && inner > 0, "silu_mul: rows=%d inner=%d must be positive", rows, inner);
-  NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "silu_mul: unknown dtype %d", dtype);
-  if (dtype == kF32)
-    silu_mul_kernel<float><<<rows, 256, 0, stream>>>((const float*)x, (float*)out, inner);
-  else
-    silu_mul_kernel<bf16><<<rows, 256, 0, stream>>>((const bf16*)x, (bf16*)out, inner);
-  NINFER_LAUNCH_CHECK();
-  return 0;
-}
 
 extern "C" int ninfer_embed(const int* tokens, const void* table, float* out, int T, int H,
                             int dtype, hipStream_t stream) {

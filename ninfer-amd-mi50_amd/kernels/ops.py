@@ -186,10 +186,11 @@ class HipOps:
         # 8.32 without, 256 tokens 7.30 against 7.28)
         self.beside_min_rows = 512
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
-        # ... a SwiGLU's gate/up product only beyond this many: up to here the tile kernel with
-        # the activation in its epilogue beats the library's product followed by a kernel for
-        # the activation (measured at 33, 64 and 128 rows: 70 against 98 us at 40960 x 3584)
-        self.library_min_rows_fused = 128
+        # ... but never a SwiGLU's gate/up product: the tile kernels here have the activation in
+        # their epilogue, which beats the library's product followed by a kernel for the
+        # activation at every row count (70 against 98 us at 64 rows of 40960 x 3584; whole
+        # prompt portions of 256 to 8,192 tokens 2 to 4% faster at 2048 -> 2 x 5632, the same
+        # within 1% at 3584 -> 2 x 20480)
         self.split_max_rows = 512   # most rows of a product that may be cut along K (gemm_split)
         self._attn_ws = None
         self._outgrown = []     # workspaces that captured graphs may still point to
@@ -539,14 +540,6 @@ class HipOps:
         return (not self.force_generic and x.dtype == torch.bfloat16 and out.dtype == x.dtype
                 and x.shape[0] > self.library_min_rows)
 
-    def silu_mul(self, x, out):
-        _dev(x, "x", dims=2)
-        _dev(out, "out", x.dtype, 2)
-        _need(x.shape[1] == 2 * out.shape[1] and x.shape[0] == out.shape[0], "silu_mul: shapes")
-        self._ok(self.lib.ninfer_silu_mul(ctypes.c_void_p(x.data_ptr()),
-                                          ctypes.c_void_p(out.data_ptr()), x.shape[0],
-                                          out.shape[1], _DT[x.dtype], self._stream()))
-
     def swiglu_linear(self, x, w_gate_up, out):
         """out = silu(x Wg^T) * (x Wu^T), Wg = rows [0, I), Wu = rows [I, 2I)."""
         _dev(x, "x", dims=2)
@@ -555,11 +548,6 @@ class HipOps:
         inner = w_gate_up.shape[0] // 2
         _need(w_gate_up.shape == (2 * inner, x.shape[1]), "swiglu_linear: weight shape")
         _need(out.shape == (x.shape[0], inner), "swiglu_linear: out has the wrong shape")
-        if self._use_library(x, out) and x.shape[0] > self.library_min_rows_fused:
-            gu = torch.empty((x.shape[0], 2 * inner), dtype=x.dtype, device=x.device)
-            torch.matmul(x, w_gate_up.t(), out=gu)
-            self.silu_mul(gu, out)
-            return
         self._gemm(x, w_gate_up, out, m=x.shape[0], n=inner, k=x.shape[1], epilogue=1)
 
     def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None):
