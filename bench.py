@@ -79,6 +79,8 @@ def main() -> int:
     ap.add_argument("--requests", type=int, default=8, help="--scenario long: concurrent requests")
     ap.add_argument("--prompt", type=int, default=32768, help="--scenario long: prompt tokens")
     ap.add_argument("--new", type=int, default=256, help="--scenario long: new tokens a request")
+    ap.add_argument("--portion", type=int, default=2048,
+                    help="--scenario long: the scheduler's token budget of a step")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -156,7 +158,7 @@ def main() -> int:
     def prefill_run(T: int, reps: int):
         toks = torch.randint(0, V, (T,), generator=gen).tolist()
         times = []
-        for _ in range(reps + 1):
+        for _ in range(reps + 2):
             s = runner.open()
             torch.cuda.synchronize()
             t = time.perf_counter()
@@ -164,7 +166,9 @@ def main() -> int:
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t)
             runner.close(s)
-        dt = sorted(times[1:])[len(times[1:]) // 2]
+        dt = sorted(times[2:])[len(times[2:]) // 2]
+        print(f"[bench] prefill of {T} tokens, ms: " + " ".join(f"{x * 1e3:.2f}" for x in times)
+              + " (the first two are warm-up; the median of the rest counts)", file=sys.stderr, flush=True)
         flops = T * 2 * L * ((Hq + 2 * Hkv) * D * H + Hq * D * H + E * H + k * 3 * Im * H
                              + 3 * Is * H + H) + L * 2 * Hq * D * T * T + 2 * V * H
         return dt, flops
@@ -408,7 +412,7 @@ def main() -> int:
     result["roofline"]["frac_of_read"] = round(nbytes / dt / plain_read, 4)
     if not args.no_prefill:
         pt = min(args.prefill_tokens, ctx)
-        pdt, flops = prefill_run(pt, 3)
+        pdt, flops = prefill_run(pt, 5)
         result["prefill"] = {"value": round(pt / pdt, 1), "tokens": pt,
                              "ms": round(pdt * 1e3, 3),
                              "frac": round(flops / pdt / FLOP_PEAK[args.dtype], 4)}
@@ -457,7 +461,7 @@ def long_scenario(args, raw, model_name, layers_full) -> int:
     from ninfer_amd.sampling import Sampler, SamplingParams
 
     n, plen, new = args.requests, args.prompt, args.new
-    page, chunk = 16, 2048
+    page, chunk = 16, args.portion
     ctx = -(-(plen + new) // page) * page
     opt = EngineOptions(dtype=args.dtype, max_context=ctx, prefill_chunk=chunk, num_sequences=n,
                         page_size=page, use_graph=args.graph)

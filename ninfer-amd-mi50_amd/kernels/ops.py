@@ -19,6 +19,9 @@ _c_int_p = ctypes.c_void_p
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 class KernelError(RuntimeError):
     """The kernel library refused a call (bad size, dtype or launch)."""
 
@@ -91,6 +94,9 @@ def _need(cond: bool, msg: str) -> None:
 
 
 def _dev(t: torch.Tensor, name: str, dtype=None, dims: Optional[int] = None) -> None:
+    if t.is_cuda and t.is_contiguous() and (dtype is None or t.dtype == dtype) \
+            and (dims is None or t.dim() == dims):
+        return   # (a step makes about a thousand of these checks: the good case is one test)
     _need(t.is_cuda, f"{name} must be on the GPU")
     _need(t.is_contiguous(), f"{name} must be contiguous")
     if dtype is not None:
@@ -176,14 +182,16 @@ class HipOps:
         self.lib.ninfer_attention_workspace_floats.restype = ctypes.c_longlong
         self.lib.ninfer_sample_few_places.restype = ctypes.c_longlong
         self.force_generic = False  # tests: run the plain kernels whatever the shape
+        self._device_index = None   # the one GPU's index, asked for at the first launch
         self._held = None           # products held back inside `together()`
         self._held_route = None     # ... and a routing by the logits one of them writes
         self._side = None           # the second stream of `beside()`, made at first use
         self._side_events = None    # (start, end) of the `beside()` block
         self._side_open = False     # a `beside()` block that `join()` has not waited for
         # rows from which independent work is worth a second stream (switching streams costs the
-        # host about 0.1 ms a layer; a 512-token portion of the smaller model: 7.95 ms with it,
-        # 8.32 without, 256 tokens 7.30 against 7.28)
+        # host about 0.03 ms a layer, and short portions are bound by the host: the smaller
+        # model's portion of 256 tokens 7.3 ms with it, 6.5 without; 512 tokens 7.5 against 7.7,
+        # 1,024 9.5 against 10.3, 2,048 13.7 against 15.1)
         self.beside_min_rows = 512
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
         # ... but never a SwiGLU's gate/up product: the tile kernels here have the activation in
@@ -228,6 +236,12 @@ class HipOps:
 
     # ---- helpers ----------------------------------------------------------------
     def _stream(self) -> ctypes.c_void_p:
+        # the current stream's handle, asked for with every launch: torch's own short way to it
+        # where this build has one (a tenth of the time of making a Stream object)
+        if _raw_stream is not None:
+            if self._device_index is None:
+                self._device_index = torch.cuda.current_device()
+            return ctypes.c_void_p(_raw_stream(self._device_index))
         return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
     def _ok(self, rc: int) -> None:
