@@ -39,6 +39,7 @@ class Qwen2MoeConfig:
     sliding_window: Optional[int] = None
     max_window_layers: int = 0
     qkv_bias: bool = True
+    hidden_act: str = "silu"   # the gate's activation in every feed-forward: 'silu' | 'gelu_pytorch_tanh'
     eos_token_ids: Tuple[int, ...] = ()   # every id that ends a generation (the key may hold one or a list)
     architecture: str = "Qwen2MoeForCausalLM"
 
@@ -107,8 +108,9 @@ class Qwen2MoeConfig:
         if not theta > 0:
             raise ConfigError(f"config.json: key 'rope_theta' must be > 0, got {theta}")
         act = r.opt_str("hidden_act", "silu")
-        if act != "silu":
-            raise ConfigError(f"config.json: key 'hidden_act' must be 'silu', got {act!r}")
+        if act not in ("silu", "gelu_pytorch_tanh"):
+            raise ConfigError(f"config.json: key 'hidden_act' must be 'silu' or 'gelu_pytorch_tanh', "
+                              f"got {act!r}")
         # no experts (the key absent or 0): every layer has the dense feed-forward; no shared
         # expert (absent or 0): a sparse layer is its routed experts alone
         experts = r.opt_int("num_experts", 0, 0)
@@ -152,4 +154,4 @@ class Qwen2MoeConfig:
             decoder_sparse_step=sparse_step, mlp_only_layers=mlp_only,
             use_sliding_window=use_win, sliding_window=window,
             max_window_layers=max_win_layers, qkv_bias=r.opt_bool("qkv_bias", True),
-            eos_token_ids=tuple(eos))
+            hidden_act=act, eos_token_ids=tuple(eos))

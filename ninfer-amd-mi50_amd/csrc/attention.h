@@ -33,13 +33,15 @@ struct AttnArgs {
   int max_kv_len;
   int single_rows;          // the first single_rows requests bring one row each: rows
                             // 0 .. single_rows - 1 (0 when the caller does not sort them)
+  const float* slopes;      // [Hq] or null: head h's scores get slopes[h] * (key position - row's
+                            // position) added before the softmax (a distance-based position bias)
 };
 
 int attention_check(const AttnArgs& a);
 int attention_generic(const void* q, int q_stride, const void* kpool, const void* vpool,
                       const int* block_table, int bt_stride, const int* positions,
                       const int* row_seq, void* out, int T, int Hq, int Hkv, int D, int page_size,
-                      int window, float scale, int dtype, hipStream_t stream);
+                      int window, float scale, const float* slopes, int dtype, hipStream_t stream);
 
 int64_t attention_decode_workspace_floats(int T, int Hq, int D, int max_kv_len);
 bool attention_decode_takes(const AttnArgs& a);

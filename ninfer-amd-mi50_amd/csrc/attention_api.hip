@@ -56,7 +56,7 @@ extern "C" int ninfer_paged_attention(const AttnArgs* a, int force_generic, hipS
   if (!force_generic && attention_prefill_takes(*a)) return attention_prefill(*a, stream);
   return attention_generic(a->q, a->q_stride, a->kpool, a->vpool, a->block_table, a->bt_stride,
                            a->positions, a->row_seq, a->out, a->T, a->Hq, a->Hkv, a->D,
-                           a->page_size, a->window, a->scale, a->dtype, stream);
+                           a->page_size, a->window, a->scale, a->slopes, a->dtype, stream);
 }
 
 // 32-bit floats of workspace the split-KV decode kernel needs for this shape.

@@ -86,6 +86,10 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
       for (int d = 0; d < 8; ++d) q[i][d] = 0.f;
     }
   }
+  // a distance-based bias on the scores: slope of each of the block's heads (0: none)
+  float slope[GQ];
+#pragma unroll
+  for (int i = 0; i < GQ; ++i) slope[i] = a.slopes && i < n_heads ? a.slopes[h0 + i] : 0.f;
   float m[GQ], l[GQ], acc[GQ][8];
 #pragma unroll
   for (int i = 0; i < GQ; ++i) {
@@ -119,6 +123,7 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
+      const float dist = (float)(wbase + (it0 + u) * KPI + kslot - pos);   // key's position - row's
       float kk[8], vv[8];
       if (ok[u]) {
         cvt8(kf[u], kk);
@@ -134,6 +139,7 @@ __global__ __launch_bounds__(kDecWaves * 64) void attn_decode_kernel(AttnArgs a,
         for (int d = 0; d < 8; ++d) s = fmaf(q[i][d], kk[d], s);
 #pragma unroll
         for (int off = LPK / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+        s = fmaf(slope[i], dist, s);
         if (ok[u]) {
           float m_new = fmaxf(m[i], s);
           float alpha = __expf(m[i] - m_new);

@@ -21,7 +21,8 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ kpool,
     const T* __restrict__ vpool, const int* __restrict__ block_table, int bt_stride,
     const int* __restrict__ positions, const int* __restrict__ row_seq, T* __restrict__ out,
-    int Hq, int Hkv, int D, int page_size, int window, float scale) {
+    int Hq, int Hkv, int D, int page_size, int window, float scale,
+    const float* __restrict__ slopes) {
   extern __shared__ float smem[];
   float* q_s = smem;                 // [D]
   float* p_s = smem + D;             // [64]
@@ -32,6 +33,7 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
   const int pos = positions[t];
   const int* bt = block_table + (int64_t)row_seq[t] * bt_stride;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const float slope = slopes ? slopes[h] : 0.f;
 
   const T* qr = q + (int64_t)t * q_stride + h * D;
   for (int d = lane; d < D; d += 64) q_s[d] = to_f32(qr[d]);
@@ -53,7 +55,7 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
       const T* kr = kpool + off;
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot = fmaf(q_s[d], to_f32(kr[d]), dot);
-      s = dot * scale;
+      s = fmaf(slope, (float)(j - pos), dot * scale);
     }
     float m_new = fmaxf(m, wave_max(s));
     float p = valid ? expf(s - m_new) : 0.f;
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
 int attention_generic(const void* q, int q_stride, const void* kpool, const void* vpool,
                       const int* block_table, int bt_stride, const int* positions,
                       const int* row_seq, void* out, int T, int Hq, int Hkv, int D, int page_size,
-                      int window, float scale, int dtype, hipStream_t stream) {
+                      int window, float scale, const float* slopes, int dtype, hipStream_t stream) {
   NINFER_REQUIRE(D <= 64 * kMaxDPerLane, "paged_attention: head size %d exceeds %d", D,
                  64 * kMaxDPerLane);
   dim3 grid(T, Hq);
@@ -96,11 +98,11 @@ int attention_generic(const void* q, int q_stride, const void* kpool, const void
   if (dtype == kF32)
     paged_attention_generic_kernel<float><<<grid, 64, lds, stream>>>(
         (const float*)q, q_stride, (const float*)kpool, (const float*)vpool, block_table, bt_stride,
-        positions, row_seq, (float*)out, Hq, Hkv, D, page_size, window, scale);
+        positions, row_seq, (float*)out, Hq, Hkv, D, page_size, window, scale, slopes);
   else
     paged_attention_generic_kernel<bf16><<<grid, 64, lds, stream>>>(
         (const bf16*)q, q_stride, (const bf16*)kpool, (const bf16*)vpool, block_table, bt_stride,
-        positions, row_seq, (bf16*)out, Hq, Hkv, D, page_size, window, scale);
+        positions, row_seq, (bf16*)out, Hq, Hkv, D, page_size, window, scale, slopes);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

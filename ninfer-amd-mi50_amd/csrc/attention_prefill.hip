@@ -193,6 +193,10 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
     for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
   // scores are kept in units of log 2, so that a probability is one v_exp_f32
   const float scale2 = a.scale * 1.44269504088896f;
+  // a distance-based bias: slope of this lane's head, in units of the unscaled scores (the
+  // scale is applied to score + bias together)
+  const bool biased = a.slopes != nullptr;
+  const float slope_raw = biased ? a.slopes[h + (HEADS ? (q_valid ? q_local : 0) : 0)] / a.scale : 0.f;
   float m = -1e30f, l = 0.f;
 
   // Loads. Load i of wave w fills piece i NW + w of a tile's keys (and the same piece of its
@@ -324,6 +328,15 @@ __global__ __launch_bounds__(NQ * 128, 2) void attn_prefill_kernel(AttnArgs a, i
       }
     }
     // lane holds, for query c, keys k0 + 32 kb + 8 (v / 4) + 4 j + v % 4
+    if (biased) {
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int kp = k0 + 32 * kb + 8 * (v >> 2) + 4 * j + (v & 3);
+          s[kb][v] = fmaf(slope_raw, (float)(kp - q_pos), s[kb][v]);
+        }
+    }
     float mx = -1e30f;
     if (k0 + 32 * NKB - 1 > all_see_last || k0 < all_see_first) {
 #pragma unroll

@@ -9,13 +9,21 @@
 namespace ninfer {
 
 // x[t,:] = table[token[t],:]   (reference src/ops/kernels.hip:150-159)
+// [+ pos_table[position[t],:], learned absolute positions: a second gather, summed in 32-bit;
+// a position beyond the table reads its last row, which the host refuses beforehand]
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ tokens, const T* __restrict__ table,
-                             float* __restrict__ out, int H) {
+                             float* __restrict__ out, int H, const int* __restrict__ positions,
+                             const T* __restrict__ pos_table, int pos_rows) {
   int64_t t = blockIdx.x;
   const T* src = table + (int64_t)tokens[t] * H;
   float* dst = out + t * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_f32(src[i]);
+  if (pos_table) {
+    const T* psrc = pos_table + (int64_t)min(max(positions[t], 0), pos_rows - 1) * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_f32(src[i]) + to_f32(psrc[i]);
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = to_f32(src[i]);
+  }
 }
 
 // A weighted sum of rows that a sparse feed-forward leaves to be added to the
@@ -341,14 +349,21 @@ __global__ void moe_combine_kernel(float* __restrict__ residual, const T* __rest
 
 using namespace ninfer;
 
+// positions / pos_table / pos_rows: learned absolute positions [pos_rows, H] of the table's
+// dtype, gathered by positions [T] and added; all null / 0: none.
 extern "C" int ninfer_embed(const int* tokens, const void* table, float* out, int T, int H,
-                            int dtype, hipStream_t stream) {
+                            int dtype, const int* positions, const void* pos_table, int pos_rows,
+                            hipStream_t stream) {
   NINFER_REQUIRE(T > 0 && H > 0, "embed: T=%d H=%d must be positive", T, H);
   NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "embed: unknown dtype %d", dtype);
+  NINFER_REQUIRE(!pos_table || (positions && pos_rows > 0),
+                 "embed: a table of positions needs the rows' positions and its row count (%d)", pos_rows);
   if (dtype == kF32)
-    embed_kernel<float><<<T, 256, 0, stream>>>(tokens, (const float*)table, out, H);
+    embed_kernel<float><<<T, 256, 0, stream>>>(tokens, (const float*)table, out, H, positions,
+                                               (const float*)pos_table, pos_rows);
   else
-    embed_kernel<bf16><<<T, 256, 0, stream>>>(tokens, (const bf16*)table, out, H);
+    embed_kernel<bf16><<<T, 256, 0, stream>>>(tokens, (const bf16*)table, out, H, positions,
+                                              (const bf16*)pos_table, pos_rows);
   NINFER_LAUNCH_CHECK();
   return 0;
 }

@@ -6,11 +6,20 @@
 
 namespace ninfer {
 
-enum Epilogue : int { kEpilogueNone = 0, kEpilogueSwiGLU = 1 };
+// A gated epilogue forms act(x Wg^T) * (x Wu^T) from the two halves of W's rows; the
+// activation is SiLU (SwiGLU) or the tanh form of GELU (GeGLU).
+enum Epilogue : int { kEpilogueNone = 0, kEpilogueSwiGLU = 1, kEpilogueGeGLU = 2 };
+inline bool epilogue_gated(int e) { return e == kEpilogueSwiGLU || e == kEpilogueGeGLU; }
+
+// Both activations are g * sigmoid(z): z = g for SiLU; for GELU's tanh form,
+// 0.5 g (1 + tanh(c (g + 0.044715 g^3))) with c = sqrt(2 / pi), z = 2 c (g + 0.044715 g^3).
+__device__ __forceinline__ float gate_logit(float g, bool gelu) {
+  return gelu ? 1.5957691216057308f * (g + 0.044715f * g * g * g) : g;
+}
 
 struct GemmArgs {
   const void* A;         // [rows, lda] activations
-  const void* W;         // [groups, N (2N for SwiGLU), K] weights
+  const void* W;         // [groups, N (2N with a gated epilogue), K] weights
   void* C;               // [rows, ldc]
   const float* bias;     // [N] or null
   const int* offsets;    // [groups + 1] sorted-row ranges per group, or null (dense)
@@ -21,7 +30,7 @@ struct GemmArgs {
   const int* tile_counts;  // {number of 16-row tiles, number of big tiles}
   int64_t w_group_stride;  // elements between the weights of two groups
   int M;                 // rows (dense) or number of sorted rows (grouped)
-  int N;                 // output features (per SwiGLU half)
+  int N;                 // output features (per half of a gated product)
   int K;
   int lda;
   int ldc;

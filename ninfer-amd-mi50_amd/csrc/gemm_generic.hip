@@ -109,7 +109,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs a) {
       float v = acc[i][j];
       if (SWIGLU) {
         float g = v;
-        v = g / (1.f + expf(-g)) * accu[i][j];
+        v = g / (1.f + expf(-gate_logit(g, a.epilogue == kEpilogueGeGLU))) * accu[i][j];
       } else if (a.bias) {
         v += a.bias[n];
       }
@@ -122,7 +122,7 @@ template <typename T, typename TC>
 static void launch(const GemmArgs& a, hipStream_t stream) {
   int m_tiles = (a.M + BM - 1) / BM + (a.offsets ? a.groups : 0);
   dim3 grid((a.N + BN - 1) / BN, m_tiles);
-  if (a.epilogue == kEpilogueSwiGLU)
+  if (epilogue_gated(a.epilogue))
     gemm_generic_kernel<T, TC, true><<<grid, 256, 0, stream>>>(a);
   else
     gemm_generic_kernel<T, TC, false><<<grid, 256, 0, stream>>>(a);
@@ -142,9 +142,9 @@ int gemm_check(const GemmArgs& a) {
   NINFER_REQUIRE(a.groups >= 1, "gemm: groups=%d must be >= 1", a.groups);
   NINFER_REQUIRE(a.offsets || a.groups == 1, "gemm: %d groups without offsets", a.groups);
   NINFER_REQUIRE(!a.a_index || a.a_div >= 1, "gemm: a_div=%d must be >= 1", a.a_div);
-  NINFER_REQUIRE(a.epilogue == kEpilogueNone || a.epilogue == kEpilogueSwiGLU,
+  NINFER_REQUIRE(a.epilogue == kEpilogueNone || epilogue_gated(a.epilogue),
                  "gemm: unknown epilogue %d", a.epilogue);
-  NINFER_REQUIRE(!(a.epilogue == kEpilogueSwiGLU && a.bias), "gemm: SwiGLU epilogue takes no bias");
+  NINFER_REQUIRE(!(epilogue_gated(a.epilogue) && a.bias), "gemm: a gated epilogue takes no bias");
   NINFER_REQUIRE(a.k_parts <= 1, "gemm: k_parts is set by the library, not by callers");
   NINFER_REQUIRE(!a.workspace || a.workspace_floats > 0, "gemm: a workspace of %ld floats",
                  (long)a.workspace_floats);

@@ -210,7 +210,7 @@ __device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, in
         if (col >= a.N) break;
         float v = sum[fg * HALVES];
         if (SWIGLU) {
-          v = v / (1.f + __expf(-v)) * sum[fg * HALVES + (SWIGLU ? 1 : 0)];
+          v = v / (1.f + __expf(-gate_logit(v, a.epilogue == kEpilogueGeGLU))) * sum[fg * HALVES + (SWIGLU ? 1 : 0)];
         } else if (a.bias) {
           v += a.bias[col];
         }
@@ -379,7 +379,7 @@ static void launch_skinny(const GemmArgs& a, int rows, bool two, hipStream_t str
   int m_tiles = a.offsets ? min((a.M + SM - 1) / SM + a.groups, a.M) : (a.M + SM - 1) / SM;
   dim3 grid((a.N + rows - 1) / rows, m_tiles);   // as plan_skinny counts them
   dim3 block(WAVES * 64);
-  bool swiglu = a.epilogue == kEpilogueSwiGLU;
+  bool swiglu = epilogue_gated(a.epilogue);
   if (two) {   // whole tiles, no SwiGLU (plan_skinny)
     if (a.out_dtype == kF32)
       gemm_skinny_kernel<WAVES, true, false, float, true><<<grid, block, 0, stream>>>(a, 16);
@@ -462,7 +462,7 @@ bool gemm_skinny_pair_takes(const GemmArgs& a, const GemmArgs& b) {
   if (!gemm_skinny_takes(a) || !gemm_skinny_takes(b) || a.bias || b.bias) return false;
   const bool dense_b = !b.offsets && b.out_dtype == kBF16;
   const bool first = !a.offsets && a.out_dtype == kF32 && a.epilogue == kEpilogueNone &&
-                     dense_b && b.epilogue == kEpilogueSwiGLU;
+                     dense_b && epilogue_gated(b.epilogue);
   const bool second = a.offsets && a.out_dtype == kBF16 && a.epilogue == kEpilogueNone &&
                       dense_b && b.epilogue == kEpilogueNone;
   return first || second;

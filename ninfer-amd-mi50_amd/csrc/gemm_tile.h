@@ -85,10 +85,10 @@ __device__ inline int staged_w_row(int r, int out0, int N) {
   return min(out0 + OUT_PER_WAVE * w + i, N - 1);
 }
 
-// silu(g) * u with the hardware's reciprocal (1 ulp) in place of an IEEE division: a tile's
+// act(g) * u with the hardware's reciprocal (1 ulp) in place of an IEEE division: a tile's
 // epilogue forms 128 of them per lane, and the division is ten instructions each.
-__device__ __forceinline__ float silu_times(float g, float u) {
-  return g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u;
+__device__ __forceinline__ float gated_times(float g, float u, bool gelu) {
+  return g * __builtin_amdgcn_rcpf(1.f + __expf(-gate_logit(g, gelu))) * u;
 }
 
 __device__ inline void store_quad(float* p, const float (&v)[4]) {
@@ -111,6 +111,7 @@ __device__ inline void write_accumulators(const GemmArgs& a, const f32x16 (&acc)
   TC* C = (TC*)a.C;
   // four features side by side go out in one store when every such group is whole and aligned
   const bool whole_quads = N % 4 == 0 && a.ldc % 4 == 0 && ((uintptr_t)a.C & 15) == 0;
+  const bool gelu = a.epilogue == kEpilogueGeGLU;
 #pragma unroll
   for (int jj = 0; jj < FJ; ++jj) {
     const int r_tile = row_of(tok0 + 32 * jj + lr);
@@ -128,7 +129,7 @@ __device__ inline void write_accumulators(const GemmArgs& a, const f32x16 (&acc)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const float g = acc[i][jj][4 * q + r], u = acc[i + (SWIGLU ? FI / 2 : 0)][jj][4 * q + r];
-            v[r] = silu_times(g, u);
+            v[r] = gated_times(g, u, gelu);
           }
           if (whole_quads) {
             if (f0 < N) store_quad(crow + f0, v);
@@ -181,6 +182,7 @@ __device__ inline void write_accumulators_staged(const GemmArgs& a, const f32x16
   static_assert(U >= 2 && U <= 64 && (U & (U - 1)) == 0, "row pieces");
   const int lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
   const int N = a.N;
+  const bool gelu = a.epilogue == kEpilogueGeGLU;
 #pragma unroll
   for (int jj = 0; jj < FJ; ++jj) {
     const int tok = 32 * jj + lr;
@@ -193,7 +195,7 @@ __device__ inline void write_accumulators_staged(const GemmArgs& a, const f32x16
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const float g = acc[i][jj][4 * q + r], u = acc[i + (SWIGLU ? FI / 2 : 0)][jj][4 * q + r];
-            val[r] = (__bf16)silu_times(g, u);
+            val[r] = (__bf16)gated_times(g, u, gelu);
           }
         } else {
           float b[4] = {0.f, 0.f, 0.f, 0.f};

@@ -228,7 +228,7 @@ constexpr int64_t kSplitMinBytes = 48 << 20;   // GemmArgs::split_min_bytes lowe
 
 template <int TM, int TN, int TK, int NW, int WGM, int P, int OCC = 2>
 static int launch_tile(const GemmArgs& a, hipStream_t stream) {
-  const bool swiglu = a.epilogue == kEpilogueSwiGLU;
+  const bool swiglu = epilogue_gated(a.epilogue);
   int m_tiles = (a.M + TM - 1) / TM + (a.offsets ? a.groups : 0);
   if (a.offsets) m_tiles = (m_tiles + kXcds - 1) / kXcds * kXcds;   // block_to_tile's bijection
   const int per_block = swiglu ? TN / 2 : TN;
@@ -266,7 +266,7 @@ int gemm_tile(const GemmArgs& a, hipStream_t stream) {
   } else if (a.offsets) {
     rows = kGroupedTileRows;
   } else {
-    const int n_units = a.epilogue == kEpilogueSwiGLU ? 2 * a.N : a.N;   // W rows
+    const int n_units = epilogue_gated(a.epilogue) ? 2 * a.N : a.N;   // W rows
     auto blocks = [&](int tm, int tn) { return ((a.M + tm - 1) / tm) * ((n_units + tn - 1) / tn); };
     const int cus = device_cu_count();
     rows = blocks(256, 256) >= cus ? 256 : blocks(128, 128) >= cus ? 128 : 64;

@@ -293,7 +293,7 @@ template <int TK>
 static int launch_direct(const GemmArgs& a, hipStream_t stream) {
   using namespace direct;
   constexpr int LDS_BYTES = (2 * TM + 3 * TN) * TK * 2;
-  const bool swiglu = a.epilogue == kEpilogueSwiGLU;
+  const bool swiglu = epilogue_gated(a.epilogue);
   int m_tiles = (a.M + TM - 1) / TM + (a.offsets ? a.groups : 0);
   if (a.offsets) m_tiles = (m_tiles + kXcds - 1) / kXcds * kXcds;   // block_to_tile's bijection
   const int per_block = swiglu ? TN / 2 : TN;

@@ -51,6 +51,10 @@ class ModelRunner:
             from ..kernels import load_ops
             ops = load_ops()
         self.ops = ops
+        limit = spec.max_positions()
+        if limit is not None and options.max_context > limit:
+            raise ValueError(f"max_context {options.max_context} is beyond the {limit} positions "
+                             f"that the model's parts allow")
         check_tensors(source.shapes(), spec.tensor_specs(), where, spec.unused_tensor_specs())
         binder = WeightBinder(source, self.device, self.act_dtype)
         spec.bind(binder)

@@ -57,6 +57,8 @@ ROUTE_ROWS_PER_BLOCK = 1024  # the library's kAlignRowsPerBlock
 # at 32,768
 ROUTE_MANY_MIN_ROWS = 2048
 _SCORES = {"softmax": 0, "sigmoid": 1}
+# activations of a gated product, by the names config.json gives them -> the library's epilogue
+GATE_ACTS = {"silu": 1, "gelu_pytorch_tanh": 2}
 
 
 class _AttnArgs(ctypes.Structure):
@@ -70,7 +72,8 @@ class _AttnArgs(ctypes.Structure):
                 ("S", ctypes.c_int), ("Hq", ctypes.c_int), ("Hkv", ctypes.c_int),
                 ("D", ctypes.c_int), ("page_size", ctypes.c_int), ("window", ctypes.c_int),
                 ("scale", ctypes.c_float), ("dtype", ctypes.c_int), ("max_qlen", ctypes.c_int),
-                ("max_kv_len", ctypes.c_int), ("single_rows", ctypes.c_int)]
+                ("max_kv_len", ctypes.c_int), ("single_rows", ctypes.c_int),
+                ("slopes", ctypes.c_void_p)]
 
 
 class _QkvRopeArgs(ctypes.Structure):
@@ -286,14 +289,24 @@ class HipOps:
                                             self._stream()))
 
     # ---- row-wise ---------------------------------------------------------------
-    def embed(self, tokens, table, out):
+    def embed(self, tokens, table, out, positions=None, pos_table=None):
+        """out[t] = table[tokens[t]] (+ pos_table[positions[t]]: learned absolute positions),
+        in 32-bit."""
         _dev(tokens, "tokens", torch.int32, 1)
         _dev(table, "table", dims=2)
         _dev(out, "out", torch.float32, 2)
         _need(out.shape == (tokens.shape[0], table.shape[1]), "embed: out has the wrong shape")
+        if pos_table is not None:
+            _dev(pos_table, "pos_table", table.dtype, 2)
+            _need(positions is not None, "embed: a table of positions needs the rows' positions")
+            _dev(positions, "positions", torch.int32, 1)
+            _need(pos_table.shape[1] == table.shape[1] and positions.shape[0] == tokens.shape[0],
+                  "embed: the table of positions or the positions have the wrong shape")
         self._ok(self.lib.ninfer_embed(
             ctypes.c_void_p(tokens.data_ptr()), ctypes.c_void_p(table.data_ptr()),
             ctypes.c_void_p(out.data_ptr()), tokens.shape[0], table.shape[1], _DT[table.dtype],
+            ctypes.c_void_p(_ptr(positions) if pos_table is not None else None),
+            ctypes.c_void_p(_ptr(pos_table)), 0 if pos_table is None else pos_table.shape[0],
             self._stream()))
 
     def rmsnorm(self, x, gain, eps, out, delta=None, rows=None, rows_sum=None):
@@ -554,19 +567,26 @@ class HipOps:
         return (not self.force_generic and x.dtype == torch.bfloat16 and out.dtype == x.dtype
                 and x.shape[0] > self.library_min_rows)
 
-    def swiglu_linear(self, x, w_gate_up, out):
-        """out = silu(x Wg^T) * (x Wu^T), Wg = rows [0, I), Wu = rows [I, 2I)."""
+    @staticmethod
+    def _gate_epilogue(act: str) -> int:
+        _need(act in GATE_ACTS, f"gated product: activation {act!r} is not one of {sorted(GATE_ACTS)}")
+        return GATE_ACTS[act]
+
+    def swiglu_linear(self, x, w_gate_up, out, act="silu"):
+        """out = act(x Wg^T) * (x Wu^T), Wg = rows [0, I), Wu = rows [I, 2I); act is SiLU or
+        the tanh form of GELU (`GATE_ACTS`)."""
         _dev(x, "x", dims=2)
         _dev(w_gate_up, "w_gate_up", x.dtype, 2)
         _dev(out, "out", x.dtype, 2)
         inner = w_gate_up.shape[0] // 2
         _need(w_gate_up.shape == (2 * inner, x.shape[1]), "swiglu_linear: weight shape")
         _need(out.shape == (x.shape[0], inner), "swiglu_linear: out has the wrong shape")
-        self._gemm(x, w_gate_up, out, m=x.shape[0], n=inner, k=x.shape[1], epilogue=1)
+        self._gemm(x, w_gate_up, out, m=x.shape[0], n=inner, k=x.shape[1],
+                   epilogue=self._gate_epilogue(act))
 
-    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None):
-        """out[r] = swiglu of row order[r] // top_k of x by the expert that owns
-        sorted position r."""
+    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None, act="silu"):
+        """out[r] = the gated product (see `swiglu_linear`) of row order[r] // top_k of x by
+        the expert that owns sorted position r."""
         _dev(x, "x", dims=2)
         _dev(w_gate_up, "w_gate_up", x.dtype, 3)
         _dev(out, "out", x.dtype, 2)
@@ -579,7 +599,8 @@ class HipOps:
         _need(offsets.shape[0] == e + 1, "grouped_swiglu: offsets size")
         _need(n == x.shape[0] * top_k and out.shape == (n, inner), "grouped_swiglu: row counts")
         self._gemm(x, w_gate_up, out, m=n, n=inner, k=h, offsets=offsets, a_index=order,
-                   a_div=top_k, groups=e, epilogue=1, w_group_stride=two_i * h, tiles=tiles)
+                   a_div=top_k, groups=e, epilogue=self._gate_epilogue(act),
+                   w_group_stride=two_i * h, tiles=tiles)
 
     def grouped_down(self, h, w_down, offsets, order, out, tiles=None):
         """out[order[r]] = h[r] Wd_e^T for the expert e that owns sorted position r."""
@@ -703,9 +724,12 @@ class HipOps:
 
     # ---- attention ------------------------------------------------------------------
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,
-                        page_size, window, scale, out, plan_only=False):
+                        page_size, window, scale, out, plan_only=False, slopes=None):
         """Attention of the rows' query heads (the first n_q * head_dim columns
-        of `qkv`) over their requests' cached keys and values. `plan_only`: launch
+        of `qkv`) over their requests' cached keys and values. `slopes` [n_q] (32-bit): head
+        h's scores get slopes[h] * (key's position - row's position) added before the softmax
+        (a distance-based position bias; negative distances, so a positive slope favours near
+        keys). `plan_only`: launch
         nothing and say how a step of single-token rows of this shape would run
         (which split-context kernel, keys per chunk, chunks)."""
         _dev(qkv, "qkv", dims=2)
@@ -719,6 +743,9 @@ class HipOps:
               "paged_attention: pools do not fit the head layout")
         _need(block_table.shape[0] == ctx.S, "paged_attention: block table rows != requests")
         _need(ctx.positions.shape[0] == t, "paged_attention: positions size")
+        if slopes is not None:
+            _dev(slopes, "slopes", torch.float32, 1)
+            _need(slopes.shape[0] == n_q, "paged_attention: one slope per query head")
         ws, ws_floats = None, 0
         single = int(getattr(ctx, "single_rows", 0))
         if (ctx.max_qlen == 1 or single > 0) and qkv.dtype == torch.bfloat16 \
@@ -741,7 +768,8 @@ class HipOps:
             block_table.data_ptr(), ctx.positions.data_ptr(), ctx.row_seq.data_ptr(),
             ctx.seq_row_start.data_ptr(), ctx.seq_qlen.data_ptr(), ctx.seq_pos0.data_ptr(),
             ws, ws_floats, qkv.shape[1], block_table.shape[1], t, ctx.S, n_q, n_kv, head_dim, page_size,
-            int(window or 0), float(scale), _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len, single)
+            int(window or 0), float(scale), _DT[qkv.dtype], ctx.max_qlen, ctx.max_kv_len, single,
+            _ptr(slopes))
         if plan_only:
             kernel, chunk, n_chunks = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
             self._ok(self.lib.ninfer_attention_decode_plan(

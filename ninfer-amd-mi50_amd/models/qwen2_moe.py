@@ -34,10 +34,11 @@ def build_qwen2_moe(cfg: Qwen2MoeConfig) -> ModelSpec:
             ff = make_part("feed_forward", "sparse_moe", prefix=p + "mlp.", hidden=h,
                            experts=cfg.num_experts, top_k=cfg.num_experts_per_tok,
                            inner=cfg.moe_intermediate_size, renorm=cfg.norm_topk_prob,
-                           shared_inner=cfg.shared_expert_intermediate_size)
+                           shared_inner=cfg.shared_expert_intermediate_size,
+                           act=cfg.hidden_act)
         else:
             ff = make_part("feed_forward", "swiglu", prefix=p + "mlp.", hidden=h,
-                           inner=cfg.intermediate_size)
+                           inner=cfg.intermediate_size, act=cfg.hidden_act)
         norm = lambda name: make_part("norm", "rmsnorm", prefix=p + name, size=h,
                                       eps=cfg.rms_norm_eps)
         blocks.append(make_part("block", "pre_norm", mixer_norm=norm("input_layernorm."),

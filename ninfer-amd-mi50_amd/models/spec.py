@@ -57,6 +57,11 @@ class ModelSpec:
     def parts(self) -> List[Part]:
         return [self.embedding, *self.blocks, self.final_norm, self.head]
 
+    def max_positions(self) -> Optional[int]:
+        """The longest request the parts allow (None: no part limits it)."""
+        limits = [x for x in (p.least_max_positions() for p in self.parts()) if x is not None]
+        return min(limits) if limits else None
+
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         out: Dict[str, TensorSpec] = {}
         for p in self.parts():

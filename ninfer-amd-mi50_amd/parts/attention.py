@@ -12,7 +12,7 @@ h // (Hq / Hkv) (src/ops/attention.hip:27-28); scale 1/sqrt(D)
 from __future__ import annotations
 
 import math
-from typing import Dict, List, Optional
+from typing import Dict, List, Optional, Sequence
 
 import torch
 
@@ -24,9 +24,16 @@ from .base import CacheNeed, CallInfo, Mixer, Part, PositionEncoding, StepContex
 class Attention(Mixer):
     def __init__(self, prefix: str, hidden: int, heads: int, kv_heads: int, head_dim: int,
                  position: PositionEncoding, qkv_bias: bool = True,
-                 window: Optional[int] = None, scale: Optional[float] = None):
+                 window: Optional[int] = None, scale: Optional[float] = None,
+                 score_slopes: Optional[Sequence[float]] = None):
+        """`score_slopes` [heads]: a distance-based position bias, slope * (key's position -
+        query's position) added to head h's scaled scores before the softmax (None: none).
+        It is a parameter of the attention kernels, beside or instead of the rotation that
+        `position` describes."""
         if heads % kv_heads:
             raise ValueError(f"heads ({heads}) must be a multiple of kv_heads ({kv_heads})")
+        if score_slopes is not None and len(score_slopes) != heads:
+            raise ValueError(f"score_slopes has {len(score_slopes)} entries for {heads} heads")
         self.prefix = prefix
         self.hidden = hidden
         self.heads = heads
@@ -36,6 +43,8 @@ class Attention(Mixer):
         self.qkv_bias = qkv_bias
         self.window = window
         self.scale = scale if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.score_slopes = None if score_slopes is None else [float(x) for x in score_slopes]
+        self.slopes: Optional[torch.Tensor] = None   # the same on the device (32-bit)
         self.w_qkv: Optional[torch.Tensor] = None
         self.b_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
@@ -73,6 +82,8 @@ class Attention(Mixer):
     def bind(self, w: WeightBinder) -> None:
         p, d = self.prefix, self.head_dim
         nq, nk = self.heads * d, self.kv_heads * d
+        if self.score_slopes is not None:
+            self.slopes = torch.tensor(self.score_slopes, dtype=torch.float32, device=w.device)
         self.w_qkv = torch.empty((self.qkv_width, self.hidden), dtype=w.act_dtype, device=w.device)
         w.matrix_into(p + "q_proj.weight", self.w_qkv[:nq])
         w.matrix_into(p + "k_proj.weight", self.w_qkv[nq:nq + nk])
@@ -98,7 +109,7 @@ class Attention(Mixer):
         attn = ctx.empty((ctx.T, self.heads * self.head_dim))
         ops.paged_attention(qkv, cache["k"], cache["v"], cache.block_table, ctx,
                             self.heads, self.kv_heads, self.head_dim,
-                            cache.page_size, self.window, self.scale, attn)
+                            cache.page_size, self.window, self.scale, attn, slopes=self.slopes)
         out = ctx.empty((ctx.T, self.hidden))
         ops.linear(attn, self.w_o, out)
         return out

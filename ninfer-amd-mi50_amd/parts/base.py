@@ -190,6 +190,17 @@ class Part:
     def children(self) -> List["Part"]:
         return []
 
+    def max_positions(self) -> Optional[int]:
+        """The most positions a request may have because of this part (a table of learned
+        positions has so many rows), or None: no limit of its own. The engine refuses a
+        `max_context` beyond the least of its parts' limits."""
+        return None
+
+    def least_max_positions(self) -> Optional[int]:
+        limits = [self.max_positions()] + [c.least_max_positions() for c in self.children()]
+        limits = [x for x in limits if x is not None]
+        return min(limits) if limits else None
+
     def all_tensor_specs(self) -> Dict[str, TensorSpec]:
         out = dict(self.tensor_specs())
         for c in self.children():

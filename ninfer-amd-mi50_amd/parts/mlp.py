@@ -18,10 +18,11 @@ from .base import FeedForward, StepContext, WeightBinder
 
 
 class SwiGLU(FeedForward):
-    def __init__(self, prefix: str, hidden: int, inner: int):
+    def __init__(self, prefix: str, hidden: int, inner: int, act: str = "silu"):
         self.prefix = prefix
         self.hidden = hidden
         self.inner = inner
+        self.act = act   # the gate's activation, by config.json's name: 'silu' | 'gelu_pytorch_tanh'
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
 
@@ -41,7 +42,7 @@ class SwiGLU(FeedForward):
 
     def gate_up(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
         h = ctx.empty((x.shape[0], self.inner))
-        ctx.ops.swiglu_linear(x, self.w_gate_up, h)
+        ctx.ops.swiglu_linear(x, self.w_gate_up, h, act=self.act)
         return h
 
     def down(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:

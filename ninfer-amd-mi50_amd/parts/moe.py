@@ -102,11 +102,12 @@ class RoutedExperts(Part):
     """E SwiGLU experts with stacked weights [E, 2I, hidden] and [E, hidden, I]
     built from the per-expert checkpoint tensors `experts.{e}.*_proj.weight`."""
 
-    def __init__(self, prefix: str, hidden: int, inner: int, experts: int):
+    def __init__(self, prefix: str, hidden: int, inner: int, experts: int, act: str = "silu"):
         self.prefix = prefix
         self.hidden = hidden
         self.inner = inner
         self.experts = experts
+        self.act = act
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
 
@@ -137,7 +138,7 @@ class RoutedExperts(Part):
         t, k = routing.ids.shape
         h = ctx.empty((t * k, self.inner))
         ctx.ops.grouped_swiglu(x, self.w_gate_up, routing.offsets, routing.order, k, h,
-                               tiles=routing)
+                               tiles=routing, act=self.act)
         return h
 
     def down(self, ctx: StepContext, h: torch.Tensor, routing: "Routing") -> torch.Tensor:
@@ -152,16 +153,16 @@ class RoutedExperts(Part):
 
 class SparseMoE(FeedForward):
     def __init__(self, prefix: str, hidden: int, experts: int, top_k: int, inner: int,
-                 renorm: bool, shared_inner: int = 0):
+                 renorm: bool, shared_inner: int = 0, act: str = "silu"):
         self.prefix = prefix
         self.hidden = hidden
         self.router = SoftmaxTopKRouter(prefix + "gate.", hidden, experts, top_k, renorm)
-        self.experts = RoutedExperts(prefix + "experts.", hidden, inner, experts)
+        self.experts = RoutedExperts(prefix + "experts.", hidden, inner, experts, act)
         self.shared: Optional[SwiGLU] = None
         self.shared_gate: Optional[torch.Tensor] = None
         self.last_ids: Optional[torch.Tensor] = None   # routing of the last step (for statistics)
         if shared_inner > 0:
-            self.shared = SwiGLU(prefix + "shared_expert.", hidden, shared_inner)
+            self.shared = SwiGLU(prefix + "shared_expert.", hidden, shared_inner, act)
 
     def children(self) -> List[Part]:
         return [self.router, self.experts] + ([self.shared] if self.shared else [])

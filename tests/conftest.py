@@ -46,7 +46,7 @@ CONFIG_B = {
     "decoder_sparse_step": 2, "mlp_only_layers": [0], "vocab_size": 384,
     "rope_theta": 1000000.0, "use_sliding_window": True, "sliding_window": 24,
     "max_window_layers": 2, "rms_norm_eps": 1e-5, "tie_word_embeddings": True,
-    "hidden_act": "silu",
+    "hidden_act": "gelu_pytorch_tanh",
 }
 
 # Heads of 64 in groups of three, so that the engine's bf16 steps run the matrix-core

@@ -80,12 +80,14 @@ def visibility(q_pos: Tensor, k_pos: Tensor, window: Optional[int]) -> Tensor:
 
 
 def attention_core(q: Tensor, k: Tensor, v: Tensor, q_pos: Tensor, k_pos: Tensor,
-                   window: Optional[int]) -> Tensor:
+                   window: Optional[int], slopes: Optional[Sequence[float]] = None) -> Tensor:
     """softmax(q k^T / sqrt(D) + mask) v with grouped heads.
 
     Query head h reads kv head h // (Hq/Hkv) (consecutive query heads share a
     kv head): reference src/ops/attention.hip:27-28; scale 1/sqrt(D):
     src/models/model.hip:285. q: [Tq,Hq,D]; k, v: [Tk,Hkv,D] -> [Tq,Hq,D].
+    `slopes` [Hq] (no counterpart in the reference, whose models rotate): a distance-based
+    position bias, slopes[h] * (key position - query position) added to head h's scaled scores.
     """
     tq, hq, d = q.shape
     hkv = k.shape[1]
@@ -96,6 +98,8 @@ def attention_core(q: Tensor, k: Tensor, v: Tensor, q_pos: Tensor, k_pos: Tensor
     for h in range(hq):
         g = h // group
         s = (q[:, h, :] @ k[:, g, :].T) * scale
+        if slopes is not None:
+            s = s + float(slopes[h]) * (k_pos[None, :] - q_pos[:, None]).to(s.dtype)
         s = s.masked_fill(~vis, float("-inf"))
         m = s.max(dim=-1, keepdim=True).values
         p = torch.exp(s - m)
@@ -126,14 +130,26 @@ def attention_qkv(x: Tensor, w: Dict[str, Tensor], prefix: str, n_heads: int, n_
     return q, k, v.view(t, n_kv, head_dim)
 
 
-def swiglu_mlp(x: Tensor, wg: Tensor, wu: Tensor, wd: Tensor) -> Tensor:
-    """(silu(x Wg^T) * (x Wu^T)) Wd^T, silu(z) = z / (1 + exp(-z)).
+def gate_activation(g: Tensor, act: str) -> Tensor:
+    """silu(z) = z / (1 + exp(-z)) (reference src/ops/kernels.hip:131-140, its only
+    activation), or for `hidden_act` = 'gelu_pytorch_tanh' the tanh form of GELU,
+    0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))) (no counterpart in the reference:
+    pinned by the library's gelu in tests/test_plain_model.py)."""
+    if act == "silu":
+        return g / (1.0 + torch.exp(-g))
+    if act == "gelu_pytorch_tanh":
+        return 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g * g * g)))
+    raise ValueError(f"hidden_act {act!r}")
+
+
+def swiglu_mlp(x: Tensor, wg: Tensor, wu: Tensor, wd: Tensor, act: str = "silu") -> Tensor:
+    """(act(x Wg^T) * (x Wu^T)) Wd^T.
 
     Reference: src/ops/kernels.hip:131-140, src/models/model.hip:313-337.
     """
     g = x @ wg.float().T
     u = x @ wu.float().T
-    return ((g / (1.0 + torch.exp(-g))) * u) @ wd.float().T
+    return (gate_activation(g, act) * u) @ wd.float().T
 
 
 def router(x: Tensor, wr: Tensor, top_k: int, renorm: bool) -> Tuple[Tensor, Tensor]:
@@ -167,7 +183,7 @@ def router(x: Tensor, wr: Tensor, top_k: int, renorm: bool) -> Tuple[Tensor, Ten
 
 
 def routed_experts(x: Tensor, ids: Tensor, wts: Tensor, w: Dict[str, Tensor],
-                   prefix: str) -> Tensor:
+                   prefix: str, act: str = "silu") -> Tensor:
     """y[t] = sum over selected experts of weight * expert(x[t]).
 
     Reference: src/models/model.hip:352-433 (gather, per-expert MLP, scale,
@@ -179,18 +195,18 @@ def routed_experts(x: Tensor, ids: Tensor, wts: Tensor, w: Dict[str, Tensor],
         rows, choice = torch.nonzero(ids == e, as_tuple=True)
         p = f"{prefix}experts.{e}."
         per[rows, choice] = swiglu_mlp(x[rows], w[p + "gate_proj.weight"], w[p + "up_proj.weight"],
-                                       w[p + "down_proj.weight"])
+                                       w[p + "down_proj.weight"], act)
     y = torch.zeros_like(x)
     for j in range(k):                                      # summed in the order of `ids`
         y += wts[:, j:j + 1] * per[:, j]
     return y
 
 
-def shared_expert(x: Tensor, w: Dict[str, Tensor], prefix: str) -> Tensor:
+def shared_expert(x: Tensor, w: Dict[str, Tensor], prefix: str, act: str = "silu") -> Tensor:
     """sigmoid(x w_gate^T) * mlp_shared(x); one gate scalar per token."""
     s = swiglu_mlp(x, w[prefix + "shared_expert.gate_proj.weight"],
                    w[prefix + "shared_expert.up_proj.weight"],
-                   w[prefix + "shared_expert.down_proj.weight"])
+                   w[prefix + "shared_expert.down_proj.weight"], act)
     gate = x @ w[prefix + "shared_expert_gate.weight"].float().T  # [T,1]
     return s / (1.0 + torch.exp(-gate))
 
@@ -215,16 +231,17 @@ def layer_window(cfg: dict, layer: int) -> Optional[int]:
 def feed_forward(x: Tensor, w: Dict[str, Tensor], cfg: dict, layer: int,
                  probe: Optional[dict] = None) -> Tensor:
     p = f"model.layers.{layer}.mlp."
+    act = cfg.get("hidden_act", "silu")
     if not layer_is_sparse(cfg, layer):
         return swiglu_mlp(x, w[p + "gate_proj.weight"], w[p + "up_proj.weight"],
-                          w[p + "down_proj.weight"])
+                          w[p + "down_proj.weight"], act)
     if probe is not None:
         probe.setdefault("router_logits", {})[layer] = x @ w[p + "gate.weight"].float().T
     ids, wts = router(x, w[p + "gate.weight"], cfg["num_experts_per_tok"],
                       cfg.get("norm_topk_prob", False))
-    y = routed_experts(x, ids, wts, w, p)
+    y = routed_experts(x, ids, wts, w, p, act)
     if cfg.get("shared_expert_intermediate_size", 0) > 0:
-        y = y + shared_expert(x, w, p)
+        y = y + shared_expert(x, w, p, act)
     return y
 
 

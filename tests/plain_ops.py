@@ -41,8 +41,11 @@ class PlainOps:
     def fill_nan_pages(self, pool, pages):
         pool.index_fill_(0, pages.long(), float("nan"))
 
-    def embed(self, tokens, table, out):
-        out.copy_(_f(table[tokens.long()]))
+    def embed(self, tokens, table, out, positions=None, pos_table=None):
+        x = _f(table[tokens.long()])
+        if pos_table is not None:
+            x = x + _f(pos_table[positions.long()])
+        out.copy_(x)
 
     def rmsnorm(self, x, gain, eps, out, delta=None, rows=None, rows_sum=None):
         extra = None
@@ -115,13 +118,20 @@ class PlainOps:
             r = r + bias
         out.copy_(r.to(out.dtype))
 
-    def swiglu_linear(self, x, w_gate_up, out):
+    @staticmethod
+    def _act(g, act):
+        if act == "silu":
+            return g / (1 + torch.exp(-g))
+        assert act == "gelu_pytorch_tanh", act
+        return 0.5 * g * (1 + torch.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g ** 3)))
+
+    def swiglu_linear(self, x, w_gate_up, out, act="silu"):
         inner = w_gate_up.shape[0] // 2
         g = _f(x) @ _f(w_gate_up[:inner]).T
         u = _f(x) @ _f(w_gate_up[inner:]).T
-        out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
+        out.copy_((self._act(g, act) * u).to(out.dtype))
 
-    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None):
+    def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None, act="silu"):
         e, two_i, _ = w_gate_up.shape
         inner = two_i // 2
         off = offsets.tolist()
@@ -132,7 +142,7 @@ class PlainOps:
             xs = _f(x[rows // top_k])
             gg = xs @ _f(w_gate_up[g, :inner]).T
             uu = xs @ _f(w_gate_up[g, inner:]).T
-            out[off[g]:off[g + 1]] = (gg / (1 + torch.exp(-gg)) * uu).to(out.dtype)
+            out[off[g]:off[g + 1]] = (self._act(gg, act) * uu).to(out.dtype)
 
     def grouped_down(self, h, w_down, offsets, order, out, tiles=None):
         e = w_down.shape[0]
@@ -186,7 +196,7 @@ class PlainOps:
         self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r)
 
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,
-                        page_size, window, scale, out):
+                        page_size, window, scale, out, slopes=None):
         t = qkv.shape[0]
         q = _f(qkv[:, :n_q * head_dim]).view(t, n_q, head_dim)
         group = n_q // n_kv
@@ -202,6 +212,8 @@ class PlainOps:
             for h in range(n_q):
                 g = h // group
                 s = (k[:, g, :] @ q[r, h]) * scale
+                if slopes is not None:
+                    s = s + float(slopes[h]) * (js - pos[r]).float().to(s.device)
                 p = torch.exp(s - s.max())
                 p = p / p.sum()
                 out[r, h * head_dim:(h + 1) * head_dim] = (p @ v[:, g, :]).to(out.dtype)

@@ -179,6 +179,32 @@ def test_toy_router_with_other_scores(tmp_path):
         torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
 
 
+def test_toy_learned_positions_and_score_bias(tmp_path):
+    """Positions without a rotation: a table of learned absolute positions gathered in the
+    embedding, and a distance-based bias on the attention scores; both are parameters of the
+    framework's parts. A context beyond the table's rows is refused when the engine is made."""
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, load_model
+    toy.register_routed()
+    cfg = toy.TOY_BIASED_CONFIG
+    d = str(tmp_path / "toy_biased")
+    ninfer_amd.write_random_model(d, cfg, 14, std=0.3)
+    _, w = util.read_folder(d)
+    assert w["embed_positions.weight"].shape == (160, 64)
+    runner = runner_for(d, seqs=3)
+    reqs = {f"r{i}": util.random_tokens(n, 83, 70 + i) for i, n in enumerate([7, 26, 15])}
+    ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
+    w0 = dict(w, **{"embed_positions.weight": torch.zeros_like(w["embed_positions.weight"])})
+    assert (toy.plain_forward_routed(w0, cfg, reqs["r1"]) - ref["r1"]).abs().max() > 1e-3, \
+        "the learned positions must matter"
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=7, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+    with pytest.raises(ValueError, match="160 positions"):
+        load_model(d, EngineOptions(dtype="float32", device="cpu", max_context=161, num_sequences=1,
+                                    page_size=4), ops=PlainOps())
+
+
 def test_toy_interleaved_pairs(tmp_path):
     """The second toy with neighbouring dims as rotation pairs: the pairing is a property of
     the position encoding that attention hands to the rotation, nothing else changes."""

@@ -279,6 +279,42 @@ def test_toy_router_with_other_scores_on_the_gpu(tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_learned_positions_and_score_bias_on_the_gpu(tmp_path, dtype):
+    """Positions without a rotation: learned absolute positions gathered in the embedding
+    kernel and a distance-based bias in the attention kernels (heads of 64 and pages of 16: in
+    bfloat16 the matrix-core prompt kernel and the split-context decode kernel), prompts in
+    portions beside decoded tokens, the tail token by token."""
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, load_model
+    toy.register_routed()
+    cfg = toy.TOY_BIASED_CONFIG
+    d = str(tmp_path / "toy_biased")
+    # (heads of 64 x 4 into a width of 64: std 0.2 keeps the logits at the size of the other toys',
+    # for which the 32-bit bound below is made)
+    ninfer_amd.write_random_model(d, cfg, 14, dtype=dtype, std=0.2)
+    _, w = util.read_folder(d)
+    runner = load_model(d, EngineOptions(dtype=dtype, max_context=160, num_sequences=3, page_size=16,
+                                         check_pages=True))
+    reqs = {f"r{i}": util.random_tokens(n, 83, 70 + i) for i, n in enumerate([7, 96, 15, 150])}
+    ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=8, max_live=3))
+    tail = util.run_schedule(runner, util.schedule_tail("r3", reqs["r3"], 32))["r3"]
+    if dtype == "float32":
+        for k in reqs:
+            torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+        torch.testing.assert_close(tail, ref["r3"], atol=3e-5, rtol=1e-4)
+    else:
+        # (routing is discontinuous: the typical row is what is bounded in bfloat16)
+        top = float(ref["r3"].abs().max())
+        for rows in (got["r3"], tail, got["r1"]):
+            want = ref["r3"] if rows.shape[0] == 150 else ref["r1"]
+            err = (rows - want).abs().max(-1).values
+            assert float(err.median()) < 0.03 * top
+    with pytest.raises(ValueError, match="160 positions"):
+        load_model(d, EngineOptions(dtype=dtype, max_context=176, num_sequences=1, page_size=16))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_toy_interleaved_pairs_on_the_gpu(tmp_path, dtype):
     """Neighbouring dims as rotation pairs (a partial rotation of 12 of 16 dims), chosen by
     the position encoding alone: the rotation kernel takes the pairing as a parameter."""

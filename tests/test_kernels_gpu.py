@@ -57,6 +57,16 @@ def test_embed(ops, gen, dtype):
     ops.embed(tokens, table, out)
     PlainOps().embed(tokens, table, ref)
     assert torch.equal(out, ref)
+    # learned absolute positions: a second gather, summed in 32-bit
+    pos_table = rnd((40, 72), dtype, gen)
+    positions = torch.randint(0, 40, (19,), generator=gen, device="cuda", dtype=torch.int32)
+    positions[3], positions[7] = 0, 39
+    ops.embed(tokens, table, out, positions=positions, pos_table=pos_table)
+    PlainOps().embed(tokens, table, ref, positions=positions, pos_table=pos_table)
+    assert torch.equal(out, ref)
+    assert not torch.equal(out, table[tokens.long()].float())
+    with pytest.raises(Exception, match="positions"):
+        ops.embed(tokens, table, out, pos_table=pos_table)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -106,13 +116,26 @@ def test_linear(ops_mode, gen, dtype, m, n, k):
 @pytest.mark.parametrize("m,inner,k", [(1, 48, 64), (5, 80, 96), (66, 176, 72), (20, 1408, 256),
                                        (3, 100, 2048), (130, 300, 128), (64, 128, 64)])
 def test_swiglu_linear(ops_mode, gen, dtype, m, inner, k):
+    """The gated product with either activation (SiLU, and the tanh form of GELU, whose twin
+    is written with tanh where the kernels use a sigmoid of twice the argument)."""
     ops = ops_mode
     x, w = rnd((m, k), dtype, gen), rnd((2 * inner, k), dtype, gen, 0.3)
-    o1 = torch.empty(m, inner, device="cuda", dtype=dtype)
-    o2 = torch.empty_like(o1)
-    ops.swiglu_linear(x, w, o1)
-    PlainOps().swiglu_linear(x, w, o2)
-    close(o1, o2, dtype, scale=k * 0.3)
+    for act in ("silu", "gelu_pytorch_tanh"):
+        o1 = torch.empty(m, inner, device="cuda", dtype=dtype)
+        o2 = torch.empty_like(o1)
+        ops.swiglu_linear(x, w, o1, act=act)
+        PlainOps().swiglu_linear(x, w, o2, act=act)
+        close(o1, o2, dtype, scale=k * 0.3)
+    if k == 64:   # the two activations are told apart
+        assert (o1.float() - ops_out(ops, x, w, inner, dtype)).abs().max() > 1e-2
+    with pytest.raises(Exception, match="activation"):
+        ops.swiglu_linear(x, w, o1, act="relu")
+
+
+def ops_out(ops, x, w, inner, dtype):
+    o = torch.empty(x.shape[0], inner, device="cuda", dtype=dtype)
+    ops.swiglu_linear(x, w, o)
+    return o.float()
 
 
 @pytest.mark.parametrize("variant", [1, 2, 3])
@@ -133,11 +156,10 @@ def test_tile_product_every_tile_height(ops, gen, variant, m, n, k):
         wgu = rnd((2 * n, k), torch.bfloat16, gen, 0.2)
         h1 = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
         h2 = torch.empty_like(h1)
-        ops.library_min_rows, saved = 1 << 30, ops.library_min_rows
-        ops.swiglu_linear(x, wgu, h1)
-        ops.library_min_rows = saved
-        PlainOps().swiglu_linear(x, wgu, h2)
-        close(h1, h2, torch.bfloat16, scale=k * 0.2)
+        for act in ("silu", "gelu_pytorch_tanh"):
+            ops.swiglu_linear(x, wgu, h1, act=act)
+            PlainOps().swiglu_linear(x, wgu, h2, act=act)
+            close(h1, h2, torch.bfloat16, scale=k * 0.2)
 
 
 @pytest.mark.parametrize("m,n,k", [(33, 2048, 5632), (64, 3584, 20480), (100, 300, 512),
@@ -219,6 +241,9 @@ def test_router_align_experts_combine(ops_mode, gen, dtype, t, e, k, h, inner):
     wd = rnd((e, h, inner), dtype, gen, 0.3)
     h1 = torch.zeros(t * k, inner, device="cuda", dtype=dtype)
     h2 = torch.zeros_like(h1)
+    ops.grouped_swiglu(x, wgu, off1, ord1, k, h1, act="gelu_pytorch_tanh")
+    plain.grouped_swiglu(x, wgu, off1, ord1, k, h2, act="gelu_pytorch_tanh")
+    close(h1, h2, dtype, scale=h * 0.3)
     ops.grouped_swiglu(x, wgu, off1, ord1, k, h1)
     plain.grouped_swiglu(x, wgu, off1, ord1, k, h2)
     close(h1, h2, dtype, scale=h * 0.3)
@@ -730,6 +755,38 @@ def test_paged_attention_single_rows_first(ops_mode, gen, dtype, n_q, n_kv, d, p
     ctx.single_rows = len(seqs) + 1
     with pytest.raises(Exception):
         ops.paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, page_size, window, scale, o1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_q,n_kv,d,page_size,window", [
+    (16, 16, 128, 16, 0), (28, 4, 128, 16, 0), (6, 2, 64, 32, 40), (4, 2, 64, 8, 300),
+    (3, 1, 32, 8, 24), (5, 5, 48, 16, 0)])
+def test_paged_attention_with_score_slopes(ops_mode, gen, dtype, n_q, n_kv, d, page_size, window):
+    """A distance-based bias on the scores, slope_h * (key's position - row's): in the plain
+    kernel, the split-context kernels (scalar and grouped heads, where the rows of a block
+    are heads with slopes of their own) and the prompt kernel, alone and in a mixed step."""
+    ops = ops_mode
+    slopes = torch.tensor([2.0 ** -(2 + h % 6) for h in range(n_q)], device="cuda")
+    scale = 1 / math.sqrt(d)
+    cases = [[(700, 1), (15, 1), (255, 1), (0, 37), (390, 300), (64, 64), (9, 2)],     # mixed
+             [(0, 1), (15, 1), (16, 1), (255, 1), (256, 1), (700, 1), (1023, 1), (511, 1)],   # decode
+             [(0, 129), (130, 33), (61, 5)]]                                             # portions
+    for seqs, single in zip(cases, (3, 0, 0)):
+        ctx, qkv, k_pool, v_pool, bt = _attention_case(gen, dtype, seqs, n_q, n_kv, d, page_size, 80)
+        ctx.single_rows = single
+        o1 = torch.zeros(ctx.T, n_q * d, device="cuda", dtype=dtype)
+        o2, o3 = torch.zeros_like(o1), torch.zeros_like(o1)
+        ops.paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, page_size, window, scale, o1,
+                            slopes=slopes)
+        PlainOps().paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, page_size, window,
+                                   scale, o2, slopes=slopes)
+        close(o1, o2, dtype)
+        PlainOps().paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, page_size, window,
+                                   scale, o3)
+        assert (o2.float() - o3.float()).abs().max() > 0.05, "the bias must matter"
+    with pytest.raises(Exception, match="slope"):
+        ops.paged_attention(qkv, k_pool, v_pool, bt, ctx, n_q, n_kv, d, page_size, window, scale, o1,
+                            slopes=slopes[:-1].contiguous() if n_q > 1 else torch.zeros(2, device="cuda"))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

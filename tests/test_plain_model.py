@@ -120,6 +120,30 @@ def test_attention_scale_is_one_over_sqrt_d():
                                torch.softmax(s, -1) @ v[:, 0])
 
 
+def test_attention_score_slopes_are_a_library_mask_of_distances():
+    """A distance-based bias: library attention with the float mask slope_h * (j - i); slope 0
+    is no bias; only distances count (all positions shifted: the same); a steep slope leaves a
+    row its own key (a wrong sign would leave it the farthest)."""
+    t, hq, hkv, d = 9, 4, 2, 16
+    q, k, v = randn(t, hq, d, seed=41), randn(t, hkv, d, seed=42), randn(t, hkv, d, seed=43)
+    pos = torch.arange(t)
+    slopes = [0.5, 0.25, 0.0, 2.0]
+    vis = pm.visibility(pos, pos, None)
+    dist = (pos[None, :] - pos[:, None]).float()
+    mask = torch.stack([s * dist for s in slopes]).masked_fill(~vis, float("-inf"))
+    ref = F.scaled_dot_product_attention(
+        q.transpose(0, 1), k.repeat_interleave(2, 1).transpose(0, 1),
+        v.repeat_interleave(2, 1).transpose(0, 1), attn_mask=mask).transpose(0, 1)
+    got = pm.attention_core(q, k, v, pos, pos, None, slopes)
+    torch.testing.assert_close(got, ref, atol=1e-5, rtol=1e-5)
+    plain = pm.attention_core(q, k, v, pos, pos, None)
+    torch.testing.assert_close(got[:, 2], plain[:, 2])
+    assert (got[:, 0] - plain[:, 0]).abs().max() > 1e-2
+    torch.testing.assert_close(pm.attention_core(q, k, v, pos + 70, pos + 70, None, slopes), got)
+    steep = pm.attention_core(q, k, v, pos, pos, None, [200.0] * hq)
+    torch.testing.assert_close(steep, v.repeat_interleave(2, 1))
+
+
 # ---- router and experts --------------------------------------------------------
 def test_router_equals_library_softmax_topk():
     x, wr = randn(7, 24, seed=16), randn(10, 24, seed=17)
@@ -180,6 +204,21 @@ def test_swiglu_uses_library_silu():
     x = randn(3, 8, seed=34)
     wg, wu, wd = randn(12, 8, seed=35), randn(12, 8, seed=36), randn(8, 12, seed=37)
     torch.testing.assert_close(pm.swiglu_mlp(x, wg, wu, wd), (F.silu(x @ wg.T) * (x @ wu.T)) @ wd.T)
+
+
+def test_gelu_gate_uses_library_gelu():
+    """`hidden_act` = 'gelu_pytorch_tanh': the library's tanh form (the erf form differs from
+    it by up to 5e-4 at these inputs, which the bound would not let through)."""
+    x = randn(5, 8, seed=134) * 2
+    wg, wu, wd = randn(12, 8, seed=135), randn(12, 8, seed=136), randn(8, 12, seed=137)
+    want = (F.gelu(x @ wg.T, approximate="tanh") * (x @ wu.T)) @ wd.T
+    torch.testing.assert_close(pm.swiglu_mlp(x, wg, wu, wd, "gelu_pytorch_tanh"), want)
+    g = torch.linspace(-4, 4, 101)
+    torch.testing.assert_close(pm.gate_activation(g, "gelu_pytorch_tanh"), F.gelu(g, approximate="tanh"),
+                               atol=2e-6, rtol=1e-6)
+    assert (pm.gate_activation(g, "gelu_pytorch_tanh") - F.gelu(g)).abs().max() > 1e-4
+    with pytest.raises(ValueError):
+        pm.gate_activation(g, "relu")
 
 
 def test_shared_expert_gate_zero_is_one_half():

@@ -15,9 +15,9 @@ from typing import Dict, List
 import torch
 
 from ninfer_amd.models.spec import ModelSpec
-from ninfer_amd.parts import (Attention, CacheNeed, FeedForward, LMHead, Mixer, PendingRows,
-                              PoolSpec, PositionEncoding, PreNormBlock, RMSNorm, RoutedExperts,
-                              SwiGLU, TokenEmbedding)
+from ninfer_amd.parts import (Attention, CacheNeed, FeedForward, LMHead, Mixer, NoPosition,
+                              PendingRows, PoolSpec, PositionEncoding, PreNormBlock, RMSNorm,
+                              RoutedExperts, SwiGLU, TokenEmbedding)
 from ninfer_amd.parts.moe import Routing
 from ninfer_amd.registry import register_architecture, register_part
 from ninfer_amd.weights import TensorSpec
@@ -199,17 +199,29 @@ def build_toy_routed(cfg: ToyRoutedConfig) -> ModelSpec:
     blocks = []
     for l in range(c["num_hidden_layers"]):
         p = f"layers.{l}."
-        attn = Attention(p + "attn.", h, c["heads"], c["kv_heads"], c["head_dim"],
-                         HarmonicPosition(c["rot_dim"], c["slope"], c.get("pairing", "half")),
-                         qkv_bias=False,
-                         window=c["window"])
+        if c.get("positions") == "learned+bias":
+            # no rotation: learned absolute positions in the embedding and a distance-based
+            # bias on the scores (head i: slope 2^-(i+1)), both parameters of the framework
+            attn = Attention(p + "attn.", h, c["heads"], c["kv_heads"], c["head_dim"], NoPosition(),
+                             qkv_bias=False, window=c["window"],
+                             score_slopes=[2.0 ** -(i + 1) for i in range(c["heads"])])
+        else:
+            attn = Attention(p + "attn.", h, c["heads"], c["kv_heads"], c["head_dim"],
+                             HarmonicPosition(c["rot_dim"], c["slope"], c.get("pairing", "half")),
+                             qkv_bias=False,
+                             window=c["window"])
         if c.get("router") == "scored":
             ff = ScoredExperts(p + "ff.", h, c["inner"], c["experts"], c["top_k"], c["route_scale"])
         else:
             ff = BiasedSwitch(p + "ff.", h, c["inner"], c["experts"])
         blocks.append(PreNormBlock(RMSNorm(p + "norm1.", h, c["rms_norm_eps"]), attn,
                                    RMSNorm(p + "norm2.", h, c["rms_norm_eps"]), ff))
-    return ModelSpec(TokenEmbedding("embed.", c["vocab_size"], h), blocks,
+    if c.get("positions") == "learned+bias":
+        embedding = TokenEmbedding("embed.", c["vocab_size"], h, positions=c["max_positions"],
+                                   position_prefix="embed_positions.")
+    else:
+        embedding = TokenEmbedding("embed.", c["vocab_size"], h)
+    return ModelSpec(embedding, blocks,
                      RMSNorm("norm.", h, c["rms_norm_eps"]), LMHead("head.", c["vocab_size"], h))
 
 
@@ -225,6 +237,12 @@ TOY_ROUTED_CONFIG = {"architectures": ["ToyRoutedForCausalLM"], "vocab_size": 83
 
 
 TOY_SCORED_CONFIG = dict(TOY_ROUTED_CONFIG, router="scored", top_k=2, route_scale=1.75, experts=6)
+
+# learned absolute positions (a second gather in the embedding) and a distance-based bias on the
+# attention scores instead of a rotation; heads of 64, so that bf16 steps reach the matrix-core
+# attention kernels with the bias
+TOY_BIASED_CONFIG = dict(TOY_ROUTED_CONFIG, positions="learned+bias", max_positions=160, heads=4,
+                         kv_heads=2, head_dim=64, hidden_size=64, window=None)
 
 
 def plain_forward_routed(w: Dict[str, torch.Tensor], c: dict, tokens: List[int]) -> torch.Tensor:
@@ -248,13 +266,18 @@ def plain_forward_routed(w: Dict[str, torch.Tensor], c: dict, tokens: List[int])
         return torch.cat([a * cos - b * sin, a * sin + b * cos, rest], dim=-1)
 
     x = w["embed.weight"][torch.tensor(tokens)].float()
+    slopes = None
+    if c.get("positions") == "learned+bias":
+        x = x + w["embed_positions.weight"][pos].float()
+        slopes = [2.0 ** -(i + 1) for i in range(hq)]
+        turn = lambda v: v   # noqa: E731  (no rotation)
     for l in range(c["num_hidden_layers"]):
         p = f"layers.{l}."
         a = pm.rms_norm(x, w[p + "norm1.weight"], c["rms_norm_eps"])
         q = turn((a @ w[p + "attn.q_proj.weight"].float().T).view(t, hq, d))
         k = turn((a @ w[p + "attn.k_proj.weight"].float().T).view(t, hkv, d))
         v = (a @ w[p + "attn.v_proj.weight"].float().T).view(t, hkv, d)
-        o = pm.attention_core(q, k, v, pos, pos, c["window"]).reshape(t, hq * d)
+        o = pm.attention_core(q, k, v, pos, pos, c["window"], slopes).reshape(t, hq * d)
         x = x + o @ w[p + "attn.o_proj.weight"].float().T
         m = pm.rms_norm(x, w[p + "norm2.weight"], c["rms_norm_eps"])
         y = torch.zeros_like(m)

@@ -298,6 +298,8 @@ def random_config(seed: int) -> dict:
     }
     # (drawn last, so that the configurations of earlier seeds stay what they were)
     lacks = rng.random()
+    if rng.random() < 0.35:
+        cfg["hidden_act"] = "gelu_pytorch_tanh"
     if lacks < 0.15:     # a sparse layer without a shared expert
         del cfg["shared_expert_intermediate_size"]
     elif lacks < 0.22:   # no experts at all: every layer dense
