@@ -62,6 +62,8 @@ static int route_check(const GemmArgs& a, const RouteArgs& rt) {
                  "gemm route: tile lists come together or not at all");
   NINFER_REQUIRE(rt.score == kScoreSoftmax || rt.score == kScoreSigmoid,
                  "gemm route: score function %d is neither softmax (0) nor sigmoid (1)", rt.score);
+  NINFER_REQUIRE(route_groups_ok(rt), "gemm route: %d groups of which %d are open do not fit %d "
+                 "experts and k=%d", rt.n_group, rt.topk_group, rt.E, rt.k);
   return 0;
 }
 

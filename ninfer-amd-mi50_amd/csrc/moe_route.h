@@ -12,7 +12,10 @@ enum RouteScore : int { kScoreSoftmax = 0, kScoreSigmoid = 1 };
 
 // What a router computes from its logits, and where routing writes (all on the device).
 //   s_e = softmax(logits)_e, or sigmoid(logits_e)            (`score`)
-//   chosen = the k experts with the largest s_e + choice_bias_e, ties to the lower index
+//   candidates = all experts, or with `n_group` > 1 those of the `topk_group` groups (of E /
+//            n_group neighbouring experts each) whose largest s_e + choice_bias_e is largest,
+//            ties to the lower group
+//   chosen = the k candidates with the largest s_e + choice_bias_e, ties to the lower index
 //   w_e    = s_e of the chosen (the bias decides the choice only), divided by their sum when
 //            `renorm`, times `scale`
 // Softmax without bias, scale 1: the reference's router (src/ops/moe.hip:65-82), which
@@ -33,7 +36,17 @@ struct RouteArgs {
   int renorm;
   int score;         // RouteScore
   float scale;       // factor on every weight
+  int n_group;       // groups of experts for a group-limited choice (0 or 1: none; at most 64)
+  int topk_group;    // groups whose experts are candidates
 };
+
+// A group-limited choice asks: groups of equal size, at most 64 of them, and enough candidates
+// left for k choices.
+inline bool route_groups_ok(const RouteArgs& rt) {
+  if (rt.n_group <= 1) return rt.n_group >= 0;
+  return rt.n_group <= 64 && rt.E % rt.n_group == 0 && rt.topk_group >= 1 &&
+         rt.topk_group <= rt.n_group && (long)rt.topk_group * (rt.E / rt.n_group) >= rt.k;
+}
 
 constexpr int kMaxExpertsPerLane = 16;  // up to 1024 experts
 // Many rows: the grouping runs as blocks of this many rows side by side (a launch that counts
@@ -93,6 +106,41 @@ __device__ __forceinline__ int route_row(const float* __restrict__ row, const Ro
   bad = __any(bad);
 #pragma unroll
   for (int i = 0; i < NPL; ++i) sel[i] = lane + i * 64 < E ? (bad ? 0.f : sel[i]) : -INFINITY;
+  if (rt.n_group > 1 && rt.topk_group < rt.n_group) {
+    // the groups that may be chosen from: topk_group times the group of the best remaining score
+    const int per_group = E / rt.n_group;
+    unsigned long long open_groups = 0;
+    for (int j = 0; j < rt.topk_group; ++j) {
+      float best = -INFINITY;
+      int best_g = 0x7fffffff;
+#pragma unroll
+      for (int i = 0; i < NPL; ++i) {
+        const int e = lane + i * 64;
+        if (e >= E) continue;
+        const int g = e / per_group;
+        if ((open_groups >> g) & 1ull) continue;
+        if (sel[i] > best || (sel[i] == best && g < best_g)) {
+          best = sel[i];
+          best_g = g;
+        }
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        const float ob = __shfl_xor(best, off, 64);
+        const int og = __shfl_xor(best_g, off, 64);
+        if (ob > best || (ob == best && og < best_g)) {
+          best = ob;
+          best_g = og;
+        }
+      }
+      open_groups |= 1ull << best_g;
+    }
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      const int e = lane + i * 64;
+      if (e < E && !((open_groups >> (e / per_group)) & 1ull)) sel[i] = -INFINITY;
+    }
+  }
   float chosen_sum = 0.f, my_w = 0.f;
   int my_id = 0;
   for (int j = 0; j < k; ++j) {

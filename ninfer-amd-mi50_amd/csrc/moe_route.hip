@@ -140,6 +140,9 @@ static int route_args_check(const char* who, const RouteArgs& rt, int ld) {
   NINFER_REQUIRE(rt.scale == rt.scale && fabsf(rt.scale) < INFINITY, "%s: the scale is not finite",
                  who);
   NINFER_REQUIRE(rt.ids && rt.wts, "%s: no place for the chosen experts and weights", who);
+  NINFER_REQUIRE(route_groups_ok(rt), "%s: %d groups of which %d are open do not fit %d experts and "
+                 "k=%d (equal groups, at most 64, enough candidates)", who, rt.n_group, rt.topk_group,
+                 rt.E, rt.k);
   return 0;
 }
 

@@ -47,7 +47,8 @@ class _RouteArgs(ctypes.Structure):
                 ("tiles_big", ctypes.c_void_p), ("tile_counts", ctypes.c_void_p),
                 ("choice_bias", ctypes.c_void_p), ("parts", ctypes.c_void_p),
                 ("E", ctypes.c_int), ("k", ctypes.c_int), ("renorm", ctypes.c_int),
-                ("score", ctypes.c_int), ("scale", ctypes.c_float)]
+                ("score", ctypes.c_int), ("scale", ctypes.c_float), ("n_group", ctypes.c_int),
+                ("topk_group", ctypes.c_int)]
 
 
 BIG_TILE_ROWS = 256   # rows of a tall tile of the grouped products (the library's kGroupedTileRows)
@@ -618,11 +619,13 @@ class HipOps:
 
     # ---- routing ------------------------------------------------------------------
     def _route_args(self, experts, top_k, renorm, ids, wts, r=None, score="softmax",
-                    choice_bias=None, scale=1.0):
+                    choice_bias=None, scale=1.0, n_group=0, topk_group=0):
         """The router's parameters and the places routing writes, as the library takes them.
         `score`: 'softmax' over all experts or 'sigmoid' of each logit; `choice_bias` [experts]
         is added to the scores for the choice of experts only (the weights are the scores);
-        `scale` multiplies every weight, after the renormalisation if there is one."""
+        `scale` multiplies every weight, after the renormalisation if there is one; with
+        `n_group` > 1 only the experts of the `topk_group` groups (of experts / n_group
+        neighbours each) with the largest best score (+ bias) are candidates."""
         _need(score in _SCORES, f"routing: score {score!r} is not one of {sorted(_SCORES)}")
         _need(1 <= top_k <= experts, f"routing: top_k {top_k} not in [1, {experts}]")
         if choice_bias is not None:
@@ -641,17 +644,18 @@ class HipOps:
                 parts = r.parts.data_ptr()
         args = _RouteArgs(ids.data_ptr(), wts.data_ptr(), offsets, order, t16, t64, tc,
                           _ptr(choice_bias), parts, experts, top_k, 1 if renorm else 0,
-                          _SCORES[score], float(scale))
+                          _SCORES[score], float(scale), int(n_group), int(topk_group))
         return args
 
     def router_topk(self, logits, experts, top_k, renorm, ids, wts, score="softmax",
-                    choice_bias=None, scale=1.0):
+                    choice_bias=None, scale=1.0, n_group=0, topk_group=0):
         _dev(logits, "logits", torch.float32, 2)
         _dev(ids, "ids", torch.int32, 2)
         _dev(wts, "wts", torch.float32, 2)
         t = logits.shape[0]
         _need(ids.shape == (t, top_k) and wts.shape == (t, top_k), "router_topk: output shapes")
-        args = self._route_args(experts, top_k, renorm, ids, wts, None, score, choice_bias, scale)
+        args = self._route_args(experts, top_k, renorm, ids, wts, None, score, choice_bias, scale,
+                                n_group, topk_group)
         self._ok(self.lib.ninfer_router_topk(
             ctypes.c_void_p(logits.data_ptr()), logits.shape[1], t, ctypes.byref(args),
             self._stream()))
@@ -680,7 +684,7 @@ class HipOps:
             ctypes.c_void_p(t16), ctypes.c_void_p(t64), ctypes.c_void_p(tc), self._stream()))
 
     def moe_route(self, logits, experts, top_k, renorm, r, score="softmax", choice_bias=None,
-                  scale=1.0):
+                  scale=1.0, n_group=0, topk_group=0):
         """Scores + top-k per row (see `_route_args` for the router's parameters) and the
         grouping by expert, into the routing record `r` (ids, weights, offsets, order, tile
         lists): one launch for up to 16 rows (one block does both), two for more (top-k by
@@ -698,7 +702,7 @@ class HipOps:
               and r.offsets.shape[0] == experts + 1 and r.order.shape[0] == t * top_k,
               "moe_route: output sizes")
         rargs = self._route_args(experts, top_k, renorm, r.ids, r.weights, r, score, choice_bias,
-                                 scale)
+                                 scale, n_group, topk_group)
         if self._held is not None:
             _need(self._held_route is None, "together(): one routing at most")
             self._held_route = (logits, rargs, (logits, rargs, r, choice_bias))

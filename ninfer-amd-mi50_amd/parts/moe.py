@@ -32,7 +32,8 @@ class TopKRouter(Part):
     architecture's router (reference src/ops/moe.hip:65-82, which always renormalises)."""
 
     def __init__(self, prefix: str, hidden: int, experts: int, top_k: int, renorm: bool,
-                 score: str = "softmax", scale: float = 1.0, choice_bias: bool = False):
+                 score: str = "softmax", scale: float = 1.0, choice_bias: bool = False,
+                 n_group: int = 0, topk_group: int = 0):
         if top_k > experts:
             raise ValueError(f"top_k ({top_k}) exceeds the number of experts ({experts})")
         if score not in ("softmax", "sigmoid"):
@@ -45,6 +46,13 @@ class TopKRouter(Part):
         self.score = score
         self.scale = float(scale)
         self.has_choice_bias = choice_bias
+        # a group-limited choice: only the experts of the topk_group groups (of experts /
+        # n_group neighbours each) whose best score (+ bias) is largest are candidates
+        self.n_group, self.topk_group = int(n_group), int(topk_group)
+        if self.n_group > 1 and (experts % self.n_group or not 1 <= self.topk_group <= self.n_group
+                                 or self.topk_group * (experts // self.n_group) < top_k):
+            raise ValueError(f"{self.n_group} groups of which {self.topk_group} are open do not fit "
+                             f"{experts} experts and top_k {top_k}")
         self.weight: Optional[torch.Tensor] = None
         self.choice_bias: Optional[torch.Tensor] = None
 
@@ -75,7 +83,8 @@ class TopKRouter(Part):
                     tiles_big=ctx.empty((n // Routing.BIG_ROWS + e, 4), torch.int32),
                     tile_counts=ctx.empty((2,), torch.int32))
         ctx.ops.moe_route(logits, e, k, self.renorm, r, score=self.score,
-                          choice_bias=self.choice_bias, scale=self.scale)
+                          choice_bias=self.choice_bias, scale=self.scale, n_group=self.n_group,
+                          topk_group=self.topk_group)
         return r
 
 

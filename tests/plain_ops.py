@@ -154,7 +154,7 @@ class PlainOps:
             out[rows] = (_f(h[off[g]:off[g + 1]]) @ _f(w_down[g]).T).to(out.dtype)
 
     def router_topk(self, logits, experts, top_k, renorm, ids, wts, score="softmax",
-                    choice_bias=None, scale=1.0):
+                    choice_bias=None, scale=1.0, n_group=0, topk_group=0):
         l = logits[:, :experts]
         if score == "sigmoid":
             p = 1 / (1 + torch.exp(-l))
@@ -163,6 +163,14 @@ class PlainOps:
             p = p / p.sum(-1, keepdim=True)
         work = p.clone() if choice_bias is None else p + choice_bias[None, :]
         rows = torch.arange(work.shape[0])
+        if n_group > 1 and topk_group < n_group:
+            # group-limited: the groups by their best score, a stable sort (ties: lower group)
+            per = experts // n_group
+            best_of = work.view(-1, n_group, per).max(-1).values
+            keep = torch.sort(best_of, dim=-1, descending=True, stable=True).indices[:, :topk_group]
+            is_open = torch.zeros_like(best_of, dtype=torch.bool)
+            is_open.scatter_(1, keep, True)
+            work = work.masked_fill(~is_open.repeat_interleave(per, dim=1), -float("inf"))
         for j in range(top_k):
             best = work.max(-1).values
             # lowest index among the maxima
@@ -190,9 +198,9 @@ class PlainOps:
                 tiles.tile_counts[0 if size == 16 else 1] = len(lst)
 
     def moe_route(self, logits, experts, top_k, renorm, r, score="softmax", choice_bias=None,
-                  scale=1.0):
+                  scale=1.0, n_group=0, topk_group=0):
         self.router_topk(logits, experts, top_k, renorm, r.ids, r.weights, score, choice_bias,
-                         scale)
+                         scale, n_group, topk_group)
         self.moe_align(r.ids, experts, r.offsets, r.order, tiles=r)
 
     def paged_attention(self, qkv, k_pool, v_pool, block_table, ctx, n_q, n_kv, head_dim,

@@ -174,6 +174,8 @@ def test_toy_router_with_other_scores(tmp_path):
     ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
     softmax_like = toy.plain_forward_routed(w, dict(cfg, route_scale=1.0), reqs["r1"])
     assert (softmax_like - ref["r1"]).abs().max() > 1e-3, "the scale must matter"
+    ungrouped = toy.plain_forward_routed(w, dict(cfg, n_group=0), reqs["r1"])
+    assert (ungrouped - ref["r1"]).abs().max() > 1e-3, "the groups must matter"
     got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=5, max_live=3))
     for k in reqs:
         torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)

@@ -619,9 +619,47 @@ def test_router_parameters(ops, gen, t, e, k, score):
         assert (got.ids[:, 0] == 5).all()
         s = torch.sigmoid(logits) if score == "sigmoid" else torch.softmax(logits, dim=-1)
         close(got.weights[:, 0], s[:, 5], torch.float32)
+    # a group-limited choice: only experts of the groups with the best scores are candidates
+    for n_group, topk_group in ((4, 2), (2, 1), (e, max(k, 1))):
+        if e % n_group or topk_group * (e // n_group) < k or n_group > 64:
+            continue
+        kw = dict(score=score, choice_bias=bias, scale=1.5, n_group=n_group, topk_group=topk_group)
+        want = record()
+        plain.moe_route(logits, e, k, True, want, **kw)
+        # the definition once more: every chosen expert lies in one of the topk_group groups
+        # whose best biased score is largest, and no better candidate of those groups is left out
+        s = (torch.sigmoid(logits) if score == "sigmoid" else torch.softmax(logits, dim=-1)) + bias
+        per = e // n_group
+        group_best = s.view(t, n_group, per).max(-1).values
+        open_groups = torch.topk(group_best, topk_group, dim=-1).indices
+        for r_ in range(min(t, 48)):
+            chosen = want.ids[r_].long()
+            assert set((chosen // per).tolist()) <= set(open_groups[r_].tolist())
+            cand = torch.cat([torch.arange(g * per, (g + 1) * per, device="cuda") for g in open_groups[r_].tolist()])
+            left = [c for c in cand.tolist() if c not in chosen.tolist()]
+            if left:
+                assert float(s[r_, chosen].min()) >= float(s[r_, left].max())
+        got = record()
+        ops.moe_route(logits, e, k, True, got, **kw)
+        assert torch.equal(got.ids, want.ids) and torch.equal(got.offsets, want.offsets)
+        close(got.weights, want.weights, torch.float32)
+        fused, logits2 = record(), torch.zeros_like(logits)
+        with ops.together():
+            ops.linear(x, w_router, logits2)
+            ops.moe_route(logits2, e, k, True, fused, **kw)
+        want2 = record()
+        plain.moe_route(logits2, e, k, True, want2, **kw)
+        assert torch.equal(fused.ids, want2.ids)
+        close(fused.weights, want2.weights, torch.float32)
+        if topk_group < n_group <= 4 and e >= 60 and t >= 16:
+            free = record()
+            plain.moe_route(logits, e, k, True, free, score=score, choice_bias=bias, scale=1.5)
+            assert not torch.equal(free.ids, want.ids), "the groups must matter"
     from ninfer_amd.kernels import KernelError
     with pytest.raises(KernelError, match="score"):
         ops.moe_route(logits, e, k, False, record(), score="tanh")
+    with pytest.raises(KernelError, match="groups"):
+        ops.moe_route(logits, e, k, False, record(), n_group=e + 1, topk_group=1)
 
 
 def test_router_ties_under_every_score(ops):

@@ -163,16 +163,18 @@ class BiasedSwitch(FeedForward):
 
 class ScoredExperts(FeedForward):
     """Routed experts whose router is not this architecture's: sigmoid scores, a per-expert
-    bias of the checkpoint that decides the choice only, the chosen weights renormalised and
-    scaled. All of it is parameters of the framework's router part and routing kernels; the
-    routing goes with the router's product in one together()."""
+    bias of the checkpoint that decides the choice only, a choice limited to the groups of
+    experts with the best scores, the chosen weights renormalised and scaled. All of it is
+    parameters of the framework's router part and routing kernels; the routing goes with the
+    router's product in one together()."""
 
     def __init__(self, prefix: str, hidden: int, inner: int, experts: int, top_k: int,
-                 scale: float):
+                 scale: float, n_group: int = 0, topk_group: int = 0):
         from ninfer_amd.parts.moe import TopKRouter
         self.prefix = prefix
         self.router = TopKRouter(prefix + "router.", hidden, experts, top_k, renorm=True,
-                                 score="sigmoid", scale=scale, choice_bias=True)
+                                 score="sigmoid", scale=scale, choice_bias=True,
+                                 n_group=n_group, topk_group=topk_group)
         self.experts = RoutedExperts(prefix + "experts.", hidden, inner, experts)
 
     def children(self):
@@ -211,7 +213,8 @@ def build_toy_routed(cfg: ToyRoutedConfig) -> ModelSpec:
                              qkv_bias=False,
                              window=c["window"])
         if c.get("router") == "scored":
-            ff = ScoredExperts(p + "ff.", h, c["inner"], c["experts"], c["top_k"], c["route_scale"])
+            ff = ScoredExperts(p + "ff.", h, c["inner"], c["experts"], c["top_k"], c["route_scale"],
+                               c.get("n_group", 0), c.get("topk_group", 0))
         else:
             ff = BiasedSwitch(p + "ff.", h, c["inner"], c["experts"])
         blocks.append(PreNormBlock(RMSNorm(p + "norm1.", h, c["rms_norm_eps"]), attn,
@@ -236,7 +239,8 @@ TOY_ROUTED_CONFIG = {"architectures": ["ToyRoutedForCausalLM"], "vocab_size": 83
                      "slope": 0.7, "window": 11, "inner": 24, "experts": 5, "rms_norm_eps": 1e-5}
 
 
-TOY_SCORED_CONFIG = dict(TOY_ROUTED_CONFIG, router="scored", top_k=2, route_scale=1.75, experts=6)
+TOY_SCORED_CONFIG = dict(TOY_ROUTED_CONFIG, router="scored", top_k=2, route_scale=1.75, experts=6,
+                         n_group=3, topk_group=1)
 
 # learned absolute positions (a second gather in the embedding) and a distance-based bias on the
 # attention scores instead of a rotation; heads of 64, so that bf16 steps reach the matrix-core
@@ -284,6 +288,13 @@ def plain_forward_routed(w: Dict[str, torch.Tensor], c: dict, tokens: List[int])
         if c.get("router") == "scored":
             score = torch.sigmoid(m @ w[p + "ff.router.weight"].float().T)
             biased = score + w[p + "ff.router.choice_bias"].float()
+            if c.get("n_group", 0) > 1:
+                # only the experts of the topk_group groups with the best biased score are candidates
+                per = c["experts"] // c["n_group"]
+                best_of = biased.view(t, c["n_group"], per).max(-1).values
+                keep = torch.sort(best_of, dim=-1, descending=True, stable=True).indices[:, :c["topk_group"]]
+                is_open = torch.zeros_like(best_of, dtype=torch.bool).scatter_(1, keep, True)
+                biased = biased.masked_fill(~is_open.repeat_interleave(per, dim=1), float("-inf"))
             for r in range(t):
                 # the k largest biased scores (a stable sort: ties to the lower index) choose;
                 # the weights are the plain scores of the chosen, renormalised and scaled
