@@ -231,6 +231,67 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
   }
 }
 
+// The same for query and key heads that are normed before they turn: head vector
+// v = x + bias, v * rsqrt(mean(v^2) + eps) * gain[d] (one gain vector for the query heads, one
+// for the key heads; value heads pass as they are), then the rotation. One wave per (row,
+// head): the head lies in LDS in 32-bit between the norm and the rotation.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_write_normed_kernel(
+    T* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ positions,
+    const int* __restrict__ row_seq, const float* __restrict__ inv_freq, int rot, int Hq, int Hkv,
+    int D, T* __restrict__ kpool, T* __restrict__ vpool, const int* __restrict__ block_table,
+    int bt_stride, int page_size, int write_kv, int interleaved, const float* __restrict__ q_gain,
+    const float* __restrict__ k_gain, float eps) {
+  extern __shared__ float heads_s[];   // [waves][D]
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n_heads = write_kv ? Hq + 2 * Hkv : Hq;
+  const int head = blockIdx.y * (blockDim.x >> 6) + wave;
+  if (head >= n_heads) return;   // (no block-wide barrier below: a wave works alone)
+  float* v = heads_s + wave * D;
+  const int half = rot >> 1;
+  const int W = (Hq + 2 * Hkv) * D;
+  T* row = qkv + (int64_t)t * W;
+  const int pos = positions[t];
+  const bool is_q = head < Hq, is_k = !is_q && head < Hq + Hkv;
+  const int base = head * D;
+  float sq = 0.f;
+  for (int d = lane; d < D; d += 64) {
+    const float x = to_f32(row[base + d]) + (bias ? bias[base + d] : 0.f);
+    v[d] = x;
+    sq += x * x;
+  }
+  const float* gain = is_q ? q_gain : (is_k ? k_gain : nullptr);
+  if (gain) {
+    const float inv = rsqrtf(wave_sum(sq) / (float)D + eps);
+    for (int d = lane; d < D; d += 64) v[d] = v[d] * inv * gain[d];   // each lane its own elements
+  }
+  __builtin_amdgcn_wave_barrier();
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's LDS writes are done before its reads
+  T* dst = row + base;
+  if (!is_q) {
+    const int page = block_table[(int64_t)row_seq[t] * bt_stride + pos / page_size];
+    const int kvh = is_k ? head - Hq : head - Hq - Hkv;
+    dst = (is_k ? kpool : vpool) + (((int64_t)page * Hkv + kvh) * page_size + pos % page_size) * D;
+  }
+  const int per_head = half + (D - rot);
+  for (int i = lane; i < per_head; i += 64) {
+    if (i < half && (is_q || is_k)) {
+      const int d0 = interleaved ? 2 * i : i, d1 = interleaved ? 2 * i + 1 : i + half;
+      float c, s;
+      sincosf((float)pos * inv_freq[i], &s, &c);
+      dst[d0] = from_f32<T>(v[d0] * c - v[d1] * s);
+      dst[d1] = from_f32<T>(v[d0] * s + v[d1] * c);
+    } else if (i < half) {   // a value head: both elements of the pair pass
+      const int d0 = interleaved ? 2 * i : i, d1 = interleaved ? 2 * i + 1 : i + half;
+      dst[d0] = from_f32<T>(v[d0]);
+      dst[d1] = from_f32<T>(v[d1]);
+    } else {
+      const int d0 = rot + (i - half);
+      dst[d0] = from_f32<T>(v[d0]);
+    }
+  }
+}
+
 // Eight consecutive elements at once (16 or 32 bytes).
 __device__ __forceinline__ void load8(const float* p, float* f) {
   const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
@@ -415,14 +476,36 @@ extern "C" int ninfer_rope_kv_write(void* qkv, const float* bias, const int* pos
                                     int Hkv, int D, void* kpool, void* vpool,
                                     const int* block_table, int bt_stride, int page_size,
                                     int write_kv, int interleaved, int T, int dtype,
+                                    const float* q_gain, const float* k_gain, float norm_eps,
                                     hipStream_t stream) {
   NINFER_REQUIRE(T > 0, "rope_kv_write: T=%d must be positive", T);
+  NINFER_REQUIRE((!q_gain) == (!k_gain), "rope_kv_write: the gains of the query heads' and of the key "
+                 "heads' norm come together or not at all");
   NINFER_REQUIRE(D > 0 && D <= 1024, "rope_kv_write: head size %d not in [1,1024]", D);
   NINFER_REQUIRE(rot_dim >= 0 && rot_dim <= D && rot_dim % 2 == 0,
                  "rope_kv_write: rotary size %d must be even and <= head size %d", rot_dim, D);
   NINFER_REQUIRE(rot_dim == 0 || inv_freq, "rope_kv_write: rotary size %d without a table", rot_dim);
   NINFER_REQUIRE(dtype == kF32 || dtype == kBF16, "rope_kv_write: unknown dtype %d", dtype);
   NINFER_REQUIRE(page_size > 0 && bt_stride > 0, "rope_kv_write: bad page size or table width");
+  if (q_gain) {
+    // query and key heads normed before they turn: one wave per (row, head)
+    NINFER_REQUIRE(norm_eps >= 0.f && norm_eps == norm_eps, "rope_kv_write: the norm's eps is not a number >= 0");
+    const int heads = write_kv ? Hq + 2 * Hkv : Hq;
+    const dim3 grid(T, (heads + 3) / 4);
+    const size_t lds = 4 * (size_t)D * sizeof(float);
+    if (dtype == kF32)
+      rope_kv_write_normed_kernel<float><<<grid, 256, lds, stream>>>(
+          (float*)qkv, bias, positions, row_seq, inv_freq, rot_dim, Hq, Hkv, D, (float*)kpool,
+          (float*)vpool, block_table, bt_stride, page_size, write_kv, interleaved, q_gain, k_gain,
+          norm_eps);
+    else
+      rope_kv_write_normed_kernel<bf16><<<grid, 256, lds, stream>>>(
+          (bf16*)qkv, bias, positions, row_seq, inv_freq, rot_dim, Hq, Hkv, D, (bf16*)kpool,
+          (bf16*)vpool, block_table, bt_stride, page_size, write_kv, interleaved, q_gain, k_gain,
+          norm_eps);
+    NINFER_LAUNCH_CHECK();
+    return 0;
+  }
   // many rows of a shape that takes 8-element accesses: one block per row, vectorised
   // (half-split pairs only: neighbouring pairs stay on the kernel of single items)
   const bool vec_ok = !interleaved && (rot_dim / 2) % 8 == 0 && (D - rot_dim) % 8 == 0 && D % 8 == 0 &&

@@ -355,10 +355,14 @@ class HipOps:
         return k, stride
 
     def rope_kv_write(self, qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv, head_dim,
-                      k_pool, v_pool, block_table, page_size, write_kv=True, interleaved=False):
+                      k_pool, v_pool, block_table, page_size, write_kv=True, interleaved=False,
+                      q_norm=None, k_norm=None, norm_eps=0.0):
         """Bias, rotation of q and k, and the write of k and v into pages. Pair i of the
         first `rot_dim` dims of a head turns by pos * inv_freq[i]; the pairs are
-        (i, i + rot_dim / 2), or the neighbours (2i, 2i + 1) when `interleaved`."""
+        (i, i + rot_dim / 2), or the neighbours (2i, 2i + 1) when `interleaved`. `q_norm`,
+        `k_norm` [head_dim] (32-bit gains, both or neither): every query and key head is
+        normed over its dims (x rsqrt(mean(x^2) + norm_eps) gain) after the bias and before it
+        turns."""
         _dev(qkv, "qkv", dims=2)
         t = qkv.shape[0]
         width = (n_q + 2 * n_kv) * head_dim
@@ -378,29 +382,38 @@ class HipOps:
               f"rope_kv_write: pools {tuple(k_pool.shape)} do not fit (kv heads {n_kv}, page "
               f"{page_size}, head {head_dim})")
         _dev(block_table, "block_table", torch.int32, 2)
+        _need((q_norm is None) == (k_norm is None), "rope_kv_write: both heads' norms or neither")
+        if q_norm is not None:
+            _dev(q_norm, "q_norm", torch.float32, 1)
+            _dev(k_norm, "k_norm", torch.float32, 1)
+            _need(q_norm.shape[0] == head_dim and k_norm.shape[0] == head_dim,
+                  "rope_kv_write: a head's norm has one gain per dim of a head")
         self._ok(self.lib.ninfer_rope_kv_write(
             ctypes.c_void_p(qkv.data_ptr()), ctypes.c_void_p(_ptr(bias)),
             ctypes.c_void_p(positions.data_ptr()), ctypes.c_void_p(row_seq.data_ptr()),
             ctypes.c_void_p(_ptr(inv_freq) if rot_dim else None), rot_dim, n_q, n_kv, head_dim,
             ctypes.c_void_p(k_pool.data_ptr()), ctypes.c_void_p(v_pool.data_ptr()),
             ctypes.c_void_p(block_table.data_ptr()), block_table.shape[1], page_size,
-            1 if write_kv else 0, 1 if interleaved else 0, t, _DT[qkv.dtype], self._stream()))
+            1 if write_kv else 0, 1 if interleaved else 0, t, _DT[qkv.dtype],
+            ctypes.c_void_p(_ptr(q_norm)), ctypes.c_void_p(_ptr(k_norm)), ctypes.c_float(norm_eps),
+            self._stream()))
 
     def qkv_rope(self, x, w_qkv, bias, qkv, positions, row_seq, inv_freq, rot_dim, n_q, n_kv,
                  head_dim, k_pool, v_pool, block_table, page_size, write_kv=True,
-                 interleaved=False):
+                 interleaved=False, q_norm=None, k_norm=None, norm_eps=0.0):
         """qkv = x w_qkv^T, then what `rope_kv_write` does. Few bf16 rows with a full
-        rotation in half-split pairs run as one kernel; everything else as the product
-        and the rotation kernel one after the other."""
+        rotation in half-split pairs and no norm of the heads run as one kernel (its blocks
+        hold parts of heads); everything else as the product and the rotation kernel one after
+        the other."""
         t = x.shape[0]
         fused = (not self.force_generic and not interleaved and x.dtype == torch.bfloat16
-                 and x.dim() == 2
+                 and x.dim() == 2 and q_norm is None
                  and self.lib.ninfer_qkv_rope_takes(t, x.shape[1], x.shape[1], head_dim, rot_dim))
         if not fused:
             self.linear(x, w_qkv, qkv)
             self.rope_kv_write(qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv,
                                head_dim, k_pool, v_pool, block_table, page_size, write_kv,
-                               interleaved)
+                               interleaved, q_norm, k_norm, norm_eps)
             return
         width = (n_q + 2 * n_kv) * head_dim
         _dev(x, "x", torch.bfloat16, 2)

@@ -25,11 +25,14 @@ class Attention(Mixer):
     def __init__(self, prefix: str, hidden: int, heads: int, kv_heads: int, head_dim: int,
                  position: PositionEncoding, qkv_bias: bool = True,
                  window: Optional[int] = None, scale: Optional[float] = None,
-                 score_slopes: Optional[Sequence[float]] = None):
+                 score_slopes: Optional[Sequence[float]] = None,
+                 qk_norm_eps: Optional[float] = None):
         """`score_slopes` [heads]: a distance-based position bias, slope * (key's position -
         query's position) added to head h's scaled scores before the softmax (None: none).
         It is a parameter of the attention kernels, beside or instead of the rotation that
-        `position` describes."""
+        `position` describes. `qk_norm_eps`: every query and key head is normed over its dims
+        (x rsqrt(mean(x^2) + eps) gain, gains `q_norm.weight` and `k_norm.weight` [head_dim] of the
+        checkpoint) after the bias and before it turns; None: no such norm."""
         if heads % kv_heads:
             raise ValueError(f"heads ({heads}) must be a multiple of kv_heads ({kv_heads})")
         if score_slopes is not None and len(score_slopes) != heads:
@@ -45,6 +48,9 @@ class Attention(Mixer):
         self.scale = scale if scale is not None else 1.0 / math.sqrt(head_dim)
         self.score_slopes = None if score_slopes is None else [float(x) for x in score_slopes]
         self.slopes: Optional[torch.Tensor] = None   # the same on the device (32-bit)
+        self.qk_norm_eps = qk_norm_eps
+        self.q_norm: Optional[torch.Tensor] = None
+        self.k_norm: Optional[torch.Tensor] = None
         self.w_qkv: Optional[torch.Tensor] = None
         self.b_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
@@ -71,6 +77,9 @@ class Attention(Mixer):
             specs[p + "q_proj.bias"] = TensorSpec((self.heads * d,), "bias")
             specs[p + "k_proj.bias"] = TensorSpec((self.kv_heads * d,), "bias")
             specs[p + "v_proj.bias"] = TensorSpec((self.kv_heads * d,), "bias")
+        if self.qk_norm_eps is not None:
+            specs[p + "q_norm.weight"] = TensorSpec((d,), "gain")
+            specs[p + "k_norm.weight"] = TensorSpec((d,), "gain")
         return specs
 
     def unused_tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -84,6 +93,9 @@ class Attention(Mixer):
         nq, nk = self.heads * d, self.kv_heads * d
         if self.score_slopes is not None:
             self.slopes = torch.tensor(self.score_slopes, dtype=torch.float32, device=w.device)
+        if self.qk_norm_eps is not None:
+            self.q_norm = w.float32(p + "q_norm.weight")
+            self.k_norm = w.float32(p + "k_norm.weight")
         self.w_qkv = torch.empty((self.qkv_width, self.hidden), dtype=w.act_dtype, device=w.device)
         w.matrix_into(p + "q_proj.weight", self.w_qkv[:nq])
         w.matrix_into(p + "k_proj.weight", self.w_qkv[nq:nq + nk])
@@ -105,7 +117,8 @@ class Attention(Mixer):
                      self.position.table(), self.position.rot_dim, self.heads, self.kv_heads,
                      self.head_dim, cache["k"], cache["v"], cache.block_table,
                      cache.page_size, write_kv=call.writes_cache,
-                     interleaved=self.position.pairing == "interleaved")
+                     interleaved=self.position.pairing == "interleaved",
+                     q_norm=self.q_norm, k_norm=self.k_norm, norm_eps=self.qk_norm_eps or 0.0)
         attn = ctx.empty((ctx.T, self.heads * self.head_dim))
         ops.paged_attention(qkv, cache["k"], cache["v"], cache.block_table, ctx,
                             self.heads, self.kv_heads, self.head_dim,

@@ -68,18 +68,24 @@ class PlainOps:
 
     def qkv_rope(self, x, w_qkv, bias, qkv, positions, row_seq, inv_freq, rot_dim, n_q, n_kv,
                  head_dim, k_pool, v_pool, block_table, page_size, write_kv=True,
-                 interleaved=False):
+                 interleaved=False, q_norm=None, k_norm=None, norm_eps=0.0):
         self.linear(x, w_qkv, qkv)
         self.rope_kv_write(qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv, head_dim,
-                           k_pool, v_pool, block_table, page_size, write_kv, interleaved)
+                           k_pool, v_pool, block_table, page_size, write_kv, interleaved,
+                           q_norm, k_norm, norm_eps)
 
     def rope_kv_write(self, qkv, bias, positions, row_seq, inv_freq, rot_dim, n_q, n_kv, head_dim,
-                      k_pool, v_pool, block_table, page_size, write_kv=True, interleaved=False):
+                      k_pool, v_pool, block_table, page_size, write_kv=True, interleaved=False,
+                      q_norm=None, k_norm=None, norm_eps=0.0):
         t = qkv.shape[0]
         x = _f(qkv)
         if bias is not None:
             x = x + bias
         x = x.view(t, n_q + 2 * n_kv, head_dim).clone()
+        if q_norm is not None:   # query and key heads normed over their dims before they turn
+            for lo, hi, gain in ((0, n_q, q_norm), (n_q, n_q + n_kv, k_norm)):
+                part = x[:, lo:hi]
+                x[:, lo:hi] = part * torch.rsqrt((part * part).mean(-1, keepdim=True) + norm_eps) * gain
         if rot_dim:
             half = rot_dim // 2
             phi = positions.to(torch.float32)[:, None] * inv_freq[None, :]

@@ -207,6 +207,27 @@ def test_toy_learned_positions_and_score_bias(tmp_path):
                                     page_size=4), ops=PlainOps())
 
 
+def test_toy_normed_query_and_key_heads(tmp_path):
+    """Attention whose query and key heads are normed over their dims before they turn: a
+    parameter of the attention part (two gain vectors of the checkpoint) and of the rotation's
+    kernel."""
+    import ninfer_amd
+    toy.register_routed()
+    cfg = toy.TOY_QK_NORM_CONFIG
+    d = str(tmp_path / "toy_qk_norm")
+    ninfer_amd.write_random_model(d, cfg, 15, std=0.3)
+    _, w = util.read_folder(d)
+    assert w["layers.0.attn.q_norm.weight"].shape == (16,)
+    runner = runner_for(d, seqs=3)
+    reqs = {f"r{i}": util.random_tokens(n, 83, 80 + i) for i, n in enumerate([7, 26, 15])}
+    ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
+    plain = toy.plain_forward_routed(w, dict(cfg, qk_norm_eps=None), reqs["r1"])
+    assert (plain - ref["r1"]).abs().max() > 1e-3, "the heads' norm must matter"
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=9, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+
+
 def test_toy_interleaved_pairs(tmp_path):
     """The second toy with neighbouring dims as rotation pairs: the pairing is a property of
     the position encoding that attention hands to the rotation, nothing else changes."""

@@ -315,6 +315,37 @@ def test_toy_learned_positions_and_score_bias_on_the_gpu(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_normed_query_and_key_heads_on_the_gpu(tmp_path, dtype):
+    """Query and key heads normed over their dims before the rotation, in the rotation's kernel
+    (one wave per row and head), prompts in portions beside decoded tokens."""
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, load_model
+    toy.register_routed()
+    cfg = toy.TOY_QK_NORM_CONFIG
+    d = str(tmp_path / "toy_qk_norm")
+    ninfer_amd.write_random_model(d, cfg, 15, dtype=dtype, std=0.3)
+    _, w = util.read_folder(d)
+    runner = load_model(d, EngineOptions(dtype=dtype, max_context=64, num_sequences=3, page_size=4,
+                                         check_pages=True))
+    reqs = {f"r{i}": util.random_tokens(n, 83, 80 + i) for i, n in enumerate([7, 26, 15, 33])}
+    ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=9, max_live=3))
+    tail = util.run_schedule(runner, util.schedule_tail("r3", reqs["r3"], 12))["r3"]
+    if dtype == "float32":
+        for k in reqs:
+            torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+        torch.testing.assert_close(tail, ref["r3"], atol=3e-5, rtol=1e-4)
+    else:
+        # (one expert per token: a row that routes otherwise is far off, so the typical row is
+        # what is bounded in bfloat16, against the model without the norm too)
+        other = toy.plain_forward_routed(w, dict(cfg, qk_norm_eps=None), reqs["r3"])
+        err = (tail - ref["r3"]).abs().max(-1).values
+        wrong = (tail - other).abs().max(-1).values
+        assert float(err.median()) < float(wrong.median()) / 3
+        assert float(err.median()) < 0.03 * float(ref["r3"].abs().max())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_toy_interleaved_pairs_on_the_gpu(tmp_path, dtype):
     """Neighbouring dims as rotation pairs (a partial rotation of 12 of 16 dims), chosen by
     the position encoding alone: the rotation kernel takes the pairing as a parameter."""

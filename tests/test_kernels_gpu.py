@@ -923,6 +923,25 @@ def test_rope_kv_write(ops, gen, dtype, n_q, n_kv, d, rot, seqs):
         close(v1, v2, dtype, scale=4)
         if not write:
             assert torch.equal(k1, k_pool) and torch.equal(v1, v_pool)
+    # query and key heads normed over their dims before they turn (the value heads are not)
+    qg, kg = torch.rand(d, generator=gen, device="cuda") + 0.5, torch.rand(d, generator=gen, device="cuda") + 0.5
+    for b, write, inter in ((bias, True, False), (None, True, True), (bias, False, False)):
+        q1, q2 = qkv.clone(), qkv.clone()
+        k1, k2, v1, v2 = k_pool.clone(), k_pool.clone(), v_pool.clone(), v_pool.clone()
+        kw = dict(write_kv=write, interleaved=inter, q_norm=qg, k_norm=kg, norm_eps=1e-5)
+        ops.rope_kv_write(q1, b, ctx.positions, ctx.row_seq, table, rot, n_q, n_kv, d, k1, v1, bt, ps, **kw)
+        PlainOps().rope_kv_write(q2, b, ctx.positions, ctx.row_seq, table, rot, n_q, n_kv, d, k2, v2,
+                                 bt, ps, **kw)
+        close(q1[:, :n_q * d], q2[:, :n_q * d], dtype, scale=4)
+        close(k1, k2, dtype, scale=4)
+        close(v1, v2, dtype, scale=4)
+        if write:   # normed: a key's mean square is about the gain's; a value's is what it was
+            page = bt[ctx.row_seq.long()[0], ctx.positions.long()[0] // ps].long()
+            written = k1[page, :, ctx.positions.long()[0] % ps, :].float()
+            assert 0.3 < float((written ** 2).mean()) < 3.0
+    with pytest.raises(Exception, match="neither"):
+        ops.rope_kv_write(qkv.clone(), None, ctx.positions, ctx.row_seq, table, rot, n_q, n_kv, d,
+                          k_pool.clone(), v_pool.clone(), bt, ps, q_norm=qg)
     if rot:   # the pairing matters, and the twin's pairs are the neighbours: one dim set alone
         one = torch.zeros_like(qkv[:1])
         one[0, 0] = 1.0

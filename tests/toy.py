@@ -211,7 +211,7 @@ def build_toy_routed(cfg: ToyRoutedConfig) -> ModelSpec:
             attn = Attention(p + "attn.", h, c["heads"], c["kv_heads"], c["head_dim"],
                              HarmonicPosition(c["rot_dim"], c["slope"], c.get("pairing", "half")),
                              qkv_bias=False,
-                             window=c["window"])
+                             window=c["window"], qk_norm_eps=c.get("qk_norm_eps"))
         if c.get("router") == "scored":
             ff = ScoredExperts(p + "ff.", h, c["inner"], c["experts"], c["top_k"], c["route_scale"],
                                c.get("n_group", 0), c.get("topk_group", 0))
@@ -241,6 +241,9 @@ TOY_ROUTED_CONFIG = {"architectures": ["ToyRoutedForCausalLM"], "vocab_size": 83
 
 TOY_SCORED_CONFIG = dict(TOY_ROUTED_CONFIG, router="scored", top_k=2, route_scale=1.75, experts=6,
                          n_group=3, topk_group=1)
+
+# every query and key head normed over its dims before the rotation
+TOY_QK_NORM_CONFIG = dict(TOY_ROUTED_CONFIG, qk_norm_eps=1e-5)
 
 # learned absolute positions (a second gather in the embedding) and a distance-based bias on the
 # attention scores instead of a rotation; heads of 64, so that bf16 steps reach the matrix-core
@@ -278,8 +281,12 @@ def plain_forward_routed(w: Dict[str, torch.Tensor], c: dict, tokens: List[int])
     for l in range(c["num_hidden_layers"]):
         p = f"layers.{l}."
         a = pm.rms_norm(x, w[p + "norm1.weight"], c["rms_norm_eps"])
-        q = turn((a @ w[p + "attn.q_proj.weight"].float().T).view(t, hq, d))
-        k = turn((a @ w[p + "attn.k_proj.weight"].float().T).view(t, hkv, d))
+        q = (a @ w[p + "attn.q_proj.weight"].float().T).view(t, hq, d)
+        k = (a @ w[p + "attn.k_proj.weight"].float().T).view(t, hkv, d)
+        if c.get("qk_norm_eps") is not None:   # every head normed over its dims before it turns
+            q = pm.rms_norm(q, w[p + "attn.q_norm.weight"], c["qk_norm_eps"])
+            k = pm.rms_norm(k, w[p + "attn.k_norm.weight"], c["qk_norm_eps"])
+        q, k = turn(q), turn(k)
         v = (a @ w[p + "attn.v_proj.weight"].float().T).view(t, hkv, d)
         o = pm.attention_core(q, k, v, pos, pos, c["window"], slopes).reshape(t, hq * d)
         x = x + o @ w[p + "attn.o_proj.weight"].float().T
