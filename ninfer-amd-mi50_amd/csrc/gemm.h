@@ -21,7 +21,7 @@ struct GemmArgs {
   const void* A;         // [rows, lda] activations
   const void* W;         // [groups, N (2N with a gated epilogue), K] weights
   void* C;               // [rows, ldc]
-  const float* bias;     // [N] or null
+  const float* bias;     // [N] ([2N] with a gated epilogue: the gate's, then the other half's) or null
   const int* offsets;    // [groups + 1] sorted-row ranges per group, or null (dense)
   const int* a_index;    // sorted row -> a_index[r] / a_div is the row of A, or null
   const int* c_index;    // sorted row -> row of C, or null

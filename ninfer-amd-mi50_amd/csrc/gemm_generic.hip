@@ -108,8 +108,9 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs a) {
       if (n >= a.N) continue;
       float v = acc[i][j];
       if (SWIGLU) {
-        float g = v;
-        v = g / (1.f + expf(-gate_logit(g, a.epilogue == kEpilogueGeGLU))) * accu[i][j];
+        float g = v + (a.bias ? a.bias[n] : 0.f);
+        const float u = accu[i][j] + (a.bias ? a.bias[a.N + n] : 0.f);
+        v = g / (1.f + expf(-gate_logit(g, a.epilogue == kEpilogueGeGLU))) * u;
       } else if (a.bias) {
         v += a.bias[n];
       }
@@ -144,7 +145,8 @@ int gemm_check(const GemmArgs& a) {
   NINFER_REQUIRE(!a.a_index || a.a_div >= 1, "gemm: a_div=%d must be >= 1", a.a_div);
   NINFER_REQUIRE(a.epilogue == kEpilogueNone || epilogue_gated(a.epilogue),
                  "gemm: unknown epilogue %d", a.epilogue);
-  NINFER_REQUIRE(!(epilogue_gated(a.epilogue) && a.bias), "gemm: a gated epilogue takes no bias");
+  NINFER_REQUIRE(!(epilogue_gated(a.epilogue) && a.bias && a.offsets),
+                 "gemm: a grouped product with a gated epilogue takes no bias");
   NINFER_REQUIRE(a.k_parts <= 1, "gemm: k_parts is set by the library, not by callers");
   NINFER_REQUIRE(!a.workspace || a.workspace_floats > 0, "gemm: a workspace of %ld floats",
                  (long)a.workspace_floats);

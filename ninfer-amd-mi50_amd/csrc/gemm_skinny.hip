@@ -210,7 +210,12 @@ __device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, in
         if (col >= a.N) break;
         float v = sum[fg * HALVES];
         if (SWIGLU) {
-          v = v / (1.f + __expf(-gate_logit(v, a.epilogue == kEpilogueGeGLU))) * sum[fg * HALVES + (SWIGLU ? 1 : 0)];
+          float u = sum[fg * HALVES + (SWIGLU ? 1 : 0)];
+          if (a.bias) {
+            v += a.bias[col];
+            u += a.bias[a.N + col];
+          }
+          v = v / (1.f + __expf(-gate_logit(v, a.epilogue == kEpilogueGeGLU))) * u;
         } else if (a.bias) {
           v += a.bias[col];
         }

@@ -128,7 +128,11 @@ __device__ inline void write_accumulators(const GemmArgs& a, const f32x16 (&acc)
           float v[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float g = acc[i][jj][4 * q + r], u = acc[i + (SWIGLU ? FI / 2 : 0)][jj][4 * q + r];
+            float g = acc[i][jj][4 * q + r], u = acc[i + (SWIGLU ? FI / 2 : 0)][jj][4 * q + r];
+            if (a.bias && f0 + r < N) {
+              g += a.bias[f0 + r];
+              u += a.bias[N + f0 + r];
+            }
             v[r] = gated_times(g, u, gelu);
           }
           if (whole_quads) {
@@ -192,9 +196,19 @@ __device__ inline void write_accumulators_staged(const GemmArgs& a, const f32x16
       for (int q = 0; q < 4; ++q) {
         bf16x4 val;
         if (SWIGLU) {
+          float bg[4] = {0.f, 0.f, 0.f, 0.f}, bu[4] = {0.f, 0.f, 0.f, 0.f};
+          const int f = feat0 + 32 * i + 8 * q + 4 * lk;
+          if (a.bias && f < N) {   // N % 4 == 0: four features are in or out together
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              bg[r] = a.bias[f + r];
+              bu[r] = a.bias[N + f + r];
+            }
+          }
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float g = acc[i][jj][4 * q + r], u = acc[i + (SWIGLU ? FI / 2 : 0)][jj][4 * q + r];
+            const float g = acc[i][jj][4 * q + r] + bg[r];
+            const float u = acc[i + (SWIGLU ? FI / 2 : 0)][jj][4 * q + r] + bu[r];
             val[r] = (__bf16)gated_times(g, u, gelu);
           }
         } else {

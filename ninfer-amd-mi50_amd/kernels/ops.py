@@ -586,17 +586,20 @@ class HipOps:
         _need(act in GATE_ACTS, f"gated product: activation {act!r} is not one of {sorted(GATE_ACTS)}")
         return GATE_ACTS[act]
 
-    def swiglu_linear(self, x, w_gate_up, out, act="silu"):
-        """out = act(x Wg^T) * (x Wu^T), Wg = rows [0, I), Wu = rows [I, 2I); act is SiLU or
-        the tanh form of GELU (`GATE_ACTS`)."""
+    def swiglu_linear(self, x, w_gate_up, out, act="silu", bias=None):
+        """out = act(x Wg^T [+ bg]) * (x Wu^T [+ bu]), Wg = rows [0, I), Wu = rows [I, 2I); act
+        is SiLU or the tanh form of GELU (`GATE_ACTS`); `bias` [2I] (32-bit) holds bg, then bu."""
         _dev(x, "x", dims=2)
         _dev(w_gate_up, "w_gate_up", x.dtype, 2)
         _dev(out, "out", x.dtype, 2)
         inner = w_gate_up.shape[0] // 2
         _need(w_gate_up.shape == (2 * inner, x.shape[1]), "swiglu_linear: weight shape")
         _need(out.shape == (x.shape[0], inner), "swiglu_linear: out has the wrong shape")
+        if bias is not None:
+            _dev(bias, "bias", torch.float32, 1)
+            _need(bias.shape[0] == 2 * inner, "swiglu_linear: bias has the wrong size")
         self._gemm(x, w_gate_up, out, m=x.shape[0], n=inner, k=x.shape[1],
-                   epilogue=self._gate_epilogue(act))
+                   epilogue=self._gate_epilogue(act), bias=bias)
 
     def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None, act="silu"):
         """out[r] = the gated product (see `swiglu_linear`) of row order[r] // top_k of x by

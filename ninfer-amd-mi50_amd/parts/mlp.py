@@ -18,19 +18,27 @@ from .base import FeedForward, StepContext, WeightBinder
 
 
 class SwiGLU(FeedForward):
-    def __init__(self, prefix: str, hidden: int, inner: int, act: str = "silu"):
+    def __init__(self, prefix: str, hidden: int, inner: int, act: str = "silu", bias: bool = False):
         self.prefix = prefix
         self.hidden = hidden
         self.inner = inner
         self.act = act   # the gate's activation, by config.json's name: 'silu' | 'gelu_pytorch_tanh'
+        self.bias = bias   # gate_proj.bias, up_proj.bias [inner] and down_proj.bias [hidden] are read
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
+        self.b_gate_up: Optional[torch.Tensor] = None
+        self.b_down: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         p = self.prefix
-        return {p + "gate_proj.weight": TensorSpec((self.inner, self.hidden)),
-                p + "up_proj.weight": TensorSpec((self.inner, self.hidden)),
-                p + "down_proj.weight": TensorSpec((self.hidden, self.inner))}
+        specs = {p + "gate_proj.weight": TensorSpec((self.inner, self.hidden)),
+                 p + "up_proj.weight": TensorSpec((self.inner, self.hidden)),
+                 p + "down_proj.weight": TensorSpec((self.hidden, self.inner))}
+        if self.bias:
+            specs[p + "gate_proj.bias"] = TensorSpec((self.inner,), "bias")
+            specs[p + "up_proj.bias"] = TensorSpec((self.inner,), "bias")
+            specs[p + "down_proj.bias"] = TensorSpec((self.hidden,), "bias")
+        return specs
 
     def bind(self, w: WeightBinder) -> None:
         p = self.prefix
@@ -39,15 +47,20 @@ class SwiGLU(FeedForward):
         w.matrix_into(p + "gate_proj.weight", self.w_gate_up[:self.inner])
         w.matrix_into(p + "up_proj.weight", self.w_gate_up[self.inner:])
         self.w_down = w.matrix(p + "down_proj.weight")
+        if self.bias:
+            self.b_gate_up = torch.cat([w.float32(p + "gate_proj.bias"), w.float32(p + "up_proj.bias")])
+            w.hold(p + "gate_proj.bias", self.b_gate_up[:self.inner])
+            w.hold(p + "up_proj.bias", self.b_gate_up[self.inner:])
+            self.b_down = w.float32(p + "down_proj.bias")
 
     def gate_up(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
         h = ctx.empty((x.shape[0], self.inner))
-        ctx.ops.swiglu_linear(x, self.w_gate_up, h, act=self.act)
+        ctx.ops.swiglu_linear(x, self.w_gate_up, h, act=self.act, bias=self.b_gate_up)
         return h
 
     def down(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         out = ctx.empty((h.shape[0], self.hidden))
-        ctx.ops.linear(h, self.w_down, out)
+        ctx.ops.linear(h, self.w_down, out, bias=self.b_down)
         return out
 
     def run(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:

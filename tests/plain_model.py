@@ -142,14 +142,19 @@ def gate_activation(g: Tensor, act: str) -> Tensor:
     raise ValueError(f"hidden_act {act!r}")
 
 
-def swiglu_mlp(x: Tensor, wg: Tensor, wu: Tensor, wd: Tensor, act: str = "silu") -> Tensor:
-    """(act(x Wg^T) * (x Wu^T)) Wd^T.
+def swiglu_mlp(x: Tensor, wg: Tensor, wu: Tensor, wd: Tensor, act: str = "silu",
+               biases: Optional[Tuple[Tensor, Tensor, Tensor]] = None) -> Tensor:
+    """(act(x Wg^T) * (x Wu^T)) Wd^T; with `biases` (the gate's, the other half's, the down
+    product's; the reference has none) each product gets its own added.
 
     Reference: src/ops/kernels.hip:131-140, src/models/model.hip:313-337.
     """
     g = x @ wg.float().T
     u = x @ wu.float().T
-    return (gate_activation(g, act) * u) @ wd.float().T
+    if biases is not None:
+        g, u = g + biases[0].float(), u + biases[1].float()
+    y = (gate_activation(g, act) * u) @ wd.float().T
+    return y if biases is None else y + biases[2].float()
 
 
 def router(x: Tensor, wr: Tensor, top_k: int, renorm: bool) -> Tuple[Tensor, Tensor]:

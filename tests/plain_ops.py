@@ -131,10 +131,12 @@ class PlainOps:
         assert act == "gelu_pytorch_tanh", act
         return 0.5 * g * (1 + torch.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g ** 3)))
 
-    def swiglu_linear(self, x, w_gate_up, out, act="silu"):
+    def swiglu_linear(self, x, w_gate_up, out, act="silu", bias=None):
         inner = w_gate_up.shape[0] // 2
         g = _f(x) @ _f(w_gate_up[:inner]).T
         u = _f(x) @ _f(w_gate_up[inner:]).T
+        if bias is not None:
+            g, u = g + bias[:inner], u + bias[inner:]
         out.copy_((self._act(g, act) * u).to(out.dtype))
 
     def grouped_swiglu(self, x, w_gate_up, offsets, order, top_k, out, tiles=None, act="silu"):

@@ -134,6 +134,26 @@ def test_toy_mixer_with_state_of_its_own(tmp_path):
         torch.testing.assert_close(got[k], ref[k], atol=2e-5, rtol=1e-4)
 
 
+def test_toy_feed_forward_with_biases_and_another_activation(tmp_path):
+    """The dense feed-forward with the tanh form of GELU as its gate's activation and a bias on
+    each of its three products: parameters of the framework's part."""
+    import ninfer_amd
+    toy.register()
+    cfg = toy.TOY_BIASED_MLP_CONFIG
+    d = str(tmp_path / "toy_biased_mlp")
+    ninfer_amd.write_random_model(d, cfg, 6, std=0.2)
+    _, w = util.read_folder(d)
+    assert w["layers.1.mlp.up_proj.bias"].shape == (56,) and w["layers.0.mlp.down_proj.bias"].shape == (40,)
+    runner = runner_for(d, seqs=3)
+    reqs = {f"t{i}": util.random_tokens(n, 97, 90 + i) for i, n in enumerate([9, 21, 14])}
+    ref = {k: toy.plain_forward(w, cfg, v) for k, v in reqs.items()}
+    assert (toy.plain_forward(w, dict(cfg, mlp_bias=False), reqs["t1"]) - ref["t1"]).abs().max() > 1e-3
+    assert (toy.plain_forward(w, dict(cfg, hidden_act="silu"), reqs["t1"]) - ref["t1"]).abs().max() > 1e-3
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=3, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=2e-5, rtol=1e-4)
+
+
 def test_toy_routed_feed_forward_and_another_position_encoding(tmp_path):
     """A feed-forward with routing of its own (a router bias from the checkpoint,
     one expert per token) and a position encoding with other angles and a

@@ -217,6 +217,35 @@ def test_toy_mixer_on_the_gpu(tmp_path):
         torch.testing.assert_close(got[k], ref[k], atol=2e-5, rtol=1e-4)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_feed_forward_with_biases_and_another_activation_on_the_gpu(tmp_path, dtype):
+    """A dense feed-forward with GELU's tanh form as the gate's activation and a bias on each of
+    its three products, on the product kernels' epilogues (few rows and portions)."""
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, load_model
+    toy.register()
+    cfg = toy.TOY_BIASED_MLP_CONFIG
+    d = str(tmp_path / "toy_biased_mlp")
+    ninfer_amd.write_random_model(d, cfg, 6, dtype=dtype, std=0.2)
+    _, w = util.read_folder(d)
+    runner = load_model(d, EngineOptions(dtype=dtype, max_context=64, num_sequences=3))
+    reqs = {f"t{i}": util.random_tokens(n, 97, 90 + i) for i, n in enumerate([9, 21, 14, 50])}
+    ref = {k: toy.plain_forward(w, cfg, v) for k, v in reqs.items()}
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=3, max_live=3))
+    whole = util.run_schedule(runner, util.schedule_whole("t3", reqs["t3"]))["t3"]
+    for k in reqs:
+        if dtype == "float32":
+            torch.testing.assert_close(got[k], ref[k], atol=2e-5, rtol=1e-4)
+        else:
+            assert float((got[k] - ref[k]).abs().max()) < 0.04 * float(ref[k].abs().max())
+    if dtype == "float32":
+        torch.testing.assert_close(whole, ref["t3"], atol=2e-5, rtol=1e-4)
+    else:
+        assert float((whole - ref["t3"]).abs().max()) < 0.04 * float(ref["t3"].abs().max())
+        no_bias = toy.plain_forward(w, dict(cfg, mlp_bias=False), reqs["t3"])
+        assert float((whole - ref["t3"]).abs().max()) < float((whole - no_bias).abs().max()) / 3
+
+
 def test_toy_routed_feed_forward_and_position_on_the_gpu(tmp_path):
     """The second toy (a routed feed-forward with a router bias, another position
     encoding with a partial rotation, a window) on the kernels, 32-bit."""

@@ -120,13 +120,14 @@ def test_swiglu_linear(ops_mode, gen, dtype, m, inner, k):
     is written with tanh where the kernels use a sigmoid of twice the argument)."""
     ops = ops_mode
     x, w = rnd((m, k), dtype, gen), rnd((2 * inner, k), dtype, gen, 0.3)
-    for act in ("silu", "gelu_pytorch_tanh"):
+    bias = torch.randn(2 * inner, generator=gen, device="cuda")
+    for act, b in (("silu", None), ("gelu_pytorch_tanh", None), ("silu", bias), ("gelu_pytorch_tanh", bias)):
         o1 = torch.empty(m, inner, device="cuda", dtype=dtype)
         o2 = torch.empty_like(o1)
-        ops.swiglu_linear(x, w, o1, act=act)
-        PlainOps().swiglu_linear(x, w, o2, act=act)
+        ops.swiglu_linear(x, w, o1, act=act, bias=b)
+        PlainOps().swiglu_linear(x, w, o2, act=act, bias=b)
         close(o1, o2, dtype, scale=k * 0.3)
-    if k == 64:   # the two activations are told apart
+    if k == 64:   # the activations and the bias are told apart
         assert (o1.float() - ops_out(ops, x, w, inner, dtype)).abs().max() > 1e-2
     with pytest.raises(Exception, match="activation"):
         ops.swiglu_linear(x, w, o1, act="relu")
@@ -156,9 +157,10 @@ def test_tile_product_every_tile_height(ops, gen, variant, m, n, k):
         wgu = rnd((2 * n, k), torch.bfloat16, gen, 0.2)
         h1 = torch.empty(m, n, device="cuda", dtype=torch.bfloat16)
         h2 = torch.empty_like(h1)
-        for act in ("silu", "gelu_pytorch_tanh"):
-            ops.swiglu_linear(x, wgu, h1, act=act)
-            PlainOps().swiglu_linear(x, wgu, h2, act=act)
+        gbias = torch.randn(2 * n, generator=gen, device="cuda") * 3
+        for act, b in (("silu", None), ("gelu_pytorch_tanh", gbias)):
+            ops.swiglu_linear(x, wgu, h1, act=act, bias=b)
+            PlainOps().swiglu_linear(x, wgu, h2, act=act, bias=b)
             close(h1, h2, torch.bfloat16, scale=k * 0.2)
 
 

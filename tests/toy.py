@@ -58,11 +58,14 @@ class ToyConfig:
     intermediate_size: int
     decay: float
     rms_norm_eps: float
+    mlp_bias: bool = False   # the feed-forward's three products each add a bias of the checkpoint
+    hidden_act: str = "silu"
 
     @staticmethod
     def from_dict(raw: dict) -> "ToyConfig":
         return ToyConfig(raw["vocab_size"], raw["hidden_size"], raw["num_hidden_layers"],
-                         raw["intermediate_size"], raw["decay"], raw["rms_norm_eps"])
+                         raw["intermediate_size"], raw["decay"], raw["rms_norm_eps"],
+                         raw.get("mlp_bias", False), raw.get("hidden_act", "silu"))
 
 
 def build_toy(cfg: ToyConfig) -> ModelSpec:
@@ -74,7 +77,8 @@ def build_toy(cfg: ToyConfig) -> ModelSpec:
         blocks.append(PreNormBlock(RMSNorm(p + "norm1.", h, cfg.rms_norm_eps),
                                    RunningMeanMixer(p, h, cfg.decay),
                                    RMSNorm(p + "norm2.", h, cfg.rms_norm_eps),
-                                   SwiGLU(p + "mlp.", h, cfg.intermediate_size)))
+                                   SwiGLU(p + "mlp.", h, cfg.intermediate_size, act=cfg.hidden_act,
+                                          bias=cfg.mlp_bias)))
     return ModelSpec(emb, blocks, RMSNorm("norm.", h, cfg.rms_norm_eps),
                      LMHead("head.", cfg.vocab_size, h))
 
@@ -86,6 +90,9 @@ def register() -> None:
 
 TOY_CONFIG = {"architectures": ["ToyStateForCausalLM"], "vocab_size": 97, "hidden_size": 40,
               "num_hidden_layers": 2, "intermediate_size": 56, "decay": 0.8, "rms_norm_eps": 1e-5}
+# the same with a feed-forward of another kind: the tanh form of GELU as the gate's activation and
+# a bias on each of its three products (parameters of the framework's dense feed-forward)
+TOY_BIASED_MLP_CONFIG = dict(TOY_CONFIG, mlp_bias=True, hidden_act="gelu_pytorch_tanh")
 
 
 def plain_forward(w: Dict[str, torch.Tensor], cfg: dict, tokens: List[int]) -> torch.Tensor:
@@ -102,8 +109,11 @@ def plain_forward(w: Dict[str, torch.Tensor], cfg: dict, tokens: List[int]) -> t
             y[t] = w[p + "mix.weight"].float() @ s
         x = x + y
         m = pm.rms_norm(x, w[p + "norm2.weight"], cfg["rms_norm_eps"])
+        biases = None
+        if cfg.get("mlp_bias"):
+            biases = (w[p + "mlp.gate_proj.bias"], w[p + "mlp.up_proj.bias"], w[p + "mlp.down_proj.bias"])
         x = x + pm.swiglu_mlp(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
-                              w[p + "mlp.down_proj.weight"])
+                              w[p + "mlp.down_proj.weight"], cfg.get("hidden_act", "silu"), biases)
     return pm.rms_norm(x, w["norm.weight"], cfg["rms_norm_eps"]) @ w["head.weight"].float().T
 
 
