@@ -15,10 +15,11 @@
 // is left to hide is the rest: with two waves per SIMD the epilogue and the
 // waits at the barrier of one run beside the products of the other (3 to 15%
 // on the experts' products of 1,024 to 8,192 tokens).
-// A wave column multiplies only its 32-row blocks that hold rows, and after the
-// first two k tiles a wave loads only the pieces of A that hold rows, so a tile
-// with few rows costs little more than its share: one tile height serves every
-// count of rows per expert.
+// A wave column multiplies only its 32-row blocks that hold rows (the tile's rows
+// fill the columns' blocks one after the other, the first column's first), and
+// after the first two k tiles a wave loads only the pieces of A that hold rows,
+// so a tile with few rows costs little more than its share: one tile height
+// serves every count of rows per expert.
 //
 // LDS rows are 128 bytes (64 bf16) and unpadded, because a wave's load writes
 // 1 KB contiguously (lane l at 16 l); the eight 16-byte chunks of row r are
@@ -81,8 +82,19 @@ __global__ __launch_bounds__(direct::WAVES * 64, 1) void gemm_tile_direct_kernel
   constexpr int OUT_PER_WAVE = OUT_PER_BLOCK / WGM;
   const int out0 = by * OUT_PER_BLOCK;
   const int rows_here = min(TM, row_end - row0);
-  // staged row l holds the tile's row (l % COL) * WGN + l / COL: column l / COL gets every WGN-th row
-  auto row_of = [&](int l) -> int { return (l % COL) * WGN + l / COL; };
+  // The tile's rows go to the two wave columns in whole blocks of 32, the first column
+  // taking the odd one: a SIMD holds a wave of each column, so its matrix instructions are
+  // those of both, and 137 rows cost it five blocks (3 + 2) where rows dealt in turn would
+  // cost six (69 + 68 rows). Staged row l of column l / COL holds the tile's row
+  // (l / COL) * rows0 + l % COL, or none (TM: beyond every tile's rows).
+  static_assert(WGN == 2, "the rows are dealt to two wave columns");
+  const int n_blocks = (rows_here + 31) / 32;
+  const int rows0 = min(rows_here, 32 * ((n_blocks + 1) / 2));   // rows of the first column
+  auto row_of = [&](int l) -> int {
+    const int i = l % COL;
+    if (l < COL) return i < rows0 ? i : TM;
+    return rows0 + i < rows_here ? rows0 + i : TM;
+  };
 
   // Loads: instruction i of wave w fills the 1 KB piece i * 4 + w of the X (and
   // of the W) part of a buffer: RPP rows, lane l at row l / CPR, stored chunk
@@ -173,7 +185,7 @@ __global__ __launch_bounds__(direct::WAVES * 64, 1) void gemm_tile_direct_kernel
       for (int v = 0; v < 16; ++v) acc[i][jj][v] = 0.f;
 
   // rows dealt to this wave's column, and its 32-row blocks that hold any
-  const int col_rows = rows_here > wn ? (rows_here - wn + WGN - 1) / WGN : 0;
+  const int col_rows = wn == 0 ? rows0 : rows_here - rows0;
   const int n_jj = (col_rows + 31) / 32;
   const int tok0 = wn * COL;
 
