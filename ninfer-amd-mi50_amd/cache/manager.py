@@ -1,8 +1,9 @@
 """Cache manager: paged keys and values with a block table per request, and
 slots of fixed-size per-request state.
 
-Layers whose mixers need the same span of the past form a *group*: all keys
-(window None) or the last `window` positions. A group has its own page ids,
+Layers whose mixers need the same span of the past, in pages of the same size, form
+a *group*: all keys (window None) or the last `window` positions; the engine's page
+size or one the mixer asks for. A group has its own page ids,
 allocator and block tables; every cache instance (one per plan entry that
 writes keys and values) in the group has its own pools (any number, named,
 each with a per-token shape and dtype of its own), indexed by the group's
@@ -35,6 +36,8 @@ from .pages import OutOfPages, PageAllocator
 class CacheGroup:
     window: Optional[int]
     allocator: PageAllocator
+    page_size: int = 0                                    # tokens a page of this group holds
+    max_pages: int = 0                                    # pages a request can hold at most
     instances: List[int] = field(default_factory=list)   # plan entries with pools in this group
     tables: Dict[int, List[int]] = field(default_factory=dict)  # slot -> page of each logical page
     window_freed: int = 0
@@ -57,18 +60,25 @@ class CacheManager:
         self.needs = list(needs)
         self.groups: List[CacheGroup] = []
         self.group_of_instance: Dict[int, int] = {}
-        by_window: Dict[Optional[int], int] = {}
+        by_kind: Dict[Tuple[Optional[int], int], int] = {}
         for i, need in enumerate(self.needs):
             if need is None:
                 continue
-            if need.window not in by_window:
-                by_window[need.window] = len(self.groups)
-                self.groups.append(CacheGroup(need.window, PageAllocator(num_pages)))
-            g = by_window[need.window]
+            ps = need.page_size if need.page_size is not None else page_size
+            if ps < 1:
+                raise ValueError(f"a mixer asks for pages of {ps} tokens")
+            if (need.window, ps) not in by_kind:
+                by_kind[(need.window, ps)] = len(self.groups)
+                # `num_pages` counts pages of the engine's size: a group with pages of another
+                # size gets as many as hold the same number of tokens
+                n = num_pages if ps == page_size else max(1, num_pages * page_size // ps)
+                self.groups.append(CacheGroup(need.window, PageAllocator(n), page_size=ps,
+                                              max_pages=-(-max_context // ps)))
+            g = by_kind[(need.window, ps)]
             self.groups[g].instances.append(i)
             self.group_of_instance[i] = g
         for g in self.groups:
-            g.rows = np.full((max_seqs, self.max_pages_per_request), -1, dtype=np.int32)
+            g.rows = np.full((max_seqs, g.max_pages), -1, dtype=np.int32)
         self._free_slots: List[int] = list(range(max_seqs - 1, -1, -1))
         self._length: Dict[int, int] = {}
         self.pools: Dict[int, Dict[str, object]] = {}   # cache instance -> pool name -> tensor
@@ -89,7 +99,8 @@ class CacheManager:
         for i, need in enumerate(self.needs):
             if need is None:
                 continue
-            n = self.groups[self.group_of_instance[i]].allocator.num_pages
+            group = self.groups[self.group_of_instance[i]]
+            n = group.allocator.num_pages
             self.pools[i] = {}
             for spec in need.pools:
                 if spec.name in self.pools[i]:
@@ -97,7 +108,7 @@ class CacheManager:
                 if spec.dtype is not None and spec.dtype not in named:
                     raise ValueError(f"pool {spec.name!r}: dtype {spec.dtype!r} is not one of "
                                      f"{sorted(named)}")
-                shape = (n, *spec.outer, self.page_size, *spec.inner)
+                shape = (n, *spec.outer, group.page_size, *spec.inner)
                 self.pools[i][spec.name] = torch.zeros(
                     shape, dtype=named[spec.dtype] if spec.dtype else dtype, device=device)
         self.state = torch.zeros((self.max_seqs, max(self.state_floats, 1)),
@@ -155,8 +166,7 @@ class CacheManager:
 
     # ---- pages ---------------------------------------------------------------
     def pages_needed(self, slot: int, new_len: int) -> List[int]:
-        want = -(-new_len // self.page_size)
-        return [max(0, want - len(g.tables[slot])) for g in self.groups]
+        return [max(0, -(-new_len // g.page_size) - len(g.tables[slot])) for g in self.groups]
 
     def can_reserve(self, slot: int, new_len: int) -> bool:
         return all(n <= g.allocator.free_pages
@@ -207,7 +217,7 @@ class CacheManager:
                 continue
             table = g.tables[slot]
             # pages whose last position (p+1)*ps - 1 <= new_len - window
-            dead = (new_len - g.window + 1) // self.page_size
+            dead = (new_len - g.window + 1) // g.page_size
             gone = []
             for p in range(min(max(dead, 0), len(table))):
                 if table[p] >= 0:

@@ -176,11 +176,12 @@ class ModelRunner:
         graph = (self.options.use_graph and self.device.type == "cuda" and int(qlen.max()) == 1
                  and want_rows == list(range(T)))
         # a graph is replayed for many steps: fixed table width, context rounded up
-        width = cache.max_pages_per_request if graph else None
         if graph:
             max_kv_len = min(-(-max_kv_len // self.graph_context_step) * self.graph_context_step,
-                             cache.max_pages_per_request * cache.page_size)
-        tables = [cache.block_table(g, slots, width) for g in range(len(cache.groups))]
+                             min(g.max_pages * g.page_size for g in cache.groups)
+                             if cache.groups else cache.max_pages_per_request * cache.page_size)
+        tables = [cache.block_table(g, slots, cache.groups[g].max_pages if graph else None)
+                  for g in range(len(cache.groups))]
         if self.options.check_pages:
             self._check_pages(chunks, pos0, tables)
         parts = [tokens, positions, row_seq, np.asarray(slots, np.int32), row_start, qlen,
@@ -231,8 +232,8 @@ class ModelRunner:
         the step writes, and every earlier one its rows can see, lies in a page that the
         allocator counts as held; no page stands in two requests' rows. (The reference's
         analogue is the overflow throw of its slab, src/runtime/kv_cache.cpp:35-37.)"""
-        ps = self.cache.page_size
         for g, table in zip(self.cache.groups, tables):
+            ps = g.page_size
             owner: Dict[int, int] = {}
             for i, (c, p) in enumerate(zip(chunks, pos0)):
                 row = table[i]
@@ -329,7 +330,7 @@ class ModelRunner:
             view = None
             if owner in cache.pools:
                 g = cache.group_of_instance[owner]
-                view = CacheView(cache.pools[owner], d_tables[g], cache.page_size,
+                view = CacheView(cache.pools[owner], d_tables[g], cache.groups[g].page_size,
                                  cache.groups[g].window)
             rng = self._state_range[i]
             state = cache.state[:, rng] if rng is not None else None

@@ -133,8 +133,8 @@ class Scheduler:
         step of n tokens touches, the window - 1 keys before its first row and its n rows
         (pages the window has passed are given back after every step): window + n - 1
         positions, which lie in at most ceil(that / page) + 1 pages wherever they start."""
-        ps = self.cache.page_size
         for g in self.cache.groups:
+            ps = g.page_size
             most = -(-total // ps)
             if g.window is not None:
                 most = min(most, -(-(g.window + self.max_batch_tokens - 1) // ps) + 1)

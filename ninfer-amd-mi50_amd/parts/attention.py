@@ -26,13 +26,14 @@ class Attention(Mixer):
                  position: PositionEncoding, qkv_bias: bool = True,
                  window: Optional[int] = None, scale: Optional[float] = None,
                  score_slopes: Optional[Sequence[float]] = None,
-                 qk_norm_eps: Optional[float] = None):
+                 qk_norm_eps: Optional[float] = None, page_size: Optional[int] = None):
         """`score_slopes` [heads]: a distance-based position bias, slope * (key's position -
         query's position) added to head h's scaled scores before the softmax (None: none).
         It is a parameter of the attention kernels, beside or instead of the rotation that
         `position` describes. `qk_norm_eps`: every query and key head is normed over its dims
         (x rsqrt(mean(x^2) + eps) gain, gains `q_norm.weight` and `k_norm.weight` [head_dim] of the
-        checkpoint) after the bias and before it turns; None: no such norm."""
+        checkpoint) after the bias and before it turns; None: no such norm. `page_size`: tokens
+        in a page of this layer's keys and values (None: the engine's)."""
         if heads % kv_heads:
             raise ValueError(f"heads ({heads}) must be a multiple of kv_heads ({kv_heads})")
         if score_slopes is not None and len(score_slopes) != heads:
@@ -49,6 +50,7 @@ class Attention(Mixer):
         self.score_slopes = None if score_slopes is None else [float(x) for x in score_slopes]
         self.slopes: Optional[torch.Tensor] = None   # the same on the device (32-bit)
         self.qk_norm_eps = qk_norm_eps
+        self.page_size = page_size
         self.q_norm: Optional[torch.Tensor] = None
         self.k_norm: Optional[torch.Tensor] = None
         self.w_qkv: Optional[torch.Tensor] = None
@@ -60,7 +62,7 @@ class Attention(Mixer):
         return (self.heads + 2 * self.kv_heads) * self.head_dim
 
     def cache_need(self) -> Optional[CacheNeed]:
-        return CacheNeed.keys_values(self.kv_heads, self.head_dim, self.window)
+        return CacheNeed.keys_values(self.kv_heads, self.head_dim, self.window, self.page_size)
 
     def children(self) -> List[Part]:
         return [self.position]

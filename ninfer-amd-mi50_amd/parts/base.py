@@ -42,18 +42,20 @@ class PoolSpec:
 class CacheNeed:
     """What a mixer needs of the paged cache for each token it has seen: any
     number of named pools, each with a per-token shape and dtype of its own,
-    for all positions (window None) or only the last `window` of them. Mixers
-    with the same window share page numbers and block tables; each has pools
-    of its own."""
+    for all positions (window None) or only the last `window` of them, in pages
+    of `page_size` tokens (None: the engine's). Mixers with the same window and
+    page size share page numbers and block tables; each has pools of its own."""
     pools: Tuple[PoolSpec, ...]
     window: Optional[int] = None
+    page_size: Optional[int] = None
 
     @staticmethod
-    def keys_values(kv_heads: int, head_dim: int, window: Optional[int] = None) -> "CacheNeed":
+    def keys_values(kv_heads: int, head_dim: int, window: Optional[int] = None,
+                    page_size: Optional[int] = None) -> "CacheNeed":
         """Keys and values of `kv_heads` heads of `head_dim`: pools 'k' and 'v',
         each [pages, kv_heads, page_size, head_dim]."""
         return CacheNeed((PoolSpec("k", (kv_heads,), (head_dim,)),
-                          PoolSpec("v", (kv_heads,), (head_dim,))), window)
+                          PoolSpec("v", (kv_heads,), (head_dim,))), window, page_size)
 
 
 @dataclass

@@ -41,6 +41,32 @@ def test_groups_by_window():
     assert same.kv_bytes_per_token(2) == 2 * (2 * 8 + 4 * 16) * 2
 
 
+def test_groups_by_page_size():
+    """Mixers that ask for pages of another size form groups of their own, with as many pages
+    as hold the same number of tokens and tables as wide as the longest request needs."""
+    needs = [CacheNeed.keys_values(2, 8), CacheNeed.keys_values(2, 8, None, page_size=8),
+             CacheNeed.keys_values(2, 8, 6, page_size=8), CacheNeed.keys_values(1, 4, None, page_size=4)]
+    m = CacheManager(needs, 4, 10, 3, 30)
+    assert [(g.window, g.page_size, g.allocator.num_pages, g.max_pages) for g in m.groups] == \
+        [(None, 4, 10, 8), (None, 8, 5, 4), (6, 8, 5, 4)]
+    assert m.group_of_instance == {0: 0, 1: 1, 2: 2, 3: 0}
+    s = m.acquire()
+    assert m.pages_needed(s, 9) == [3, 2, 2]
+    m.reserve(s, 9)
+    m.commit(s, 9)
+    assert m.block_table(0, [s]).tolist() == [[0, 1, 2]] and m.block_table(1, [s]).tolist() == [[0, 1]]
+    m.reserve(s, 17)
+    m.commit(s, 17)                       # the window of 6 has passed positions 0..7: one page of 8
+    assert m.block_table(2, [s]).tolist() == [[-1, 1, 2]] and m.groups[2].window_freed == 1
+    t = m.acquire()
+    with pytest.raises(OutOfPages):
+        m.reserve(t, 24)                  # 6 pages of 4 are wanted, 5 are free
+    assert m.pages_free(1) == 2 and m.block_table(1, [t]).tolist() == [[-1]]
+    m.check()
+    with pytest.raises(ValueError, match="pages of 0"):
+        CacheManager([CacheNeed.keys_values(2, 8, None, page_size=0)], 4, 10, 3, 30)
+
+
 def test_reserve_commit_release_and_block_table():
     m = manager()
     s = m.acquire()
@@ -108,10 +134,15 @@ def test_slots_run_out_and_come_back():
     assert m.acquire() == a and m.length(a) == 0
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(8))
 def test_random_orders_of_requests(seed):
     rng = random.Random(seed)
-    m = manager(num_pages=24, window=10, page_size=4, seqs=5, max_context=80)
+    if seed < 6:
+        m = manager(num_pages=24, window=10, page_size=4, seqs=5, max_context=80)
+    else:                                 # groups with pages of 4, 8 and 2 tokens
+        needs = [CacheNeed.keys_values(2, 8), CacheNeed.keys_values(2, 8, 10, page_size=8),
+                 CacheNeed.keys_values(2, 8, None, page_size=2)]
+        m = CacheManager(needs, 4, 24, 5, 80)
     live = {}
     for _ in range(600):
         action = rng.random()

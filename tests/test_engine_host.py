@@ -227,6 +227,28 @@ def test_toy_learned_positions_and_score_bias(tmp_path):
                                     page_size=4), ops=PlainOps())
 
 
+def test_attention_layers_with_pages_of_other_sizes(tmp_path):
+    """The framework's attention part with a page size per layer (8, 32 and the engine's 16):
+    three groups with block tables of their own, the same logits."""
+    import ninfer_amd
+    toy.register_routed()
+    cfg = toy.TOY_PAGES_CONFIG
+    d = str(tmp_path / "toy_pages")
+    ninfer_amd.write_random_model(d, cfg, 16, std=0.3)
+    _, w = util.read_folder(d)
+    runner = runner_for(d, page_size=16, num_pages=12, seqs=3)
+    assert [(g.page_size, g.allocator.num_pages) for g in runner.cache.groups] == \
+        [(8, 24), (32, 6), (16, 12)]
+    assert runner.cache.pools[1]["k"].shape == (6, 2, 32, 64)
+    reqs = {f"r{i}": util.random_tokens(n, 83, 90 + i) for i, n in enumerate([7, 70, 15, 40, 33])}
+    ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=5, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+    runner.cache.check()
+    assert runner.cache.pages_reused() > 0
+
+
 def test_toy_normed_query_and_key_heads(tmp_path):
     """Attention whose query and key heads are normed over their dims before they turn: a
     parameter of the attention part (two gain vectors of the checkpoint) and of the rotation's
@@ -297,6 +319,40 @@ def test_toy_mixer_with_pools_of_its_own(tmp_path):
         torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
     runner.cache.check()
     assert runner.cache.pages_reused() > 0 and runner.cache.groups[1].window_freed > 0
+
+
+def test_toy_mixer_with_a_page_size_of_its_own(tmp_path):
+    """A mixer may ask for pages of another size than the engine's: its layers form a group of
+    their own with as many pages as hold the same number of tokens, their own block tables and
+    their own giving back; the step function and the scheduler take each group's page size."""
+    import ninfer_amd
+    from ninfer_amd import Request, SamplingParams, Scheduler
+    toy.register_latent()
+    cfg = dict(toy.TOY_LATENT_CONFIG, windows=[None, 9, None], page_sizes=[None, 8, 2],
+               num_hidden_layers=3)
+    d = str(tmp_path / "toy_latent_pages")
+    ninfer_amd.write_random_model(d, cfg, 12, std=0.3)
+    _, w = util.read_folder(d)
+    runner = runner_for(d, page_size=4, num_pages=26, seqs=3)
+    cache = runner.cache
+    assert [(g.window, g.page_size, g.allocator.num_pages, g.max_pages) for g in cache.groups] == \
+        [(None, 4, 26, 32), (9, 8, 13, 16), (None, 2, 52, 64)]
+    assert cache.pools[1]["latent"].shape == (13, 8, 12) and cache.pools[2]["pos_key"].shape == (52, 2, 6)
+    reqs = {f"l{i}": util.random_tokens(n, 61, 70 + i) for i, n in enumerate([9, 30, 17, 41, 5])}
+    ref = {k: toy.plain_forward_latent(w, cfg, v) for k, v in reqs.items()}
+    for k, v in reqs.items():
+        for sched in (util.schedule_whole(k, v), util.schedule_tail(k, v, 5),
+                      util.schedule_portions(k, v, 1)):
+            torch.testing.assert_close(util.run_schedule(runner, sched)[k], ref[k],
+                                       atol=3e-5, rtol=1e-4)
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=8, max_live=3))
+    for k in reqs:
+        torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+    cache.check()
+    assert cache.pages_reused() > 0 and cache.groups[1].window_freed > 0
+    # the scheduler plans with every group's page size (here the pages of 2 tokens run out first)
+    sched = Scheduler(runner, None, max_batch_tokens=16, max_seqs=3)
+    assert sched._fits_alone(100) and not sched._fits_alone(105)   # 52 pages of 2 tokens
 
 
 def test_page_checks_name_a_table_that_the_kernels_could_not_trust(model_dirs):

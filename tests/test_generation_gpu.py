@@ -343,6 +343,44 @@ def test_toy_learned_positions_and_score_bias_on_the_gpu(tmp_path, dtype):
         load_model(d, EngineOptions(dtype=dtype, max_context=176, num_sequences=1, page_size=16))
 
 
+@pytest.mark.parametrize("dtype,graph", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
+def test_attention_layers_with_pages_of_other_sizes_on_the_gpu(tmp_path, dtype, graph):
+    """A page size per layer (8, 32 and the engine's 16; heads of 64, so that the bfloat16 steps
+    run the matrix-core kernels with each): three cache groups with block tables of their own,
+    so few pages that they are used again, decoding also from a captured graph (whose tables
+    have each group's full width)."""
+    import ninfer_amd
+    from ninfer_amd import EngineOptions, load_model
+    toy.register_routed()
+    cfg = toy.TOY_PAGES_CONFIG
+    d = str(tmp_path / "toy_pages")
+    ninfer_amd.write_random_model(d, cfg, 16, dtype=dtype, std=0.2)
+    _, w = util.read_folder(d)
+    runner = load_model(d, EngineOptions(dtype=dtype, max_context=160, num_sequences=3, page_size=16,
+                                         num_pages=22, check_pages=True, poison_freed_pages=True,
+                                         use_graph=graph))
+    assert [(g.page_size, g.allocator.num_pages, g.max_pages) for g in runner.cache.groups] == \
+        [(8, 44, 20), (32, 11, 5), (16, 22, 10)]
+    reqs = {f"r{i}": util.random_tokens(n, 83, 90 + i) for i, n in enumerate([7, 96, 15, 150, 33])}
+    ref = {k: toy.plain_forward_routed(w, cfg, v) for k, v in reqs.items()}
+    got = util.run_schedule(runner, util.schedule_mixed(reqs, seed=5, max_live=3))
+    tail = util.run_schedule(runner, util.schedule_tail("r3", reqs["r3"], 32))["r3"]
+    if dtype == "float32":
+        for k in reqs:
+            torch.testing.assert_close(got[k], ref[k], atol=3e-5, rtol=1e-4)
+        torch.testing.assert_close(tail, ref["r3"], atol=3e-5, rtol=1e-4)
+    else:
+        top = float(ref["r3"].abs().max())
+        for rows in (got["r3"], tail, got["r1"]):
+            assert torch.isfinite(rows).all()
+            want = ref["r3"] if rows.shape[0] == 150 else ref["r1"]
+            err = (rows - want).abs().max(-1).values
+            assert float(err.median()) < 0.03 * top
+    runner.cache.check()
+    assert runner.cache.pages_reused() > 0
+    assert bool(runner._graphs) == graph
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_toy_normed_query_and_key_heads_on_the_gpu(tmp_path, dtype):
     """Query and key heads normed over their dims before the rotation, in the rotation's kernel

@@ -216,7 +216,8 @@ def build_toy_routed(cfg: ToyRoutedConfig) -> ModelSpec:
             # bias on the scores (head i: slope 2^-(i+1)), both parameters of the framework
             attn = Attention(p + "attn.", h, c["heads"], c["kv_heads"], c["head_dim"], NoPosition(),
                              qkv_bias=False, window=c["window"],
-                             score_slopes=[2.0 ** -(i + 1) for i in range(c["heads"])])
+                             score_slopes=[2.0 ** -(i + 1) for i in range(c["heads"])],
+                             page_size=c.get("page_sizes", [None] * 99)[l])
         else:
             attn = Attention(p + "attn.", h, c["heads"], c["kv_heads"], c["head_dim"],
                              HarmonicPosition(c["rot_dim"], c["slope"], c.get("pairing", "half")),
@@ -260,6 +261,10 @@ TOY_QK_NORM_CONFIG = dict(TOY_ROUTED_CONFIG, qk_norm_eps=1e-5)
 # attention kernels with the bias
 TOY_BIASED_CONFIG = dict(TOY_ROUTED_CONFIG, positions="learned+bias", max_positions=160, heads=4,
                          kv_heads=2, head_dim=64, hidden_size=64, window=None)
+
+
+# the same with pages of another size on each layer (the engine's on the last)
+TOY_PAGES_CONFIG = dict(TOY_BIASED_CONFIG, num_hidden_layers=3, page_sizes=[8, 32, None])
 
 
 def plain_forward_routed(w: Dict[str, torch.Tensor], c: dict, tokens: List[int]) -> torch.Tensor:
@@ -346,14 +351,15 @@ class LatentMixer(Mixer):
     table: what it shows is that the cache manager hands any named pools to a mixer."""
 
     def __init__(self, prefix: str, hidden: int, latent: int, pos_dim: int, slope: float,
-                 window=None):
+                 window=None, page_size=None):
         self.prefix, self.hidden, self.latent, self.pos_dim = prefix, hidden, latent, pos_dim
-        self.slope, self.window = slope, window
+        self.slope, self.window, self.page_size = slope, window, page_size
         self.w = {}
 
     def cache_need(self):
+        # (a page size of its own, where the configuration names one: None is the engine's)
         return CacheNeed((PoolSpec("latent", (), (self.latent,), "float32"),
-                          PoolSpec("pos_key", (), (self.pos_dim,))), self.window)
+                          PoolSpec("pos_key", (), (self.pos_dim,))), self.window, self.page_size)
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         p, h = self.prefix, self.hidden
@@ -405,7 +411,7 @@ def build_toy_latent(cfg: ToyRoutedConfig) -> ModelSpec:
         p = f"layers.{l}."
         blocks.append(PreNormBlock(RMSNorm(p + "norm1.", h, c["rms_norm_eps"]),
                                    LatentMixer(p + "mix.", h, c["latent"], c["pos_dim"], c["slope"],
-                                               c["windows"][l]),
+                                               c["windows"][l], c.get("page_sizes", [None] * 99)[l]),
                                    RMSNorm(p + "norm2.", h, c["rms_norm_eps"]),
                                    SwiGLU(p + "mlp.", h, c["inner"])))
     return ModelSpec(TokenEmbedding("embed.", c["vocab_size"], h), blocks,
