@@ -525,11 +525,18 @@ bool gemm_skinny_route_pair_takes(const GemmArgs& a, const GemmArgs& b, const Ro
 int gemm_skinny_route_pair(const GemmArgs& a, const GemmArgs& b, const RouteArgs& rt,
                            hipStream_t stream) {
   const SkinnyPlan pb = plan_skinny(b);
-  const int threads = 1024;                      // the router's block has work for 16 waves
+  // The router's block has work for 16 waves and is the launch's longest beside a short
+  // dense product. But a block of 16 waves is alone on its CU, and the dense product's blocks
+  // then follow each other with nothing overlapping their starts and ends (they stream at 5.5
+  // TB/s instead of 6.8): beside a long dense product (100 MB of weights and more) every block
+  // has the dense product's waves, and the router's block makes do with them.
+  const bool long_b = (int64_t)b.N * b.K * (epilogue_gated(b.epilogue) ? 4 : 2) >= (100LL << 20);
+  const int threads = long_b ? 64 * max(pb.waves, 8) : 1024;
   const size_t lds = (size_t)(threads / 64) * 4096;
   // the router's block: 5 KB of logits, E + 1 counters and 16 k chosen experts in its 32 KB
-  static_assert(16 * kRouteMaxFeatures * 4 + (kRouteMaxFeatures + 1) * 4 + 16 * 64 * 4 <= 16 * 2048,
-                "the routing block's LDS");
+  static_assert(16 * kRouteMaxFeatures * 4 + (kRouteMaxFeatures + 1) * 4 + 16 * 64 * 4 <= 8 * 2048,
+                "the routing block's LDS (8 waves' stage at least)");
+  static_assert((kRouteMaxFeatures + 15) / 16 <= 8, "a wave's two feature groups x 8 waves hold them");
   const long blocks = 1 + (long)pb.grid_x * pb.grid_y;
   NINFER_REQUIRE(blocks < (1L << 31), "gemm pair: %ld blocks are too many", blocks);
   gemm_skinny_route_pair_kernel<false, true, bf16>

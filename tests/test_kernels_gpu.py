@@ -448,6 +448,7 @@ def test_products_launched_together(ops_mode, gen, dtype, t, e, k, h, inner, sha
 @pytest.mark.parametrize("t,e,k,h,shared_inner,extra", [
     (1, 60, 4, 2048, 5632, 1), (8, 60, 4, 2048, 1408, 1), (16, 64, 8, 3584, 512, 1),
     (5, 7, 3, 384, 1000, 0), (16, 79, 5, 256, 96, 1), (2, 8, 8, 64, 96, 1), (11, 33, 1, 160, 48, 2),
+    (7, 64, 8, 3584, 7424, 1),    # a long dense product (106 MB): the launch has its waves, not 16
     (17, 60, 4, 256, 352, 1),     # more rows than one tile: products, then the routing kernels
     (3, 100, 6, 128, 96, 0),      # more experts than the routing block takes
     (40, 6, 2, 128, 96, 1)])
