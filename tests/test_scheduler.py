@@ -259,3 +259,48 @@ def test_a_windowed_group_admits_what_its_window_can_serve(model_dirs):
         sched.add(req2)
         sched.run()
         assert req2.status == "failed" and "fit" in req2.error
+
+
+def test_groups_with_pages_of_other_sizes_under_the_scheduler(tmp_path):
+    """Layers with pages of 8, 32 and 16 tokens (three cache groups): the scheduler counts
+    every group's pages in that group's size, gives requests back when any group runs out,
+    and the tokens are those of a run with room for everything."""
+    import ninfer_amd
+    import toy
+    from ninfer_amd import EngineOptions, Request, SamplingParams, Sampler, Scheduler, load_model
+    toy.register_routed()
+    cfg = toy.TOY_PAGES_CONFIG
+    d = str(tmp_path / "toy_pages")
+    ninfer_amd.write_random_model(d, cfg, 16, std=0.3)
+
+    def run(num_pages):
+        opt = EngineOptions(dtype="float32", max_context=96, prefill_chunk=16, num_sequences=4,
+                            page_size=16, num_pages=num_pages, device="cpu", check_pages=True)
+        runner = load_model(d, opt, ops=PlainOps())
+        sched = Scheduler(runner, Sampler(PlainOps(), runner.device))
+        params = SamplingParams(max_new_tokens=12, temperature=0.8, top_k=20, top_p=0.9, seed=5)
+        reqs = [Request(f"q{i}", util.random_tokens(n, 83, 60 + i), params)
+                for i, n in enumerate([30, 28, 25, 21])]
+        for r in reqs:
+            sched.add(r)
+        sched.run()
+        runner.cache.check()
+        assert all(g.allocator.in_use == 0 for g in runner.cache.groups)
+        return runner, sched, reqs
+
+    _, roomy, ref = run(64)
+    assert roomy.preemptions == 0
+    # 9 pages of 16 tokens, hence 18 of 8 and 4 of 32: the four prompts take a page of 32 each
+    # and all are admitted; grown past 32 tokens each needs a second one, and there is none
+    runner, tight, again = run(9)
+    assert [(g.page_size, g.allocator.num_pages) for g in runner.cache.groups] == \
+        [(8, 18), (32, 4), (16, 9)]
+    assert tight.preemptions > 0
+    for a, b in zip(ref, again):
+        assert b.status == "finished" and a.output == b.output
+    # a request that needs more pages of 32 than there are (3 of 2) fails alone
+    runner, sched, _ = run(4)
+    big = Request("big", util.random_tokens(70, 83, 1), SamplingParams.greedy(10))
+    sched.add(big)
+    sched.run()
+    assert big.status == "failed" and "fit" in big.error
