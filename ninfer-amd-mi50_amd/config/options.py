@@ -37,20 +37,25 @@ class EngineOptions:
             raise ValueError(f"kv_bytes must be >= 1, got {self.kv_bytes}")
         if self.kv_bytes is not None and self.num_pages is not None:
             raise ValueError("give num_pages or kv_bytes, not both")
-        if self.dtype == "bfloat16" and not self.page_size_suits_fast_attention():
+        self.warn_of_slow_pages(self.page_size)
+
+    def warn_of_slow_pages(self, page_size: int) -> None:
+        """Warns of a page size (the engine's, or one a mixer asks for) with which bfloat16
+        attention runs the plain kernel."""
+        if self.dtype == "bfloat16" and not self.page_size_suits_fast_attention(page_size):
             import warnings
             warnings.warn(
-                f"page_size {self.page_size}: the matrix-core attention kernels take pages of "
+                f"page_size {page_size}: the matrix-core attention kernels take pages of "
                 f"8, 16, 32 or 64 tokens (4 too with heads of 128); with this size every bfloat16 step runs the plain "
                 f"attention kernel (one wave per row and head), which is right and many times "
-                f"slower", stacklevel=2)
+                f"slower", stacklevel=3)
 
-    def page_size_suits_fast_attention(self) -> bool:
+    def page_size_suits_fast_attention(self, page_size: Optional[int] = None) -> bool:
         """The bfloat16 prompt kernel walks keys in tiles of 64 that whole pages must fill, one of
         its loads (1 KB of a head's rows: 4 rows of heads of 128, 8 of 64) must stay inside a
         page, and both fast kernels find a key's page by a shift: a power of two from 4 to 64
         (pages of 4 with heads of 64 still run the plain kernel for prompt portions)."""
-        ps = self.page_size
+        ps = self.page_size if page_size is None else page_size
         return ps >= 4 and ps & (ps - 1) == 0 and ps <= 64
 
     def pages_per_request(self) -> int:

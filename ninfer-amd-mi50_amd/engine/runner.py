@@ -75,6 +75,9 @@ class ModelRunner:
                         for n in needs if n is not None for p in n.pools)
         self.cache = CacheManager(needs, options.page_size, options.pool_pages(per_token),
                                   options.num_sequences, options.max_context, floats)
+        for g in self.cache.groups:
+            if g.page_size != options.page_size:   # a mixer's own page size: the same warning
+                options.warn_of_slow_pages(g.page_size)
         self.cache.allocate_pools(self.device, self.act_dtype, ops=self.ops)
         self.cache.poison_freed = options.poison_freed_pages
         self.vocab_size = spec.vocab_size

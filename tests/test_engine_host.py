@@ -406,6 +406,12 @@ def test_a_page_size_the_fast_attention_kernels_do_not_take_is_said(recwarn):
     for ps in (48, 128, 24, 2):
         with pytest.warns(UserWarning, match=f"page_size {ps}.*plain attention kernel"):
             EngineOptions(dtype="bfloat16", page_size=ps).validate()
+    # ... and so of a page size that a mixer asks for itself
+    opt = EngineOptions(dtype="bfloat16", page_size=16)
+    opt.warn_of_slow_pages(32)
+    assert not [w for w in recwarn.list if "page_size 32" in str(w.message)]
+    with pytest.warns(UserWarning, match="page_size 24.*plain attention kernel"):
+        opt.warn_of_slow_pages(24)
     with pytest.raises(ValueError, match="max_graphs"):
         EngineOptions(max_graphs=0).validate()
 
