@@ -45,6 +45,8 @@ struct SkinnyOperands {
   bool w_valid;                 // lanes of rows the tile does not have load nothing
   const bf16* xrow;             // lane (r, j): row r of A at k = 8 j
   bool m_valid;
+  bool w_again;                 // another block beside this one reads the same weights (a dense
+                                // product of several row tiles): they are to stay in L2
 };
 
 // One wave's part of the K range: `waves` waves split K in chunks of four steps (256 bytes
@@ -54,7 +56,7 @@ struct SkinnyOperands {
 // 16-byte units of row R stored in the order u ^ (R % 8), so that the writes (a row per 8
 // lanes) and the fragment reads (lane (r, j): row r, unit 4 i + j) both spread evenly over
 // the banks.
-template <int SETS>
+template <int SETS, bool AGAIN = false>
 __device__ __forceinline__ void skinny_walk(const SkinnyOperands<SETS>& o, int K, int wave,
                                             int waves, unsigned char* my_stage, int lane,
                                             f32x4 (&acc)[SETS]) {
@@ -79,8 +81,9 @@ __device__ __forceinline__ void skinny_walk(const SkinnyOperands<SETS>& o, int K
         for (int s = 0; s < SETS; ++s)
 #pragma unroll
           for (int q = 0; q < 2; ++q)
-            wl[s][h][q] = o.line_valid[q] ? stream_load((const bf16x8*)(o.wline[s][q] + s0 * 32 + h * 64))
-                                          : zero;
+            wl[s][h][q] = !o.line_valid[q] ? zero
+                          : AGAIN ? *(const bf16x8*)(o.wline[s][q] + s0 * 32 + h * 64)
+                                  : stream_load((const bf16x8*)(o.wline[s][q] + s0 * 32 + h * 64));
 #pragma unroll
       for (int i = 0; i < 4; ++i) x[i] = o.m_valid ? *(const bf16x8*)(o.xrow + (s0 + i) * 32) : zero;
 #pragma unroll
@@ -106,6 +109,21 @@ __device__ __forceinline__ void skinny_walk(const SkinnyOperands<SETS>& o, int K
       }
     }
   }
+}
+
+// A dense product of several row tiles is launched as one line of blocks in which the row
+// tiles of a feature tile lie side by side on one XCD (blocks go to the XCDs in turn): the
+// weights then come from HBM once and from that XCD's L2 for the other row tiles (with plain
+// loads: SkinnyOperands::w_again). line_ids: the blocks of such a line; line_tile: the tile of
+// block `id`, false for the ids that pad the line.
+__host__ __device__ inline int line_ids(int grid_x, int grid_y) {
+  return (grid_x + kXcds - 1) / kXcds * kXcds * grid_y;
+}
+__device__ __forceinline__ bool line_tile(int id, int grid_x, int grid_y, int& bx, int& by) {
+  const int x = id % kXcds, slot = id / kXcds;
+  by = slot % grid_y;
+  bx = (slot / grid_y) * kXcds + x;
+  return bx < grid_x;
 }
 
 // The work of one block: tile (bx, by) of the product `a`. WAVES > 0 fixes the waves that
@@ -155,6 +173,7 @@ __device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, in
   const bf16* W = (const bf16*)a.W + (int64_t)group * a.w_group_stride;
   SkinnyOperands<SETS> o;
   o.w_valid = w_valid;
+  o.w_again = !a.offsets && a.M > SM;
   // set s: feature group s / HALVES; with SwiGLU the odd sets are the up rows, N rows further
 #pragma unroll
   for (int s = 0; s < SETS; ++s)
@@ -180,7 +199,10 @@ __device__ __forceinline__ void skinny_block(const GemmArgs& a, int rows_arg, in
   f32x4 acc[SETS];
 #pragma unroll
   for (int s = 0; s < SETS; ++s) acc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
-  skinny_walk<SETS>(o, K, wave, waves, stage + wave * 2048, lane, acc);
+  if (o.w_again)
+    skinny_walk<SETS, true>(o, K, wave, waves, stage + wave * 2048, lane, acc);
+  else
+    skinny_walk<SETS>(o, K, wave, waves, stage + wave * 2048, lane, acc);
 
   // partial tiles -> LDS, element (feature f, token m) of set s at [m * 16 + f]
 #pragma unroll
@@ -230,8 +252,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(GemmArgs a, int
   __shared__ float red[WAVES * (SWIGLU ? 2 : 1) * (TWO ? 2 : 1) * 256];
   __shared__ __attribute__((aligned(16))) unsigned char stage[WAVES * 2048];
   __shared__ int tile_info[3];
-  skinny_block<WAVES, FULL, SWIGLU, TC, TWO>(a, rows_arg, WAVES, blockIdx.x, blockIdx.y, red,
-                                            stage, tile_info);
+  int bx = blockIdx.x, by = blockIdx.y;
+  if (!a.offsets && a.M > SM) {   // launched as one line of blocks (line_tile)
+    if (!line_tile(blockIdx.x, (a.N + rows_arg - 1) / rows_arg, (a.M + SM - 1) / SM, bx, by)) return;
+  }
+  skinny_block<WAVES, FULL, SWIGLU, TC, TWO>(a, rows_arg, WAVES, bx, by, red, stage, tile_info);
 }
 
 // Two products that do not depend on each other in one launch: the first blocks are the
@@ -261,11 +286,13 @@ __global__ __launch_bounds__(1024) void gemm_skinny_pair_kernel(GemmArgs a, Skin
   unsigned char* stage = pair_lds + (blockDim.x >> 6) * 2048;
   const int wave = threadIdx.x >> 6;
   int id = blockIdx.x;
-  const int blocks_b = pb.grid_x * pb.grid_y;
+  // (the dense product's blocks come first, so that its line starts at an XCD's turn)
+  const int blocks_b = pb.grid_y > 1 ? line_ids(pb.grid_x, pb.grid_y) : pb.grid_x;
   if (id < blocks_b) {
     if (wave >= pb.waves) return;
-    skinny_block<0, FULL_B, SW_B, TC_B>(b, pb.rows, pb.waves, id % pb.grid_x, id / pb.grid_x, red,
-                                        stage, tile_info);
+    int bx = id, by = 0;
+    if (pb.grid_y > 1 && !line_tile(id, pb.grid_x, pb.grid_y, bx, by)) return;
+    skinny_block<0, FULL_B, SW_B, TC_B>(b, pb.rows, pb.waves, bx, by, red, stage, tile_info);
   } else {
     id -= blocks_b;
     if (wave >= pa.waves) return;
@@ -302,6 +329,7 @@ __device__ __forceinline__ void skinny_route_block(const GemmArgs& a, const Rout
     const bf16* W = (const bf16*)a.W;
     SkinnyOperands<GS> o;
     o.w_valid = true;
+    o.w_again = false;
 #pragma unroll
     for (int s = 0; s < GS; ++s) o.wrow[s] = W + (int64_t)min(16 * (GS * g + s) + r, N - 1) * K + 8 * j;
 #pragma unroll
@@ -383,6 +411,8 @@ template <int WAVES>
 static void launch_skinny(const GemmArgs& a, int rows, bool two, hipStream_t stream) {
   int m_tiles = a.offsets ? min((a.M + SM - 1) / SM + a.groups, a.M) : (a.M + SM - 1) / SM;
   dim3 grid((a.N + rows - 1) / rows, m_tiles);   // as plan_skinny counts them
+  if (!a.offsets && m_tiles > 1)   // one line of blocks, the row tiles of a feature tile side by side
+    grid = dim3(line_ids(grid.x, m_tiles), 1);
   dim3 block(WAVES * 64);
   bool swiglu = epilogue_gated(a.epilogue);
   if (two) {   // whole tiles, no SwiGLU (plan_skinny)
@@ -484,7 +514,8 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream) {
   if (a.offsets && (long)pa.grid_x * pa.grid_y >= 2048) pb.waves = pa.waves;
   const int threads = 64 * max(pa.waves, pb.waves);
   const size_t lds = (size_t)(threads / 64) * 4096;   // partial sums and weight lines, per wave
-  const long blocks = (long)pa.grid_x * pa.grid_y + (long)pb.grid_x * pb.grid_y;
+  const long blocks = (long)pa.grid_x * pa.grid_y +
+                      (pb.grid_y > 1 ? (long)line_ids(pb.grid_x, pb.grid_y) : (long)pb.grid_x);
   NINFER_REQUIRE(blocks < (1L << 31), "gemm pair: %ld blocks are too many", blocks);
   if (!a.offsets)
     gemm_skinny_pair_kernel<false, false, float, false, true, bf16>
