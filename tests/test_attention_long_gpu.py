@@ -3,7 +3,7 @@ benchmark run (2,048 to 32,768 keys, 8 and 64 decoded rows, 16 kv heads and 28
 query heads on 4 kv heads), against the plain twin (tests/plain_ops.py).
 
 With few rows and short contexts the split-context kernels always cut the
-context into chunks of 128 keys; the larger chunks (256 for the scalar kernel,
+context into chunks of 128 keys; the larger chunks (256 for the scalar kernel from 24 blocks a CU on,
 256, 512 and 1,024 for the matrix-core kernel of grouped heads) and a merge over
 a hundred and more chunks are reached only by the shapes here. Each case first
 asks the library which kernel and chunk size it would run and asserts that it is
@@ -100,8 +100,11 @@ def run_both(ops, case, n_q, n_kv, d, ps, window, dtype):
 # the kernel, chunk size and least number of chunks the case is for)
 DECODE_CASES = {
     # 8 rows x 16 kv heads over 8,192 keys: the benchmark's default step
-    "scalar256-b8-8k": (16, 16, 128, 16, 0,
-                        [8191, 8192, 8447, 8448, 5000, 255, 256, 0], "scalar", 256, 34),
+    "scalar128-b8-8k": (16, 16, 128, 16, 0,
+                        [8191, 8192, 8447, 8448, 5000, 255, 256, 0], "scalar", 128, 67),
+    # the same with 32 rows: blocks enough for the larger chunks
+    "scalar256-b32-8k": (16, 16, 128, 16, 0,
+                         [8191, 8192, 8447, 8448, 5000, 255, 256, 0] * 4, "scalar", 256, 34),
     # 64 rows over about 2,048 keys, contexts that end at, before and after chunk edges
     "scalar256-b64-2k": (16, 16, 128, 16, 0,
                          [2047, 2048, 2049, 2303, 2304, 1023, 1024, 1100, 511, 512, 767, 768, 3,
@@ -112,8 +115,10 @@ DECODE_CASES = {
     # one row, two kv heads: the GPU is not filled, chunks of 128, 256 of them to merge
     "scalar128-b1-32k": (4, 2, 64, 16, 0, [32767], "scalar", 128, 256),
     # a window whose first key lies inside a chunk and inside a page
-    "scalar256-b8-8k-window": (16, 16, 128, 16, 4000,
-                               [8191, 8192, 8447, 8448, 5000, 255, 4000, 3999], "scalar", 256, 34),
+    "scalar128-b8-8k-window": (16, 16, 128, 16, 4000,
+                               [8191, 8192, 8447, 8448, 5000, 255, 4000, 3999], "scalar", 128, 67),
+    "scalar256-b32-8k-window": (16, 16, 128, 16, 4000,
+                                [8191, 8192, 8447, 8448, 5000, 255, 4000, 3999] * 4, "scalar", 256, 34),
     "scalar256-b64-d64-window": (8, 8, 64, 32, 1500,
                                  [4095, 4096, 2047, 1499, 1500, 1501, 3000, 2999] * 8,
                                  "scalar", 256, 17),
@@ -159,8 +164,9 @@ def test_decode_rows_at_long_contexts(ops, name):
     assert float(o2.float().abs().mean()) > 0.1
 
 
-@pytest.mark.parametrize("name", ["scalar256-b8-8k", "scalar256-b8-32k", "heads1024-b8-32k",
-                                  "heads512-b8-8k", "heads256-b8-4k", "scalar256-b8-8k-window",
+@pytest.mark.parametrize("name", ["scalar128-b8-8k", "scalar256-b32-8k", "scalar256-b8-32k",
+                                  "heads1024-b8-32k", "heads512-b8-8k", "heads256-b8-4k",
+                                  "scalar128-b8-8k-window", "scalar256-b32-8k-window",
                                   "heads512-b8-8k-window"])
 def test_decode_rows_find_one_key_at_chunk_edges(ops, name):
     """Row 0 (the longest context of the case) is made to look for one key: the context's
