@@ -468,7 +468,10 @@ static SkinnyPlan plan_skinny(const GemmArgs& a) {
     const long per_cu = ((long)a.N * m_tiles + 16 * cus - 1) / (16 * cus);
     p.rows = (int)(((long)a.N * m_tiles + per_cu * cus - 1) / (per_cu * cus));
   }
-  p.waves = (blocks < 2 * cus && chunks >= 16) ? 16 : (blocks < 8 * cus && chunks >= 8) ? 8 : 4;
+  // (16 waves only while the blocks are fewer than the CUs: a block of 16 waves is alone on its
+  // CU, and with more blocks than CUs they follow each other there with nothing overlapping
+  // their starts and ends; two blocks of 8 waves side by side: a batch-1 step 1.5 to 2% faster)
+  p.waves = (blocks < cus && chunks >= 16) ? 16 : (blocks < 8 * cus && chunks >= 8) ? 8 : 4;
   // a grouped product without SwiGLU whose tiles are many and short (K small): two feature
   // sets per block, so that blocks are half as many and each does twice the work
   p.two = a.skinny_two >= 0 && a.offsets && a.epilogue == kEpilogueNone && p.rows == 16 &&
