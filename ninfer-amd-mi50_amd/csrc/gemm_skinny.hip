@@ -515,6 +515,12 @@ int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream) {
     pa.grid_x = (a.N + 15) / 16;
   }
   if (a.offsets && (long)pa.grid_x * pa.grid_y >= 2048) pb.waves = pa.waves;
+  // ... and 8 waves at most where the launch has more blocks than there are CUs (a block has
+  // the places of the larger need, and blocks of 16 waves follow each other on a CU with
+  // nothing overlapping their starts and ends): batch 1 and 2 steps 1.5 to 2% faster
+  if (pb.waves == 16 && pa.waves <= 8 &&
+      (long)pa.grid_x * pa.grid_y + (long)pb.grid_x * pb.grid_y >= device_cu_count())
+    pb.waves = 8;
   const int threads = 64 * max(pa.waves, pb.waves);
   const size_t lds = (size_t)(threads / 64) * 4096;   // partial sums and weight lines, per wave
   const long blocks = (long)pa.grid_x * pa.grid_y +
