@@ -20,6 +20,7 @@ from typing import List, Optional
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 LIB_NAME = "libninfer_hip.so"
+ENGINE_LIB_NAME = "libninfer_engine.so"   # the engine's C interface (csrc/engine_api)
 ARCH = "gfx950"
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC",
          # packed 32-bit float instructions are kept out of all device code
@@ -37,9 +38,14 @@ def sources() -> List[str]:
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
 
 
+def engine_api_sources() -> List[str]:
+    return sorted(glob.glob(os.path.join(CSRC, "engine_api", "*.cpp")))
+
+
 def _fingerprint() -> str:
     h = hashlib.sha256(" ".join(FLAGS).encode())
-    for path in sources() + sorted(glob.glob(os.path.join(CSRC, "*.h"))):
+    for path in sources() + sorted(glob.glob(os.path.join(CSRC, "*.h"))) + engine_api_sources() \
+            + sorted(glob.glob(os.path.join(CSRC, "engine_api", "*.h"))):
         h.update(os.path.basename(path).encode())
         with open(path, "rb") as f:
             h.update(f.read())
@@ -147,10 +153,33 @@ def _compile_and_link(srcs: List[str], out_dir: str, jobs: int) -> str:
     _run([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-Wl,-z,defs", "-o", lib + ".tmp",
           *objs])
     os.replace(lib + ".tmp", lib)
+    _link_engine_api(out_dir)
     with open(os.path.join(out_dir, "fingerprint"), "w") as f:
         f.write(_fingerprint())
     _say(f"built {lib} in {time.time() - t0:.0f} s")
     return lib
+
+
+def _link_engine_api(out_dir: str) -> None:
+    """The engine's C interface: host code only, over the interpreter this build runs in (its
+    headers and library); the folder of the package's parent goes in as the place to import
+    the engine from."""
+    import sysconfig
+    cfg = sysconfig.get_config_var
+    lib = os.path.join(out_dir, ENGINE_LIB_NAME)
+    root = os.path.dirname(os.path.dirname(CSRC))
+    libdir, version = cfg("LIBDIR"), cfg("LDVERSION") or cfg("VERSION")
+    _run([os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared",
+          "-I", sysconfig.get_paths()["include"], f'-DNINFER_AMD_ROOT="{root}"',
+          *engine_api_sources(), "-o", lib + ".tmp", f"-L{libdir}", f"-Wl,-rpath,{libdir}",
+          f"-lpython{version}", "-ldl"])
+    os.replace(lib + ".tmp", lib)
+    _say(f"built {lib}")
+
+
+def engine_library() -> str:
+    """Path of the engine's C interface beside a kernel library that matches the sources."""
+    return os.path.join(os.path.dirname(ensure_built()), ENGINE_LIB_NAME)
 
 
 def ensure_built() -> str:
