@@ -153,7 +153,11 @@ def _compile_and_link(srcs: List[str], out_dir: str, jobs: int) -> str:
     _run([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-Wl,-z,defs", "-o", lib + ".tmp",
           *objs])
     os.replace(lib + ".tmp", lib)
-    _link_engine_api(out_dir)
+    try:
+        _link_engine_api(out_dir)
+    except (RuntimeError, OSError) as e:
+        # the engine runs without it (it serves host programs in C): say so and go on
+        _say(f"the engine's C interface was not built: {e}")
     with open(os.path.join(out_dir, "fingerprint"), "w") as f:
         f.write(_fingerprint())
     _say(f"built {lib} in {time.time() - t0:.0f} s")
@@ -179,7 +183,11 @@ def _link_engine_api(out_dir: str) -> None:
 
 def engine_library() -> str:
     """Path of the engine's C interface beside a kernel library that matches the sources."""
-    return os.path.join(os.path.dirname(ensure_built()), ENGINE_LIB_NAME)
+    path = os.path.join(os.path.dirname(ensure_built()), ENGINE_LIB_NAME)
+    if not os.path.isfile(path):
+        raise RuntimeError(f"{path} is missing: the host compiler or the interpreter's headers "
+                           "were not there when the kernel library was built")
+    return path
 
 
 def ensure_built() -> str:
