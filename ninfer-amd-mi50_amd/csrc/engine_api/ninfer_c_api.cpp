@@ -144,6 +144,25 @@ long long engine_number(ninfer_engine_t* e, const char* what) {
   return as_number(call("engine_number", "(Os)", e->obj, what), -1);
 }
 
+// the sessions' Python objects as a list (a new reference), or null with last_error set
+PyObject* session_list(ninfer_session_t** sessions, int n, const char* who) {
+  PyObject* list = PyList_New(n);
+  if (!list) {
+    last_error = fetch_exception();
+    return nullptr;
+  }
+  for (int i = 0; i < n; ++i) {
+    if (!sessions[i]) {
+      Py_DECREF(list);
+      last_error = std::string(who) + ": null session";
+      return nullptr;
+    }
+    Py_INCREF(sessions[i]->obj);
+    PyList_SET_ITEM(list, i, sessions[i]->obj);
+  }
+  return list;
+}
+
 }  // namespace
 
 extern "C" {
@@ -183,12 +202,19 @@ long long ninfer_kv_bytes_per_token(ninfer_engine_t* e) { return engine_number(e
 long long ninfer_kv_total_bytes(ninfer_engine_t* e) { return engine_number(e, "kv_total_bytes"); }
 long long ninfer_kv_seq_stride_elems(ninfer_engine_t* e) { return e ? 0 : -1; }
 
-int ninfer_kv_pages(ninfer_engine_t* e, long long* total, long long* free_pages) {
-  const long long t = engine_number(e, "pages_total"), f = engine_number(e, "pages_free");
-  if (t < 0 || f < 0) return -1;
-  if (total) *total = t;
-  if (free_pages) *free_pages = f;
-  return 0;
+long long ninfer_kv_pages_total(ninfer_engine_t* e) { return engine_number(e, "pages_total"); }
+long long ninfer_kv_pages_free(ninfer_engine_t* e) { return engine_number(e, "pages_free"); }
+long long ninfer_kv_pages_reused(ninfer_engine_t* e) { return engine_number(e, "pages_reused"); }
+
+int ninfer_tensor_read(ninfer_engine_t* engine, const char* name, long long offset, long long count,
+                       float* out) {
+  if (!engine || !name || !out || count < 0) {
+    last_error = "ninfer_tensor_read: null argument or negative count";
+    return -1;
+  }
+  Lock lock;
+  return (int)as_number(call("tensor_read", "(OsLLK)", engine->obj, name, offset, count,
+                             (unsigned long long)(uintptr_t)out), -1);
 }
 
 int ninfer_tokenize(ninfer_engine_t*, const char*, long long*, int) {
@@ -261,25 +287,63 @@ int ninfer_decode_batch(ninfer_engine_t* engine, ninfer_session_t** sessions, co
     return -1;
   }
   Lock lock;
-  PyObject* list = PyList_New(n);
-  if (!list) {
-    last_error = fetch_exception();
-    return -1;
-  }
-  for (int i = 0; i < n; ++i) {
-    if (!sessions[i]) {
-      Py_DECREF(list);
-      last_error = "ninfer_decode_batch: null session";
-      return -1;
-    }
-    Py_INCREF(sessions[i]->obj);
-    PyList_SET_ITEM(list, i, sessions[i]->obj);
-  }
+  PyObject* list = session_list(sessions, n, "ninfer_decode_batch");
+  if (!list) return -1;
   const int rc = (int)as_number(call("decode_batch", "(OOKKi)", engine->obj, list,
                                      (unsigned long long)(uintptr_t)tokens,
                                      (unsigned long long)(uintptr_t)out_logits, capacity), -1);
   Py_DECREF(list);
   return rc;
+}
+
+int ninfer_step(ninfer_engine_t* engine, ninfer_session_t** sessions, const int* q_len, int n_sessions,
+                const long long* tokens, const int* logit_rows, int n_rows, float* out_logits,
+                int capacity) {
+  if (!engine || !sessions || !q_len || !tokens || n_sessions <= 0 || n_rows < 0 ||
+      (n_rows > 0 && (!logit_rows || !out_logits))) {
+    last_error = "ninfer_step: null argument or no sessions";
+    return -1;
+  }
+  Lock lock;
+  PyObject* list = session_list(sessions, n_sessions, "ninfer_step");
+  if (!list) return -1;
+  const int rc = (int)as_number(call("step", "(OOKKKiKi)", engine->obj, list,
+                                     (unsigned long long)(uintptr_t)q_len,
+                                     (unsigned long long)(uintptr_t)tokens,
+                                     (unsigned long long)(uintptr_t)logit_rows, n_rows,
+                                     (unsigned long long)(uintptr_t)out_logits, capacity), -1);
+  Py_DECREF(list);
+  return rc;
+}
+
+long long ninfer_request_add(ninfer_engine_t* engine, const long long* prompt, int count, int max_new_tokens,
+                             float temperature, int top_k, float top_p, float repetition_penalty,
+                             unsigned long long seed, const long long* stop_ids, int n_stop) {
+  if (!engine || !prompt || count <= 0 || n_stop < 0 || (n_stop > 0 && !stop_ids)) {
+    last_error = "ninfer_request_add: null argument or no prompt";
+    return -1;
+  }
+  Lock lock;
+  return as_number(call("request_add", "(OKiififfKKi)", engine->obj, (unsigned long long)(uintptr_t)prompt,
+                        count, max_new_tokens, (double)temperature, top_k, (double)top_p,
+                        (double)repetition_penalty, seed, (unsigned long long)(uintptr_t)stop_ids, n_stop),
+                   -1);
+}
+
+int ninfer_run_step(ninfer_engine_t* engine) {
+  if (!engine) return -1;
+  Lock lock;
+  return (int)as_number(call("run_step", "(O)", engine->obj), -1);
+}
+
+int ninfer_request_take(ninfer_engine_t* engine, long long id, long long* out_tokens, int capacity) {
+  if (!engine || (capacity > 0 && !out_tokens) || capacity < 0) {
+    last_error = "ninfer_request_take: null argument";
+    return -1;
+  }
+  Lock lock;
+  return (int)as_number(call("request_take", "(OLKi)", engine->obj, id,
+                             (unsigned long long)(uintptr_t)out_tokens, capacity), -1);
 }
 
 long long ninfer_sample(ninfer_engine_t* engine, const float* logits, float temperature, int top_k, float top_p,

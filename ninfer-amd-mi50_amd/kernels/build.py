@@ -158,6 +158,9 @@ def _compile_and_link(srcs: List[str], out_dir: str, jobs: int) -> str:
     except (RuntimeError, OSError) as e:
         # the engine runs without it (it serves host programs in C): say so and go on
         _say(f"the engine's C interface was not built: {e}")
+        for stale in (ENGINE_LIB_NAME, ENGINE_LIB_NAME + ".tmp"):
+            if os.path.exists(os.path.join(out_dir, stale)):
+                os.remove(os.path.join(out_dir, stale))
     with open(os.path.join(out_dir, "fingerprint"), "w") as f:
         f.write(_fingerprint())
     _say(f"built {lib} in {time.time() - t0:.0f} s")

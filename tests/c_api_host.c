@@ -63,14 +63,30 @@ int main(int argc, char** argv) {
   printf("\n");
   if (ninfer_decode_batch(eng, both, tok_a, 2, logits, vocab) != -3) die("a short buffer must give -3");
 
-  long long total = 0, free_pages = 0;
-  if (ninfer_kv_pages(eng, &total, &free_pages) != 0 || free_pages >= total) die("pages in use");
+  const long long total = ninfer_kv_pages_total(eng);
+  if (total <= 0 || ninfer_kv_pages_free(eng) >= total) die("pages in use");
   ninfer_session_free(a);
   ninfer_session_free(b);
-  long long free_after = 0;
-  ninfer_kv_pages(eng, &total, &free_after);
-  if (free_after != total) die("pages given back");
+  if (ninfer_kv_pages_free(eng) != total) die("pages given back");
   printf("pages: %lld\n", total);
+
+  /* the engine's own scheduler: the same request and a second one, step by step */
+  const long long ra = ninfer_request_add(eng, prompt, n_prompt, n_new, 0.f, 0, 1.f, 1.f, 0, NULL, 0);
+  const long long rb = ninfer_request_add(eng, prompt + 2, n_prompt - 2, n_new, 0.f, 0, 1.f, 1.f, 0, NULL, 0);
+  if (ra < 0 || rb < 0 || ra == rb) die("ninfer_request_add");
+  long long out[64];
+  if (ninfer_request_take(eng, ra, out, 64) != -4) die("a request that has not run yet is not finished");
+  int left, steps = 0;
+  while ((left = ninfer_run_step(eng)) > 0) ++steps;
+  if (left < 0) die("ninfer_run_step");
+  const int got = ninfer_request_take(eng, ra, out, 64);
+  if (got != n_new) die("ninfer_request_take");
+  printf("scheduled:");
+  for (int i = 0; i < got; ++i) printf(" %lld", out[i]);
+  printf("\n");
+  if (ninfer_request_take(eng, ra, out, 64) != -1) die("a request is taken once");
+  if (ninfer_request_take(eng, rb, out, 64) != n_new) die("the second request");
+  if (ninfer_kv_pages_free(eng) != total || steps < n_new) die("after the scheduler");
   ninfer_engine_free(eng);
   return 0;
 }

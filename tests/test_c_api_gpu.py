@@ -32,7 +32,9 @@ def lib():
     lib.ninfer_last_error.restype = ctypes.c_char_p
     lib.ninfer_session_create.restype = ctypes.c_void_p
     lib.ninfer_sample.restype = ctypes.c_longlong
-    for name in ("ninfer_kv_bytes_per_token", "ninfer_kv_total_bytes", "ninfer_kv_seq_stride_elems"):
+    lib.ninfer_request_add.restype = ctypes.c_longlong
+    for name in ("ninfer_kv_bytes_per_token", "ninfer_kv_total_bytes", "ninfer_kv_seq_stride_elems",
+                 "ninfer_kv_pages_total", "ninfer_kv_pages_free", "ninfer_kv_pages_reused"):
         getattr(lib, name).restype = ctypes.c_longlong
     return lib
 
@@ -79,6 +81,36 @@ def test_c_interface_in_process(lib, model_dirs):
     t1 = lib.ninfer_sample(eng, logits, ctypes.c_float(0.9), 20, ctypes.c_float(0.9),
                            ctypes.c_float(1.1), ctypes.c_ulonglong(77))
     assert t1 == py.sample(np.ctypeslib.as_array(logits), 0.9, 20, 0.9, 1.1, 77)
+    # a mixed step: a portion of a second request's prompt beside the first one's next token
+    t_next = int(np.argmax(np.ctypeslib.as_array(logits)))
+    other = util.random_tokens(5, vocab, 8)
+    s2 = ctypes.c_void_p(lib.ninfer_session_create(eng))
+    sessions = (ctypes.c_void_p * 2)(s, s2)
+    q_len = (ctypes.c_int * 2)(1, 5)
+    flat = (ctypes.c_longlong * 6)(t_next, *other)
+    rows = (ctypes.c_int * 3)(0, 2, 5)
+    out3 = (ctypes.c_float * (3 * vocab))()
+    assert lib.ninfer_step(eng, sessions, q_len, 2, flat, rows, 3, out3, 3 * vocab - 1) == -3
+    assert lib.ninfer_step(eng, sessions, q_len, 2, flat, rows, 3, out3, 3 * vocab) == 0, lib.ninfer_last_error()
+    got = np.ctypeslib.as_array(out3).reshape(3, vocab)
+    ref_a = plain_model.forward(w, cfg, prompt + out + [t_next])[-1].numpy()
+    ref_b = plain_model.forward(w, cfg, other).numpy()
+    np.testing.assert_allclose(got[0], ref_a, atol=3e-5, rtol=1e-4)
+    np.testing.assert_allclose(got[1:], ref_b[[1, 4]], atol=3e-5, rtol=1e-4)
+    assert lib.ninfer_step(eng, sessions, q_len, 2, flat, None, 0, None, 0) == 0   # no logits wanted
+    assert lib.ninfer_session_length(s2) == 10
+    rows_bad = (ctypes.c_int * 2)(3, 1)
+    assert lib.ninfer_step(eng, sessions, q_len, 2, flat, rows_bad, 2, out3, 3 * vocab) == -1
+    lib.ninfer_session_free(s2)
+    # what the engine holds under a checkpoint name
+    name = "model.norm.weight"
+    buf = (ctypes.c_float * 7)()
+    assert lib.ninfer_tensor_read(eng, name.encode(), ctypes.c_longlong(3), ctypes.c_longlong(7), buf) == 0
+    np.testing.assert_array_equal(np.ctypeslib.as_array(buf), w[name].float().numpy()[3:10])
+    assert lib.ninfer_tensor_read(eng, b"no.such.tensor", ctypes.c_longlong(0), ctypes.c_longlong(1), buf) == -1
+    total = lib.ninfer_kv_pages_total(eng)
+    assert total == py.kv_pages()["total"] and 0 < lib.ninfer_kv_pages_free(eng) < total
+    assert lib.ninfer_kv_pages_reused(eng) >= 0
     # errors: a message and a negative code, and the engine goes on
     bad = (ctypes.c_longlong * 2)(vocab + 5, 1)
     assert lib.ninfer_prefill(s, bad, 2, logits, vocab) == -1
@@ -87,6 +119,31 @@ def test_c_interface_in_process(lib, model_dirs):
     lib.ninfer_session_reset(s)
     assert lib.ninfer_session_length(s) == 0
     lib.ninfer_session_free(s)
+    assert lib.ninfer_kv_pages_free(eng) == total
+    # the scheduler through the C interface gives what the Python entry point's gives: seeded
+    # sampling, a stop token, a request that can never fit
+    prompts = [util.safe_prompt(w, cfg, n, 40 + n) for n in (9, 21, 14)]
+    params = ninfer_amd.SamplingParams(0.8, 20, 0.9, 1.05, 123, 7)
+    ids = []
+    for p in prompts:
+        arr = (ctypes.c_longlong * len(p))(*p)
+        ids.append(lib.ninfer_request_add(eng, arr, len(p), 7, ctypes.c_float(0.8), 20, ctypes.c_float(0.9),
+                                          ctypes.c_float(1.05), ctypes.c_ulonglong(123), None, 0))
+    assert ids == [0, 1, 2]
+    long_prompt = (ctypes.c_longlong * 95)(*([1] * 95))
+    too_long = lib.ninfer_request_add(eng, long_prompt, 95, 7, ctypes.c_float(0.0), 0, ctypes.c_float(1.0),
+                                      ctypes.c_float(1.0), ctypes.c_ulonglong(0), None, 0)
+    while lib.ninfer_run_step(eng) > 0:
+        pass
+    want = py.generate(prompts, params, stop_ids=[])
+    outbuf = (ctypes.c_longlong * 16)()
+    for rid, ref_tokens in zip(ids, want):
+        assert lib.ninfer_request_take(eng, ctypes.c_longlong(rid), outbuf, 3) == -3
+        n = lib.ninfer_request_take(eng, ctypes.c_longlong(rid), outbuf, 16)
+        assert list(outbuf[:n]) == ref_tokens
+    assert lib.ninfer_request_take(eng, ctypes.c_longlong(too_long), outbuf, 16) == -1
+    assert b"max_context" in lib.ninfer_last_error()
+    assert lib.ninfer_request_take(eng, ctypes.c_longlong(99), outbuf, 16) == -1
     lib.ninfer_engine_free(eng)
     eng2 = ctypes.c_void_p()
     for quant, parallel, gpus in ((b"q4", None, 1), (None, b"tp", 1), (None, None, 2)):
@@ -116,4 +173,5 @@ def test_c_interface_from_a_c_program(model_dirs, tmp_path):
     want = plain_model.greedy_generate(w, cfg, prompt, 5)
     assert [int(t) for t in lines["a"].split()] == want
     assert [int(t) for t in lines["batch"].split()] == want
+    assert [int(t) for t in lines["scheduled"].split()] == want
     assert int(lines["pages"]) > 0
