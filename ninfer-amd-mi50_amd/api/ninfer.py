@@ -116,6 +116,11 @@ class Ninfer:
         return self.runner.cache.kv_bytes_per_token(2 if self.options.dtype == "bfloat16" else 4)
 
     @property
+    def state_bytes_per_request(self) -> int:
+        """Fixed-size state of a request, apart from its pages (0 for this architecture)."""
+        return self.runner.cache.state_bytes_per_request()
+
+    @property
     def kv_total_bytes(self) -> int:
         c = self.runner.cache
         return sum(t.numel() * t.element_size() for pools in c.pools.values()

@@ -238,6 +238,12 @@ class CacheManager:
         return g.rows[np.asarray(slots, dtype=np.intp), :width]   # a copy
 
     # ---- introspection -------------------------------------------------------
+    def state_bytes_per_request(self) -> int:
+        """Bytes of fixed-size state a request holds whatever its length (32-bit floats of every
+        mixer that keeps such state): reported apart from the pages' bytes per token, so that
+        whoever sizes the cache can count both."""
+        return 4 * self.state_floats
+
     def kv_bytes_per_token(self, bytes_per_element: int) -> int:
         """Bytes of paged cache one token takes over all cache instances; pools without a
         dtype of their own count `bytes_per_element` per number."""

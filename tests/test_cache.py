@@ -125,6 +125,12 @@ def test_window_gives_pages_back_as_it_passes():
     assert m.pages_free(0) == 8 and m.pages_free(1) == 8
 
 
+def test_state_bytes_are_reported_apart_from_the_pages():
+    m = CacheManager([CacheNeed.keys_values(2, 8), None], 4, 8, 3, 32, state_floats=10)
+    assert m.state_bytes_per_request() == 40 and m.kv_bytes_per_token(2) == 2 * 2 * 8 * 2
+    assert manager().state_bytes_per_request() == 0
+
+
 def test_slots_run_out_and_come_back():
     m = manager(seqs=2)
     a, b = m.acquire(), m.acquire()
