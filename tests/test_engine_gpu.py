@@ -96,6 +96,31 @@ def test_pages_given_back_are_never_read(case, dtype):
         assert torch.isnan(k_pool).any(), "pages were given back, so some are poisoned now"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_logits_do_not_depend_on_where_the_cache_puts_a_request(case, dtype):
+    """The same request in a fresh engine (slot 0, pages 0, 1, 2, ...), and in one whose free
+    pages were shuffled and whose first slots other requests hold: the same logits bit for
+    bit. With another page size: the same within rounding (the kernels walk other tiles)."""
+    import random
+    from ninfer_amd import Chunk
+    rid, toks = "r3", case["reqs"]["r3"]
+    first = util.run_schedule(make_runner(case, dtype, 8, 40), util.schedule_portions(rid, toks, 1))[rid]
+    runner = make_runner(case, dtype, 8, 40)
+    for g in runner.cache.groups:
+        random.Random(5).shuffle(g.allocator._free)
+    held = [runner.open() for _ in range(2)]           # the request gets the third slot
+    runner.step([Chunk(held[0], [1, 2, 3], [])])
+    again = util.run_schedule(runner, util.schedule_portions(rid, toks, 1))[rid]
+    assert torch.equal(first, again)
+    for s in held:
+        runner.close(s)
+    runner.cache.check()
+    other = util.run_schedule(make_runner(case, dtype, 16, 20), util.schedule_portions(rid, toks, 1))[rid]
+    torch.testing.assert_close(other, first, **bound(dtype))
+    if dtype == "float32":
+        assert torch.equal(other, first), "the 32-bit kernels sum in the same order whatever the page"
+
+
 def test_32bit_does_not_depend_on_the_cut(case):
     """In 32-bit every way of cutting gives the same logits to the last bit or
     nearly so (far inside the bound against the plain implementation)."""
