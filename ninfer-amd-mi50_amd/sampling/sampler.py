@@ -99,6 +99,33 @@ class Sampler:
     def __init__(self, ops, device):
         self.ops = ops
         self.device = device
+        self._staging: List[list] = []   # pinned buffers (and the event after each one's copy)
+        self._staging_next = 0
+
+    def _to_device(self, packed: np.ndarray) -> torch.Tensor:
+        """The rows' packed parameters on the device, through one of a few pinned buffers used in
+        turn: the copy is queued behind the step that makes the logits and the host goes on (a
+        copy out of pageable memory makes the host wait until the device has reached it, and the
+        sampling kernel would then be launched only after the step has ended)."""
+        host = torch.from_numpy(packed)
+        if self.device.type != "cuda":
+            return host.to(self.device)
+        n = host.numel()
+        if len(self._staging) < 4:
+            self._staging.append([torch.empty(max(n, 1024), dtype=torch.int32).pin_memory(),
+                                  torch.cuda.Event()])
+            slot = self._staging[-1]
+        else:
+            slot = self._staging[self._staging_next]
+            self._staging_next = (self._staging_next + 1) % len(self._staging)
+            slot[1].synchronize()
+            if slot[0].numel() < n:
+                slot[0] = torch.empty(2 * n, dtype=torch.int32).pin_memory()
+        slot[0][:n].copy_(host)
+        dev = torch.empty(n, dtype=torch.int32, device=self.device)
+        dev.copy_(slot[0][:n], non_blocking=True)
+        slot[1].record()
+        return dev
 
     def sample(self, logits: torch.Tensor, rows: Sequence[SampleRow]) -> List[int]:
         """One token per row of `logits` [R, vocab]."""
@@ -127,7 +154,7 @@ class Sampler:
         top_k = np.asarray([row.params.top_k for row in rows], np.int32)
         n_pen = int(pen_o[-1])
         packed = np.concatenate([floats.reshape(-1).view(np.int32), top_k, pen_o] + pen_t + pen_c)
-        dev = torch.from_numpy(packed).to(self.device)
+        dev = self._to_device(packed)
         f = dev[:4 * r].view(torch.float32)
         o = 4 * r
         pen = {}
