@@ -5,9 +5,14 @@
 using namespace ninfer;
 
 // many rows per weight matrix: 64-row tiles and taller; few: 16-row tiles that stream the
-// weights (a product with few output features has too few 128-wide tiles to fill the GPU)
+// weights (a product with few output features has too few 128-wide tiles to fill the GPU).
+// Grouped products count as many above 8 rows a group on average: some groups then have
+// several 16-row tiles, each of which would stream the group's weights again (60 groups of
+// 2 x 1408 x 2048 and 2048 x 1408: a 224-token portion 6.4 against 7.6 ms, 160 tokens 5.8
+// against 6.4, the same at 8 and below; 64 groups of 2 x 2560 x 3584: 127 tokens 22.4 against 28.0,
+// 80 tokens 21.7 against 23.1)
 static bool many_rows(const GemmArgs& a) {
-  return a.offsets ? a.M >= 16 * a.groups : (a.M > 32 && a.N > 128);
+  return a.offsets ? a.M > 8 * a.groups : (a.M > 32 && a.N > 128);
 }
 
 // force_generic != 0 runs the plain tiled kernel whatever the shape (tests

@@ -131,7 +131,9 @@ class _Together:
 class _Beside:
     """Work on a second stream that starts after everything the current stream has been
     given so far; `HipOps.join()` makes the current stream wait for it. The two events are
-    made once and recorded again every time (an event's earlier waits keep their meaning).
+    made once and recorded again every time (an event's earlier waits keep their meaning);
+    a record and its wait are one call into the library (torch's event and stream objects
+    cost the host some 40 us a block, a third of a layer's launches).
 
     Memory: tensors made inside the block come from the second stream's part of torch's
     allocator and are read on the main stream after `join()` without `record_stream`. That
@@ -147,19 +149,20 @@ class _Beside:
         ops = self.ops
         if ops._side is None:
             ops._side = torch.cuda.Stream()   # default priority
-            ops._side_events = (torch.cuda.Event(), torch.cuda.Event())
-        self.main = torch.cuda.current_stream()
+            ops._side_events = (ops._new_event(), ops._new_event())
+        raw = ops._stream().value or 0
+        if ops._main is None or ops._main.cuda_stream != raw:
+            ops._main = torch.cuda.current_stream()   # the object is kept: making one costs
         if ops._side_open:   # a block that nobody joined (a step that failed half-way): join it now
-            self.main.wait_event(ops._side_events[1])
-            ops._side_open = False
-        ops._side_events[0].record(self.main)
-        ops._side.wait_event(ops._side_events[0])
+            ops.join()
+        ops._ok(ops.lib.ninfer_stream_after(ops._side.cuda_stream, raw, ops._side_events[0]))
         torch.cuda.set_stream(ops._side)
         return self
 
     def __exit__(self, exc_type, exc, tb):
-        self.ops._side_events[1].record(self.ops._side)
-        torch.cuda.set_stream(self.main)
+        # nothing is given to the second stream outside such blocks: the event that marks the
+        # block's end is recorded by `join()`, together with the wait for it
+        torch.cuda.set_stream(self.ops._main)
         self.ops._side_open = True
         return False
 
@@ -184,6 +187,8 @@ class HipOps:
         self.lib = ctypes.CDLL(self.lib_path)
         self.lib.ninfer_last_error.restype = ctypes.c_char_p
         self.lib.ninfer_attention_workspace_floats.restype = ctypes.c_longlong
+        self.lib.ninfer_event_create.restype = ctypes.c_void_p
+        self.lib.ninfer_stream_after.argtypes = [ctypes.c_void_p] * 3
         self.lib.ninfer_sample_few_places.restype = ctypes.c_longlong
         self.force_generic = False  # tests: run the plain kernels whatever the shape
         self._device_index = None   # the one GPU's index, asked for at the first launch
@@ -192,10 +197,12 @@ class HipOps:
         self._side = None           # the second stream of `beside()`, made at first use
         self._side_events = None    # (start, end) of the `beside()` block
         self._side_open = False     # a `beside()` block that `join()` has not waited for
-        # rows from which independent work is worth a second stream (switching streams costs the
-        # host about 0.03 ms a layer, and short portions are bound by the host: the smaller
-        # model's portion of 256 tokens 7.3 ms with it, 6.5 without; 512 tokens 7.5 against 7.7,
-        # 1,024 9.5 against 10.3, 2,048 13.7 against 15.1)
+        self._main = None           # the stream that the last `beside()` block left and returns to
+        # rows from which independent work is worth a second stream (with fewer rows the
+        # products on it lose more by sharing the units than the step gains: the smaller
+        # model's portion of 256 tokens 7.6 ms with it, 6.6 without; 512 tokens 7.5 against 7.8,
+        # 1,024 9.5 against 10.3, 2,048 13.6 against 15.0; the two waits between the streams
+        # alone cost 0.1 to 0.2 ms a step)
         self.beside_min_rows = 512
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
         # ... but never a SwiGLU's gate/up product: the tile kernels here have the activation in
@@ -204,6 +211,11 @@ class HipOps:
         # prompt portions of 256 to 8,192 tokens 2 to 4% faster at 2048 -> 2 x 5632, the same
         # within 1% at 3584 -> 2 x 20480)
         self.split_max_rows = 512   # most rows of a product that may be cut along K (gemm_split)
+        # a plain product of at most this many rows runs on the tile kernel here when it is on
+        # the second stream: the library's product there took the 512-token portion 7.25 ms in
+        # some processes and 8.2 in others (7.5 to 7.8 with the tile kernel in all of them),
+        # 576 tokens 8.17 against 7.9, 640 tokens 8.05 to 8.2 against 8.0; from 704 rows the same
+        self.side_own_max_rows = 640
         self._attn_ws = None
         self._outgrown = []     # workspaces that captured graphs may still point to
         self._split_ws = None   # 32 MB of 32-bit scratch for products cut along K, made at first use
@@ -480,8 +492,7 @@ class HipOps:
             # along K (its output tiles alone would not fill the GPU). The one workspace of
             # the cut belongs to the main stream: on the second stream nothing is cut (the
             # library's product runs instead).
-            if self._side is not None \
-                    and torch.cuda.current_stream().cuda_stream == self._side.cuda_stream:
+            if self._on_side():
                 return False
             if self._split_ws is None:
                 self._split_ws = torch.empty(1 << 23, dtype=torch.float32, device=a.device)
@@ -496,6 +507,14 @@ class HipOps:
             return
         self._ok(self.lib.ninfer_gemm(ctypes.byref(args), 1 if self.force_generic else 0,
                                       self._stream()))
+
+    def _on_side(self) -> bool:
+        return self._side is not None and (self._stream().value or 0) == self._side.cuda_stream
+
+    def _new_event(self) -> ctypes.c_void_p:
+        ev = self.lib.ninfer_event_create()
+        _need(ev, "no event: " + self.lib.ninfer_last_error().decode())
+        return ctypes.c_void_p(ev)
 
     def together(self):
         """Context manager for products that do not depend on each other: the
@@ -523,7 +542,8 @@ class HipOps:
     def join(self) -> None:
         """The current stream waits for the `beside()` block before."""
         if self._side_open:
-            torch.cuda.current_stream().wait_event(self._side_events[1])
+            self._ok(self.lib.ninfer_stream_after(self._stream(), self._side.cuda_stream,
+                                                  self._side_events[1]))
             self._side_open = False
 
     def _launch_held(self, held, route=None):
@@ -566,7 +586,8 @@ class HipOps:
         if bias is not None:
             _dev(bias, "bias", torch.float32, 1)
             _need(bias.shape[0] == w.shape[0], "linear: bias has the wrong size")
-        if self._use_library(x, out) and bias is None:
+        if self._use_library(x, out) and bias is None and not (
+                x.shape[0] <= self.side_own_max_rows and self._on_side()):
             if x.shape[0] > self.split_max_rows or not self._gemm(
                     x, w, out, m=x.shape[0], n=w.shape[0], k=x.shape[1], only_if_split=True):
                 torch.matmul(x, w.t(), out=out)

@@ -343,20 +343,26 @@ def test_long_prompt_on_the_many_row_kernels(wide_case, dtype):
     runner = load_model(dirs[dtype], EngineOptions(dtype=dtype, max_context=704, prefill_chunk=640,
                                                    num_sequences=2, page_size=16))
     # with the shared expert on a stream of its own beside the routed path (the engine does so
-    # from 1,024 rows), and on one stream: the same kernels, the same bits; and a second run
+    # from 512 rows), and on one stream: the same kernels, the same bits; and a second run
     # gives them again (no result depends on the order in which the grouping's counters placed
-    # an expert's rows)
+    # an expert's rows). The rule that gives a product on the second stream to another kernel
+    # than on the first is off for that comparison, and on for a run of its own.
     ops = runner.ops
-    saved = ops.beside_min_rows
+    saved = ops.beside_min_rows, ops.side_own_max_rows
     try:
-        ops.beside_min_rows = 512
+        ops.beside_min_rows, ops.side_own_max_rows = 512, 0
         whole = util.run_schedule(runner, util.schedule_whole("a", toks))["a"]
         assert ops._side is not None and not ops._side_open
         again = util.run_schedule(runner, util.schedule_whole("a2", toks))["a2"]
         ops.beside_min_rows = 1 << 30
         one_stream = util.run_schedule(runner, util.schedule_whole("a1", toks))["a1"]
+        ops.beside_min_rows, ops.side_own_max_rows = 512, 1 << 30
+        other_kernel = util.run_schedule(runner, util.schedule_whole("a3", toks))["a3"]
+        other_again = util.run_schedule(runner, util.schedule_whole("a4", toks))["a4"]
     finally:
-        ops.beside_min_rows = saved
+        ops.beside_min_rows, ops.side_own_max_rows = saved
+    torch.testing.assert_close(other_kernel, ref, **bound(dtype), msg=lambda m: f"other: {m}")
+    assert torch.equal(other_again, other_kernel)
     torch.testing.assert_close(whole, ref, **bound(dtype), msg=lambda m: f"whole: {m}")
     assert torch.equal(one_stream, whole) and torch.equal(again, whole)
     cut = [("b", toks[:200], list(range(200))), ("b", toks[200:260], list(range(60))),
