@@ -528,12 +528,15 @@ def test_routing_launched_with_the_products(ops_mode, gen, dtype, t, e, k, h, sh
 
 @pytest.mark.parametrize("counts", [[17, 31, 32, 33, 63], [64, 65, 127, 128, 129], [255, 256, 257, 300, 16],
                                     [511, 512, 513, 20, 700], [16, 16, 200, 16, 290], [69, 70, 71, 72, 73],
-                                    [96, 97, 160, 161, 192, 193, 224, 225]])
+                                    [96, 97, 160, 161, 192, 193, 224, 225],
+                                    [0, 1, 2, 40, 9], [9, 9, 9, 9, 10], [0, 0, 0, 0, 41], [1, 1, 1, 1, 60]])
 @pytest.mark.parametrize("h,inner", [(256, 192), (2048, 1408)])
 def test_grouped_products_at_the_edges_of_the_row_blocks(ops, gen, counts, h, inner):
     """Chosen rows per expert around the 32-row blocks and the 256-row tiles of the tall
     tile kernel, which loads and multiplies only the blocks that hold rows: an expert with one
-    row more or fewer than a block, a tile and a row, two tiles and a row."""
+    row more or fewer than a block, a tile and a row, two tiles and a row; and just above the
+    8 rows per expert on average from which that kernel is picked, with experts of no row, one
+    row and two."""
     from ninfer_amd.parts.moe import Routing
     plain = PlainOps()
     dtype = torch.bfloat16
