@@ -204,6 +204,13 @@ class HipOps:
         # 1,024 9.5 against 10.3, 2,048 13.6 against 15.0; the two waits between the streams
         # alone cost 0.1 to 0.2 ms a step)
         self.beside_min_rows = 512
+        # ... and from far fewer rows where the work on the second stream reads a lot of
+        # weights, so that it is long whatever the rows (a shared expert of 440 MB beside 64
+        # experts of 55 MB: 64 rows 20.8 against 21.0 ms, 128 rows 21.6 against 22.6, 256 rows
+        # 23.4 against 25.1, 448 rows 26.2 against 29.8; the smaller model's 69 MB beside 60
+        # experts of 17 MB: 128 to 448 rows 7.6 to 7.8 ms with it, 5.6 to 7.5 without)
+        self.beside_heavy_min_rows = 64
+        self.beside_heavy_bytes = 256 << 20
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
         # ... but never a SwiGLU's gate/up product: the tile kernels here have the activation in
         # their epilogue, which beats the library's product followed by a kernel for the
@@ -214,8 +221,11 @@ class HipOps:
         # a plain product of at most this many rows runs on the tile kernel here when it is on
         # the second stream: the library's product there took the 512-token portion 7.25 ms in
         # some processes and 8.2 in others (7.5 to 7.8 with the tile kernel in all of them),
-        # 576 tokens 8.17 against 7.9, 640 tokens 8.05 to 8.2 against 8.0; from 704 rows the same
+        # 576 tokens 8.17 against 7.9, 640 tokens 8.05 to 8.2 against 8.0; from 704 rows the same.
+        # That product's weights are 23 MB; with 147 MB (3584 x 20480) the library's is the
+        # faster one there too (64 to 640 rows: steps up to 3% shorter), hence the second bound
         self.side_own_max_rows = 640
+        self.side_own_max_bytes = 64 << 20
         self._attn_ws = None
         self._outgrown = []     # workspaces that captured graphs may still point to
         self._split_ws = None   # 32 MB of 32-bit scratch for products cut along K, made at first use
@@ -524,11 +534,14 @@ class HipOps:
         are valid after the block, not inside it."""
         return _Together(self)
 
-    def wants_beside(self, rows: int) -> bool:
-        """Is independent work of this many rows worth the second stream? Not while a graph
-        is being captured: its steps have few rows each, and a fork inside a capture is
-        one more thing a replay would have to get right."""
-        return rows >= self.beside_min_rows and not torch.cuda.is_current_stream_capturing()
+    def wants_beside(self, rows: int, weight_bytes: int = 0) -> bool:
+        """Is independent work of this many rows, which reads this many bytes of weights, worth
+        the second stream? Not while a graph is being captured: its steps have few rows each,
+        and a fork inside a capture is one more thing a replay would have to get right."""
+        if rows < self.beside_min_rows and (rows < self.beside_heavy_min_rows
+                                            or weight_bytes < self.beside_heavy_bytes):
+            return False
+        return not torch.cuda.is_current_stream_capturing()
 
     def beside(self):
         """Context manager for work that nothing on the current stream waits for until
@@ -587,7 +600,8 @@ class HipOps:
             _dev(bias, "bias", torch.float32, 1)
             _need(bias.shape[0] == w.shape[0], "linear: bias has the wrong size")
         if self._use_library(x, out) and bias is None and not (
-                x.shape[0] <= self.side_own_max_rows and self._on_side()):
+                x.shape[0] <= self.side_own_max_rows
+                and w.numel() * w.element_size() <= self.side_own_max_bytes and self._on_side()):
             if x.shape[0] > self.split_max_rows or not self._gemm(
                     x, w, out, m=x.shape[0], n=w.shape[0], k=x.shape[1], only_if_split=True):
                 torch.matmul(x, w.t(), out=out)

@@ -53,6 +53,10 @@ class SwiGLU(FeedForward):
             w.hold(p + "up_proj.bias", self.b_gate_up[self.inner:])
             self.b_down = w.float32(p + "down_proj.bias")
 
+    def weight_bytes(self) -> int:
+        """What one pass over the two weight matrices reads."""
+        return 3 * self.inner * self.hidden * self.w_down.element_size()
+
     def gate_up(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
         h = ctx.empty((x.shape[0], self.inner))
         ctx.ops.swiglu_linear(x, self.w_gate_up, h, act=self.act, bias=self.b_gate_up)

@@ -206,7 +206,7 @@ class SparseMoE(FeedForward):
         # they run on a stream of their own beside the routed path, whose kernels leave part
         # of the device empty in their last round of blocks.
         logits = ctx.empty((x.shape[0], self.router.experts + 1), torch.float32)
-        if ctx.ops.wants_beside(x.shape[0]):
+        if ctx.ops.wants_beside(x.shape[0], self.shared.weight_bytes()):
             # routing first: its short kernels would crawl beside the shared expert's long ones
             ctx.ops.linear(x, self.router_and_gate, logits)
             routing = self.router.route(ctx, logits)

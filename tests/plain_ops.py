@@ -28,7 +28,7 @@ class PlainOps:
 
     beside_min_rows = 8   # low, so that the host tests walk the many-row branch too
 
-    def wants_beside(self, rows):
+    def wants_beside(self, rows, weight_bytes=0):
         return rows >= self.beside_min_rows
 
     def beside(self):
