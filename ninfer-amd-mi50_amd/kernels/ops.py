@@ -209,7 +209,8 @@ class HipOps:
         # experts of 55 MB: 64 rows 20.8 against 21.0 ms, 128 rows 21.6 against 22.6, 256 rows
         # 23.4 against 25.1, 448 rows 26.2 against 29.8; the smaller model's 69 MB beside 60
         # experts of 17 MB: 128 to 448 rows 7.6 to 7.8 ms with it, 5.6 to 7.5 without)
-        self.beside_heavy_min_rows = 64
+        # (65: a decode step of up to 64 rows takes the same kernels run eagerly and captured)
+        self.beside_heavy_min_rows = 65
         self.beside_heavy_bytes = 256 << 20
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
         # ... but never a SwiGLU's gate/up product: the tile kernels here have the activation in

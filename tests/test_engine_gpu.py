@@ -363,13 +363,13 @@ def test_long_prompt_on_the_many_row_kernels(wide_case, dtype):
         ops.beside_min_rows, ops.side_own_max_rows = saved
     torch.testing.assert_close(other_kernel, ref, **bound(dtype), msg=lambda m: f"other: {m}")
     assert torch.equal(other_again, other_kernel)
-    # the second stream from 64 rows on, as for a shared expert with very large weights
+    # the second stream from 65 rows on, as for a shared expert with very large weights
     saved = ops.beside_heavy_bytes, ops.side_own_max_rows
     try:
         ops.side_own_max_rows = 0
         few_one = util.run_schedule(runner, util.schedule_whole("f1", toks[:90]))["f1"]
         ops.beside_heavy_bytes = 0
-        assert ops.wants_beside(90, 1) and not ops.wants_beside(63, 1)
+        assert ops.wants_beside(90, 1) and not ops.wants_beside(64, 1)
         few_two = util.run_schedule(runner, util.schedule_whole("f2", toks[:90]))["f2"]
     finally:
         ops.beside_heavy_bytes, ops.side_own_max_rows = saved
