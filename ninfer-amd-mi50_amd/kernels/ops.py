@@ -132,8 +132,8 @@ class _Beside:
     """Work on a second stream that starts after everything the current stream has been
     given so far; `HipOps.join()` makes the current stream wait for it. The two events are
     made once and recorded again every time (an event's earlier waits keep their meaning);
-    a record and its wait are one call into the library (torch's event and stream objects
-    cost the host some 40 us a block, a third of a layer's launches).
+    a record and its wait are one call into the library (with torch's event and stream
+    objects a block cost the host some 100 us, half of a layer's launches).
 
     Memory: tensors made inside the block come from the second stream's part of torch's
     allocator and are read on the main stream after `join()` without `record_stream`. That
