@@ -1238,3 +1238,22 @@ def test_router_rows_without_a_softmax_still_choose(ops, t):
     assert torch.isfinite(w[0]).all() and torch.isfinite(w[3:]).all()
     for row in ids.tolist():
         assert len(set(row)) == k
+
+
+def test_one_stream_after_another(ops):
+    """The library's record-and-wait call: work given to the later stream after it sees
+    everything the earlier stream had been given before it, and a missing event is refused."""
+    earlier, later = torch.cuda.Stream(), torch.cuda.Stream()
+    x = torch.zeros(1 << 26, device="cuda")
+    torch.cuda.synchronize()
+    event = ops._new_event()
+    with torch.cuda.stream(earlier):
+        for _ in range(8):
+            x.add_(1.0)
+    ops._ok(ops.lib.ninfer_stream_after(later.cuda_stream, earlier.cuda_stream, event))
+    with torch.cuda.stream(later):
+        y = x[::4097].clone()
+    torch.cuda.synchronize()
+    assert float(y.min()) == 8.0 and float(y.max()) == 8.0
+    assert ops.lib.ninfer_stream_after(later.cuda_stream, earlier.cuda_stream, None) == -1
+    assert b"no event" in ops.lib.ninfer_last_error()
