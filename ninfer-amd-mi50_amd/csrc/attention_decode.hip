@@ -29,16 +29,18 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kDecWaves = 4;
 
-// Keys per block: 128, or 256 from 24 blocks a CU on. Blocks live long (all of a CU's share
+// Keys per block: 128, or 256 above 24 blocks a CU. Blocks live long (all of a CU's share
 // the CU's part of the memory system), so with few rounds of them the last ones to finish
 // leave the device half empty for a while, and shorter blocks end more evenly: 8 rows x 8,192
 // keys take 82 us with 128 keys a block against 85 to 87 with 256, and the step 1.5% less
 // (4,991 to 5,025 against 5,064 to 5,104 us in one process). From 16 rows on the larger
 // blocks win the step (7,964 to 7,975 against 8,003 to 8,098 us; 64 rows: 633 against 651 us
-// a layer: half the partial results to write and merge).
+// a layer: half the partial results to write and merge). At 24 blocks a CU: 8 rows x 12,288
+// keys 6,005 to 6,011 us a step against 6,058, 12 rows x 8,192 the same; at 32 (8 x 16,384)
+// the larger blocks by 1%.
 static int decode_chunk(int T, int Hkv, int max_kv_len) {
   long blocks = (long)T * Hkv * ((max_kv_len + 255) / 256);
-  return blocks < 24L * device_cu_count() ? 128 : 256;
+  return blocks <= 24L * device_cu_count() ? 128 : 256;
 }
 
 __device__ __forceinline__ void cvt8(const bf16x8& v, float* f) {
