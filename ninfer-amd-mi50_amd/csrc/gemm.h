@@ -111,6 +111,8 @@ __device__ inline bool grouped_tile(const GemmArgs& a, const int* __restrict__ t
 int gemm_check(const GemmArgs& a);
 bool gemm_skinny_takes(const GemmArgs& a);
 int gemm_skinny(const GemmArgs& a, hipStream_t stream);
+bool gemm_skinny_rows_takes(const GemmArgs& a);
+int gemm_skinny_rows(const GemmArgs& a, hipStream_t stream);
 bool gemm_skinny_pair_takes(const GemmArgs& a, const GemmArgs& b);
 int gemm_skinny_pair(const GemmArgs& a, const GemmArgs& b, hipStream_t stream);
 struct RouteArgs;

@@ -23,6 +23,7 @@ extern "C" int ninfer_gemm(const GemmArgs* args, int force_generic, hipStream_t 
   const GemmArgs& a = *args;
   if (!force_generic) {
     if (gemm_split_parts(a) >= 2) return gemm_split(a, stream);
+    if (gemm_skinny_rows_takes(a)) return gemm_skinny_rows(a, stream);
     if (many_rows(a) && gemm_tile_takes(a)) return gemm_tile(a, stream);
     if (gemm_skinny_takes(a)) return gemm_skinny(a, stream);
   }

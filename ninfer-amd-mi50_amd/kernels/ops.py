@@ -213,6 +213,8 @@ class HipOps:
         self.beside_heavy_min_rows = 65
         self.beside_heavy_bytes = 256 << 20
         self.library_min_rows = 32  # dense bf16 products with more rows go to the library
+        self.rows_kernel_max = 64   # ... unless the kernel for 33 to 64 rows takes them
+        self.rows_kernel_features = (4096, 32768)   # (gemm_skinny_rows.hip: where it beats the library)
         # ... but never a SwiGLU's gate/up product: the tile kernels here have the activation in
         # their epilogue, which beats the library's product followed by a kernel for the
         # activation at every row count (70 against 98 us at 64 rows of 40960 x 3584; whole
@@ -600,7 +602,7 @@ class HipOps:
         if bias is not None:
             _dev(bias, "bias", torch.float32, 1)
             _need(bias.shape[0] == w.shape[0], "linear: bias has the wrong size")
-        if self._use_library(x, out) and bias is None and not (
+        if self._use_library(x, out, w) and bias is None and not (
                 x.shape[0] <= self.side_own_max_rows
                 and w.numel() * w.element_size() <= self.side_own_max_bytes and self._on_side()):
             if x.shape[0] > self.split_max_rows or not self._gemm(
@@ -609,13 +611,19 @@ class HipOps:
             return
         self._gemm(x, w, out, m=x.shape[0], n=w.shape[0], k=x.shape[1], bias=bias)
 
-    def _use_library(self, x, out) -> bool:
+    def _use_library(self, x, out, w) -> bool:
         """Plain dense products of many bf16 rows go to the vendor library, as
         the reference sends every multi-row product to rocBLAS
         (src/ops/linear.hip:21-35); few rows, 32-bit, grouped and fused products
-        run on the hand-written kernels."""
-        return (not self.force_generic and x.dtype == torch.bfloat16 and out.dtype == x.dtype
-                and x.shape[0] > self.library_min_rows)
+        run on the hand-written kernels, and so do products of up to `rows_kernel_max` rows
+        whose sizes the kernel for them takes (gemm_skinny_rows.hip)."""
+        if self.force_generic or x.dtype != torch.bfloat16 or out.dtype != x.dtype:
+            return False
+        rows = x.shape[0]
+        if rows <= self.rows_kernel_max and w.shape[0] % 32 == 0 and w.shape[1] % 128 == 0 \
+                and self.rows_kernel_features[0] <= w.shape[0] <= self.rows_kernel_features[1]:
+            return False
+        return rows > self.library_min_rows
 
     @staticmethod
     def _gate_epilogue(act: str) -> int:

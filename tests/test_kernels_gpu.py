@@ -178,7 +178,11 @@ def test_linear_cut_along_k(ops, gen, m, n, k):
         assert ops._gemm(x, w, o1, m=m, n=n, k=k, only_if_split=True), "not cut along K"
         PlainOps().linear(x, w, o2)
         close(o1, o2, torch.bfloat16, scale=math.sqrt(k))
-        if not ops.force_generic:   # (another test's fixture may have switched the fast kernels off)
+        # (another test's fixture may have switched the fast kernels off; and up to 64 rows
+        # `linear` prefers the kernel that streams the weights past all rows, where it takes
+        # the sizes)
+        if not ops.force_generic and (m > ops.rows_kernel_max or n % 32 or k % 128
+                                      or not 4096 <= n <= 32768):
             ops.linear(x, w, o3)
         else:
             ops._gemm(x, w, o3, m=m, n=n, k=k, only_if_split=True)
@@ -191,6 +195,33 @@ def test_linear_cut_along_k(ops, gen, m, n, k):
         close(f1, f2, torch.float32, scale=200 * math.sqrt(k))
     if n * k * 2 < (48 << 20):   # by default only long weight streams are cut
         assert not ops._gemm(x, w, o3, m=m, n=n, k=k, only_if_split=True)
+
+
+@pytest.mark.parametrize("m,n,k", [(33, 4096, 2048), (48, 6144, 2048), (49, 4128, 5632),
+                                   (64, 8192, 640), (40, 32768, 128), (57, 4608, 1024)])
+def test_linear_of_33_to_64_rows(ops, gen, m, n, k):
+    """Dense bf16 products of 33 to 64 rows on the kernel that reads every weight once for all
+    the rows (three or four row tiles of 16 per block): against the plain product, with and
+    without a bias, bf16 and 32-bit results; nothing written beyond the rows; and a row's
+    bits are the same among 33 rows as among all (each row tile has its own accumulator)."""
+    x, w = rnd((m, k), torch.bfloat16, gen), rnd((n, k), torch.bfloat16, gen)
+    bias = torch.randn(n, generator=gen, device="cuda")
+    saved = ops.force_generic   # (another test's fixture may have switched the fast kernels off)
+    ops.force_generic = False
+    try:
+        for out_dtype in (torch.bfloat16, torch.float32):
+            for b in (None, bias):
+                whole = torch.full((m + 1, n), 7.0, device="cuda", dtype=out_dtype)
+                o2 = torch.empty(m, n, device="cuda", dtype=out_dtype)
+                ops.linear(x, w, whole[:m], bias=b)
+                PlainOps().linear(x, w, o2, bias=b)
+                close(whole[:m], o2, out_dtype, scale=math.sqrt(k))
+                assert bool((whole[m] == 7.0).all())
+                part = torch.empty(33, n, device="cuda", dtype=out_dtype)
+                ops.linear(x[:33].contiguous(), w, part, bias=b)
+                assert torch.equal(part, whole[:33])
+    finally:
+        ops.force_generic = saved
 
 
 def test_linear_row_result_does_not_depend_on_batch(ops, gen):
