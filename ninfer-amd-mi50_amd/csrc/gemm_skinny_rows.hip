@@ -14,10 +14,14 @@
 //
 // Every block reads all of A (from L2): twice the bytes of its weights at 64 rows. Measured
 // against the library's kernels in a replayed decode step of 64 rows: 6144 features of K =
-// 2048 15.2 against 18.8 us; 2048 features (K = 2048 and 5632; 16 features a block, 128
-// blocks) 18.7 against 12.1 and 13.2; 151,936 features 244 us (the activations' 1.2 GB from
-// L2 bound it). So the kernel takes products of 4,096 to 32,768 features, where its blocks
-// fill the device and the activations' traffic stays small; the others stay with the
+// 2048 15.7 against 13.2 us; 2048 features (16 features a block, 128 blocks) 18.7 against
+// 12.0 (K = 2048) and 18.5 (K = 5632); 151,936 features 244 us (the activations' 1.2 GB from
+// L2 bound it). On the device the library's kernels are the faster ones, then; but a launch
+// here costs the host 3 us and the library's call 18, and the steps that bring 33 to 64
+// rows eagerly (short prompt portions, portions beside decoded tokens) are bound by the
+// host: 4.9 against 5.3 ms with the qkv product here, replayed decode steps of 40 to 64 rows
+// the same within 0.3%. So the kernel takes products of 4,096 to 32,768 features, where its
+// blocks fill the device and the activations' traffic stays small; the others stay with the
 // library. The reference sends all products of this size to the library
 // (src/ops/linear.hip:21-35).
 #include "gemm.h"
