@@ -14,7 +14,7 @@
 //
 // Every block reads all of A (from L2): twice the bytes of its weights at 64 rows. Measured
 // against the library's kernels in a replayed decode step of 64 rows: 6144 features of K =
-// 2048 15.7 against 13.2 us; 2048 features (16 features a block, 128 blocks) 18.7 against
+// 2048 15.2 against 13.2 us; 2048 features (16 features a block, 128 blocks) 18.7 against
 // 12.0 (K = 2048) and 18.5 (K = 5632); 151,936 features 244 us (the activations' 1.2 GB from
 // L2 bound it). On the device the library's kernels are the faster ones, then; but a launch
 // here costs the host 3 us and the library's call 18, and the steps that bring 33 to 64
@@ -77,27 +77,32 @@ __global__ __launch_bounds__(kRowsWaves * 64) void gemm_skinny_rows_kernel(GemmA
   const int st_read = r * 128;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   const int chunks = K / 128, per_wave = (chunks + kRowsWaves - 1) / kRowsWaves;
-  for (int c = wave * per_wave; c < min((wave + 1) * per_wave, chunks); ++c) {
-    const int k0 = c * 128;
-    bf16x8 wl[FG][2][2], x[RT][4];   // [feature group][half of the chunk][q]
+  const int c_end = min((wave + 1) * per_wave, chunks);
+  // the weights of a chunk are asked for a chunk ahead of its products (with K = 2048 a wave
+  // has two chunks: all its weights are under way before the first product); the activations,
+  // which come from L2, with the chunk itself (both a chunk ahead: the registers spill)
+  bf16x8 wl[2][FG][2][2], x[RT][4];   // [buffer][feature group][half of the chunk][q]
+  auto load_w = [&](int c, int b) {
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
       for (int s = 0; s < FG; ++s)
 #pragma unroll
         for (int q = 0; q < 2; ++q)
-          wl[s][h][q] = stream_load((const bf16x8*)(wline[s][q] + k0 + h * 64));
+          wl[b][s][h][q] = stream_load((const bf16x8*)(wline[s][q] + c * 128 + h * 64));
+  };
+  auto multiply = [&](int c, int b) {
 #pragma unroll
     for (int t = 0; t < RT; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        x[t][i] = m_valid[t] ? *(const bf16x8*)(xrow[t] + k0 + i * 32) : zero;
+        x[t][i] = m_valid[t] ? *(const bf16x8*)(xrow[t] + c * 128 + i * 32) : zero;
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
       for (int s = 0; s < FG; ++s) {
 #pragma unroll
-        for (int q = 0; q < 2; ++q) *(bf16x8*)(my_stage + st_write + 1024 * q) = wl[s][h][q];
+        for (int q = 0; q < 2; ++q) *(bf16x8*)(my_stage + st_write + 1024 * q) = wl[b][s][h][q];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
           const bf16x8 wf = *(const bf16x8*)(my_stage + st_read + 16 * ((4 * i + j) ^ (r & 7)));
@@ -106,7 +111,16 @@ __global__ __launch_bounds__(kRowsWaves * 64) void gemm_skinny_rows_kernel(GemmA
             acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, x[t][2 * h + i], acc[s][t], 0, 0, 0);
         }
       }
+  };
+  int c = wave * per_wave;
+  if (c < c_end) load_w(c, 0);
+  for (; c + 1 < c_end; c += 2) {
+    load_w(c + 1, 1);
+    multiply(c, 0);
+    if (c + 2 < c_end) load_w(c + 2, 0);
+    multiply(c + 1, 1);
   }
+  if (c < c_end) multiply(c, 0);
 
   __syncthreads();   // every wave is done with its weight lines
   // the accumulator holds out[feature 4 j + v][token r]; stored as [token][feature]
