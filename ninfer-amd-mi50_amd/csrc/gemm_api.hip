@@ -10,9 +10,15 @@ using namespace ninfer;
 // several 16-row tiles, each of which would stream the group's weights again (60 groups of
 // 2 x 1408 x 2048 and 2048 x 1408: a 224-token portion 6.4 against 7.6 ms, 160 tokens 5.8
 // against 6.4, the same at 8 and below; 64 groups of 2 x 2560 x 3584: 127 tokens 22.4 against 28.0,
-// 80 tokens 21.7 against 23.1)
+// 80 tokens 21.7 against 23.1). A plain product of 17 to 32 rows whose weights are very large
+// (256 Mi elements and more: a vocabulary's output head) counts as many too: the few-row
+// kernel's second row tile would read them again, and they are beyond any cache (151,936 x
+// 2048: 181 us there against 127 on the tile kernel; replayed decode steps of 17 to 32 rows
+// 1% faster)
 static bool many_rows(const GemmArgs& a) {
-  return a.offsets ? a.M > 8 * a.groups : (a.M > 32 && a.N > 128);
+  if (a.offsets) return a.M > 8 * a.groups;
+  const bool huge = a.M > 16 && a.epilogue == kEpilogueNone && (int64_t)a.N * a.K >= (256LL << 20);
+  return (a.M > 32 || huge) && a.N > 128;
 }
 
 // force_generic != 0 runs the plain tiled kernel whatever the shape (tests

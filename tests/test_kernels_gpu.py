@@ -224,6 +224,28 @@ def test_linear_of_33_to_64_rows(ops, gen, m, n, k):
         ops.force_generic = saved
 
 
+@pytest.mark.parametrize("m", [17, 32])
+def test_linear_with_very_large_weights_at_17_to_32_rows(ops, gen, m):
+    """A plain product of 17 to 32 rows against weights that no cache holds (an output head of
+    140,000 features) runs on the tile kernel instead of two row tiles of the few-row kernel:
+    against the plain product, 32-bit and bf16 results, nothing written beyond the rows."""
+    n, k = 140000, 2048
+    x = rnd((m, k), torch.bfloat16, gen)
+    w = rnd((n, k), torch.bfloat16, gen, 0.05)
+    saved = ops.force_generic
+    ops.force_generic = False
+    try:
+        for out_dtype in (torch.float32, torch.bfloat16):
+            whole = torch.full((m + 1, n), 7.0, device="cuda", dtype=out_dtype)
+            o2 = torch.empty(m, n, device="cuda", dtype=out_dtype)
+            ops.linear(x, w, whole[:m])
+            PlainOps().linear(x, w, o2)
+            close(whole[:m], o2, out_dtype, scale=0.05 * math.sqrt(k))
+            assert bool((whole[m] == 7.0).all())
+    finally:
+        ops.force_generic = saved
+
+
 def test_linear_row_result_does_not_depend_on_batch(ops, gen):
     """32-bit: a row's product is bit-identical alone and inside a batch."""
     x, w = rnd((70, 136), torch.float32, gen), rnd((200, 136), torch.float32, gen)
